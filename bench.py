@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE layer forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3_mixtral]
+
+A step is one forward of the whole layer (gate -> count/scan/pos -> FFN1+GELU ->
+FFN2 -> combine) over one synthetic batch already resident in HBM, issued as a
+single C-ABI call.  Prints ONE JSON line: layer tokens/s as ``value``; the
+grouped-GEMM TFLOP/s and its fraction of the fp16 dense MFMA peak; a
+``roofline`` object for the dominant kernel, timed with HIP events recorded on
+the layer's stream inside the timed region; and ``cpu_baseline``, the same
+layer through torch on this box's host cores.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0          # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+class HipEvents:
+    """hipEvent_t handles through the HIP runtime (torch's events hide the handle)."""
+
+    def __init__(self):
+        self.hip = ctypes.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p,
+                                                 ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+
+    def create(self):
+        ev = ctypes.c_void_p()
+        rc = self.hip.hipEventCreate(ctypes.byref(ev))
+        if rc != 0:
+            raise RuntimeError(f"hipEventCreate failed: {rc}")
+        return ev
+
+    def elapsed_ms(self, a, b):
+        ms = ctypes.c_float()
+        rc = self.hip.hipEventElapsedTime(ctypes.byref(ms), a, b)
+        if rc != 0:
+            raise RuntimeError(f"hipEventElapsedTime failed: {rc}")
+        return float(ms.value)
+
+    def destroy(self, ev):
+        self.hip.hipEventDestroy(ev)
+
+
+def cpu_baseline(wl, max_seconds=30.0):
+    """The layer through torch on the host cores, fp32 math on the fp16-rounded
+    values (the oracle's torch-only form).  1 warm-up + up to 3 timed runs,
+    stopping early once ``max_seconds`` is spent."""
+    import torch
+    from oracle import moe_oracle as O
+    t = wl.tensors
+    names = ("x", "wg", "bg", "w1", "b1", "w2", "b2")
+    args = [t[n].float() for n in names]
+    threads = torch.get_num_threads()
+    with torch.no_grad():
+        t0 = time.perf_counter()
+        O.reference_layer_torch(*args, wl.top_k, capacity=wl.capacity)
+        first = time.perf_counter() - t0
+        times = []
+        spent = first
+        while len(times) < 3 and (not times or spent + times[-1] < max_seconds):
+            t0 = time.perf_counter()
+            O.reference_layer_torch(*args, wl.top_k, capacity=wl.capacity)
+            times.append(time.perf_counter() - t0)
+            spent += times[-1]
+    med = sorted(times)[len(times) // 2]
+    return {"value": wl.tokens / med, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"full {wl.name} batch ({wl.tokens} tokens), fp32 torch on {threads} threads, "
+                      f"1 warm-up + median of {len(times)} runs",
+            "ms_per_step": med * 1e3}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3_mixtral")
+    ap.add_argument("--gemm-variant", type=int, default=None)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU's share only: this build has no collectives or sharding "
+              "code, so --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from ccfuser_amd import _lib, ops
+    from ccfuser_amd.workloads import make_workload
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the layer has no CPU path", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    lib = _lib.lib()
+    if a.gemm_variant is not None:
+        ops.set_option("gemm_variant", a.gemm_variant)
+
+    wl = make_workload(a.workload)
+    if wl.dtype != torch.float16:
+        for k, v in wl.tensors.items():
+            if v.is_floating_point():
+                wl.tensors[k] = v.half()
+    t = wl.tensors
+    T, d, f, E, k = wl.tokens, wl.d_model, wl.d_ffn, wl.num_expert, wl.top_k
+    ev = HipEvents()
+    K, W = a.steps, a.warmup
+    stream = torch.cuda.current_stream().cuda_stream
+
+    if a.workload == "c4_ep_share":
+        names = ("x", "seg_start", "seg_len", "seg_expert", "w1", "b1", "w2", "b2")
+        g = [t[n].cuda() for n in names]
+        y = torch.zeros(T, d, dtype=torch.float16, device="cuda")
+        run = lambda: ops.moe_ffn_segments(*g, y=y)
+        routed = T
+        stage_ms = None
+        for _ in range(W):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(K):
+            run()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    else:
+        names = ("x", "wg", "bg", "w1", "b1", "w2", "b2")
+        g = [t[n].cuda() for n in names]
+        ws = ops.moe_workspace(T, d, f, E, k, "cuda")
+        out = torch.empty(T, d, dtype=torch.float16, device="cuda")
+        offsets = torch.empty(E + 1, dtype=torch.int32, device="cuda")
+        ptrs = [x.data_ptr() for x in g]
+
+        def run():
+            _lib.call("ccf_moe_forward", *ptrs, T, d, f, E, k, wl.capacity, out.data_ptr(), None,
+                      None, None, None, offsets.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+
+        for _ in range(W):
+            run()
+        torch.cuda.synchronize()
+        routed = int(offsets[-1].item())
+        events = [[ev.create() for _ in range(6)] for _ in range(K)]
+        arrs = [(ctypes.c_void_p * 6)(*row) for row in events]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(K):
+            _lib.call("ccf_moe_forward_set_events", arrs[i], 6)
+            run()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        _lib.call("ccf_moe_forward_set_events", None, 0)
+        stage_names = ("gate", "route", "ffn1", "ffn2", "combine")
+        stage_ms = {n: sum(ev.elapsed_ms(events[i][s], events[i][s + 1]) for i in range(K)) / K
+                    for s, n in enumerate(stage_names)}
+        for row in events:
+            for e in row:
+                ev.destroy(e)
+
+    ms = wall / K * 1e3
+    flops = wl.flops(routed)
+    tflops = flops / (ms * 1e-3) / 1e12
+    line = {
+        "metric": "moe_layer_forward_tokens_per_s", "value": T / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"{wl.name}: {wl.description}", "tokens": T, "top_k": k,
+                   "num_expert": E, "d_model": d, "d_ffn": f, "routed_rows": routed,
+                   "capacity": wl.capacity, "seed": wl.seed},
+        "gemm_tflops": tflops, "frac_fp16_mfma_peak": tflops / PEAK_FP16_TFLOPS,
+    }
+    if stage_ms is not None:
+        line["stages_ms"] = stage_ms
+        dom = "ffn1" if stage_ms["ffn1"] >= stage_ms["ffn2"] else "ffn2"
+        ach = (flops / 2) / (stage_ms[dom] * 1e-3) / 1e12
+        line["roofline"] = {"kernel": f"grouped_gemm_kernel ({dom})", "bound": "mfma",
+                            "achieved": ach, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                            "frac": ach / PEAK_FP16_TFLOPS, "traffic": None,
+                            "flop_per_launch": flops / 2, "avg_launch_ms": stage_ms[dom]}
+        hbm_bytes = T * d * 2 + E * d * 2 + T * k * 10
+        line["gate_gbs"] = hbm_bytes / (stage_ms["gate"] * 1e-3) / 1e9
+    if not a.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

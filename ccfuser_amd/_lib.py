@@ -1,0 +1,75 @@
+"""ctypes binding of libccfuser_moe.so (the C ABI declared in include/ccfuser_moe.h).
+
+The library is loaded on first use.  There is no CPU fallback: if it has not
+been built, or a call fails, the caller gets an exception.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+from typing import Optional
+
+LIB_PATH = Path(__file__).resolve().parent / "libccfuser_moe.so"
+
+_lib: Optional[C.CDLL] = None
+
+_p = C.c_void_p
+_i = C.c_int
+_sz = C.c_size_t
+
+# name -> (restype, argtypes); mirrors include/ccfuser_moe.h declaration by declaration
+SIGNATURES = {
+    "ccf_version": (_i, []),
+    "ccf_last_error": (C.c_char_p, []),
+    "ccf_set_option": (_i, [C.c_char_p, _i]),
+    "ccf_gate_topk_softmax": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
+    "ccf_route_workspace_bytes": (_sz, [_i, _i]),
+    "ccf_expert_count": (_i, [_p, _i, _p, _i, _p]),
+    "ccf_assign_pos": (_i, [_p, _p, _i, _i, _p, _p, _sz, _p]),
+    "ccf_route": (_i, [_p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "ccf_segments_to_rows": (_i, [_p, _p, _p, _i, _i, _i, _p, _p, _p, _p]),
+    "ccf_local_scatter": (_i, [_p, _p, _p, _i, _i, _p]),
+    "ccf_local_gather": (_i, [_p, _p, _p, _i, _i, _p]),
+    "ccf_combine": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
+    "ccf_ffn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "ccf_ffn1_forward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p, _p, _sz, _p]),
+    "ccf_ffn2_forward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
+    "ccf_moe_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "ccf_moe_forward": (_i, [_p] * 7 + [_i] * 6 + [_p] * 6 + [_p, _sz, _p]),
+    "ccf_moe_forward_set_events": (_i, [C.POINTER(_p), _i]),
+    "ccf_segments_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "ccf_moe_ffn_segments": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),
+}
+
+
+class CcfError(RuntimeError):
+    """A C-ABI call returned a non-zero code."""
+
+    def __init__(self, fn: str, code: int, text: str):
+        super().__init__(f"{fn} failed with code {code}: {text}")
+        self.code = code
+
+
+def lib() -> C.CDLL:
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP library has not been built. "
+                "Run `python -m ccfuser_amd.build` (needs hipcc); there is no CPU fallback.")
+        handle = C.CDLL(str(LIB_PATH))
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)       # AttributeError if the symbol is not exported
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def call(name: str, *args) -> None:
+    """Call an int-returning entry point and raise CcfError on failure."""
+    handle = lib()
+    rc = getattr(handle, name)(*args)
+    if rc != 0:
+        raise CcfError(name, rc, handle.ccf_last_error().decode("utf-8", "replace"))

@@ -1,0 +1,47 @@
+// Shared helpers for the HIP sources of libccfuser_moe.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <string.h>
+
+#include "../../include/ccfuser_moe.h"
+
+namespace ccf {
+
+constexpr int kWave = 64;
+
+// Last error text, per host thread.
+char *error_buffer();
+int fail(int code, const char *fmt, ...);
+
+inline hipStream_t as_stream(ccf_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Launch check: a failed launch reports through hipGetLastError.
+inline int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(CCF_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return CCF_OK;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+typedef _Float16 half_t;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+}  // namespace ccf
+
+#define CCF_REQUIRE(cond, code, ...)                 \
+  do {                                               \
+    if (!(cond)) return ccf::fail(code, __VA_ARGS__); \
+  } while (0)

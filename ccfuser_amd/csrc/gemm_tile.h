@@ -1,0 +1,292 @@
+// Grouped fp16 GEMM main loop for gfx950 (MI355X): C[m, n] = sum_k A[m, k] * B[n, k].
+//
+// Both operands are K-contiguous ("NT"): A rows are token rows reached through
+// an optional row index (the scatter of the MoE layer fused into the tile
+// load), B rows are the rows of one expert's weight matrix exactly as the
+// reference stores it ([out, in], mix_moe/mix_moe/linear.py:198).  The
+// reference's tile kernel (mix_moe/csrc/cuda/mix_gemm.cu:22-244) is a 64x512
+// WMMA tile with fp16 accumulators fed by cp.async; this one is built for
+// CDNA4 instead:
+//
+//   * v_mfma_f32_32x32x16_f16, fp32 accumulators, 64-lane wavefronts;
+//   * tiles go HBM/L2 -> LDS with global_load_lds_dwordx4 (no VGPR staging);
+//     the LDS image is forced to be linear in lane order, so the XOR swizzle
+//     that keeps ds_read_b128 conflict-free is applied on the global side:
+//     the lane that owns LDS slot (row, c') fetches K-chunk c' ^ swz(row);
+//   * LDS is multi-buffered (STAGES), one workgroup barrier per K tile;
+//   * each stage is its own __shared__ object so the compiler can tell that a
+//     tile in flight does not alias the tile being read.
+#pragma once
+
+#include "ccf_common.h"
+
+#include <type_traits>
+
+namespace ccf {
+
+// ---- LDS layout ------------------------------------------------------------
+// A tile of ROWS x BK halves is ROWS x (BK/8) 16-byte chunks.  Row r, K-chunk c
+// lives at byte (r * CPR + (c ^ swz(r))) * 16.  swz depends on r & 15 only, so
+// rows 32 apart share it and the per-lane read addresses of the MFMA blocks of
+// a wavefront differ by compile-time constants.
+template <int CPR>
+__device__ __forceinline__ int swz(int r) {
+  static_assert(CPR == 8, "swizzle written for BK = 64");
+  return (r & 7) ^ ((r >> 3) & 1);
+}
+
+typedef __attribute__((address_space(3))) char lds_char;
+typedef __attribute__((address_space(3))) const half8 lds_half8;
+
+template <int S, int BYTES>
+__device__ __forceinline__ lds_char *stage_buf() {
+  __shared__ __attribute__((aligned(1024))) char buf[BYTES];
+  return (lds_char *)buf;
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Workgroup barrier without the memory fence __syncthreads() carries: that
+// fence makes the compiler drain every tile load in flight (vmcnt(0)), which
+// defeats multi-stage buffering.  The callers order their own LDS traffic: the
+// tile loads are waited for with wait_vmcnt, the LDS reads have returned
+// before the MFMAs that consume them issue.
+__device__ __forceinline__ void block_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// Wait until at most N LDS reads are in flight.  The two fragments the next
+// MFMA consumes are tied to the wait as in/out operands, so the MFMA cannot be
+// scheduled ahead of it.
+template <int N>
+__device__ __forceinline__ void wait_lgkmcnt(half8 &x, half8 &y) {
+  static_assert(N >= 0 && N < 15, "lgkmcnt");
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+}
+
+// 16 bytes per lane from LDS byte address addr + OFF.
+template <int OFF>
+__device__ __forceinline__ half8 lds_read_b128(uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "ds offset");
+  half8 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+
+__device__ __forceinline__ void lds_dma16(const void *gptr, lds_char *lds_wave_base) {
+  // 64 lanes x 16 bytes land at lds_wave_base + lane * 16.
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gptr,
+                                   (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
+}
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_>
+struct GemmCfg {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
+  static constexpr int NW = WM * WN;
+  static constexpr int THREADS = NW * 64;
+  static constexpr int WTM = BM / WM, WTN = BN / WN;   // wavefront tile
+  static constexpr int TM = WTM / 32, TN = WTN / 32;   // 32x32 MFMA blocks per wavefront
+  static constexpr int CPR = BK / 8;                   // 16-byte chunks per tile row
+  static constexpr int ROWS_PER_DMA = 64 / CPR;        // tile rows one wavefront load covers
+  static constexpr int A_DMA = BM / ROWS_PER_DMA / NW; // loads per wavefront per tile
+  static constexpr int B_DMA = BN / ROWS_PER_DMA / NW;
+  static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int KSTEPS = BK / 16;
+  static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wavefront tile");
+  static_assert(BM % (ROWS_PER_DMA * NW) == 0 && BN % (ROWS_PER_DMA * NW) == 0, "dma split");
+  static_assert(STAGES >= 2 && STAGES <= 4, "stages");
+};
+
+// One workgroup's main loop.  a_row_ptr(r) / b_row_ptr(r) give the global
+// address of K element 0 of tile row r (already clamped to a valid row).
+template <class Cfg>
+struct GemmMainloop {
+  using acc_t = float16v;
+
+  template <int S>
+  static __device__ __forceinline__ lds_char *stage() {
+    return stage_buf<S, Cfg::STAGE_BYTES>();
+  }
+
+  // Issue the loads of one K tile into stage S.
+  template <int S>
+  static __device__ __forceinline__ void issue(const half_t *const (&a_src)[Cfg::A_DMA],
+                                               const half_t *const (&b_src)[Cfg::B_DMA],
+                                               int k_elem, int wave) {
+    lds_char *base = stage<S>();
+#pragma unroll
+    for (int i = 0; i < Cfg::A_DMA; ++i)
+      lds_dma16(a_src[i] + k_elem, base + (i * Cfg::NW + wave) * 1024);
+#pragma unroll
+    for (int i = 0; i < Cfg::B_DMA; ++i)
+      lds_dma16(b_src[i] + k_elem, base + Cfg::A_BYTES + (i * Cfg::NW + wave) * 1024);
+  }
+
+  // Order in which the TM+TN operand fragments of one K step are read from
+  // LDS: a0, b0 .. b(TN-1), a1 .. a(TM-1), so that the first MFMA of the step
+  // can issue as early as possible.
+  static constexpr int FRAGS = Cfg::TM + Cfg::TN;
+  static constexpr int a_seq(int tm) { return tm == 0 ? 0 : Cfg::TN + tm; }
+  static constexpr int b_seq(int tn) { return 1 + tn; }
+
+  template <int S, int KS, int I>
+  static __device__ __forceinline__ void read_frag(half8 (&a)[Cfg::TM], half8 (&b)[Cfg::TN],
+                                                   const int (&a_off)[Cfg::KSTEPS],
+                                                   const int (&b_off)[Cfg::KSTEPS]) {
+    const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage<S>()));
+    if constexpr (I == 0) {
+      a[0] = lds_read_b128<0>(base + a_off[KS]);
+    } else if constexpr (I <= Cfg::TN) {
+      b[I - 1] = lds_read_b128<Cfg::A_BYTES + (I - 1) * 32 * Cfg::CPR * 16>(base + b_off[KS]);
+    } else {
+      a[I - Cfg::TN] = lds_read_b128<(I - Cfg::TN) * 32 * Cfg::CPR * 16>(base + a_off[KS]);
+    }
+  }
+
+  // MFMAs over the K tile held in stage S.  The fragments of K step ks+1 are
+  // read between the MFMAs of step ks into a second register set.  The LDS
+  // reads are inline asm (the compiler would otherwise make every LDS read
+  // wait for the tile loads in flight), so the lgkmcnt waits are placed here:
+  // LDS reads return in order, and before MFMA i of a step the reads still
+  // allowed in flight are the later fragments of this step plus the fragments
+  // of the next step issued so far.  Scheduling fences keep the source order.
+  template <int S>
+  static __device__ __forceinline__ void compute(acc_t (&acc)[Cfg::TM][Cfg::TN],
+                                                 const int (&a_off)[Cfg::KSTEPS],
+                                                 const int (&b_off)[Cfg::KSTEPS]) {
+    half8 a[2][Cfg::TM], b[2][Cfg::TN];
+    static_for<0, FRAGS>([&](auto I) { read_frag<S, 0, I.value>(a[0], b[0], a_off, b_off); });
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, Cfg::KSTEPS>([&](auto KS) {
+      constexpr int ks = KS.value;
+      constexpr int cur = ks & 1;
+      constexpr bool more = ks + 1 < Cfg::KSTEPS;
+      static_for<0, Cfg::TM * Cfg::TN>([&](auto II) {
+        constexpr int i = II.value;
+        constexpr int tm = i / Cfg::TN, tn = i % Cfg::TN;
+        constexpr int need = a_seq(tm) > b_seq(tn) ? a_seq(tm) : b_seq(tn);
+        constexpr int next_issued = more ? (i < FRAGS ? i : FRAGS) : 0;
+        wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
+        if constexpr (more && i < FRAGS) read_frag<S, ks + 1, i>(a[cur ^ 1], b[cur ^ 1], a_off, b_off);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+  }
+
+  template <int S>
+  struct Step {
+    static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
+                                               const half_t *const (&a_src)[Cfg::A_DMA],
+                                               const half_t *const (&b_src)[Cfg::B_DMA],
+                                               const int (&a_off)[Cfg::KSTEPS],
+                                               const int (&b_off)[Cfg::KSTEPS], int kt, int KT,
+                                               int wave) {
+      constexpr int NEXT = (S + Cfg::STAGES - 1) % Cfg::STAGES;   // stage of tile kt+STAGES-1
+      constexpr int PER_TILE = Cfg::A_DMA + Cfg::B_DMA;
+      if (kt >= KT) return;                                        // uniform
+      const int kpre = kt + Cfg::STAGES - 1;
+      if (kpre < KT) issue<NEXT>(a_src, b_src, kpre * Cfg::BK, wave);
+      compute<S>(acc, a_off, b_off);
+      // tile kt+1 must have landed before anyone reads it: leave at most the
+      // loads of the STAGES-2 younger tiles in flight.
+      if (kpre < KT) {
+        wait_vmcnt<PER_TILE *(Cfg::STAGES - 2)>();
+      } else {
+        wait_vmcnt<0>();
+      }
+      block_barrier();
+    }
+  };
+
+  static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
+                                             const half_t *const (&a_src)[Cfg::A_DMA],
+                                             const half_t *const (&b_src)[Cfg::B_DMA], int K) {
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+    const int KT = K / Cfg::BK;
+
+    // Per-lane LDS read offsets: row = lane % 32 of each 32x32 block, K-chunk
+    // 2*ks + lane/32.
+    int a_off[Cfg::KSTEPS], b_off[Cfg::KSTEPS];
+    {
+      const int ra = wm * Cfg::WTM + (lane & 31);
+      const int rb = wn * Cfg::WTN + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < Cfg::KSTEPS; ++ks) {
+        const int c = ks * 2 + (lane >> 5);
+        a_off[ks] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
+        b_off[ks] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
+      }
+    }
+
+    // Prologue: tiles 0 .. STAGES-2.
+    if (0 < KT) issue<0>(a_src, b_src, 0, wave);
+    if constexpr (Cfg::STAGES >= 3) {
+      if (1 < KT) issue<1>(a_src, b_src, Cfg::BK, wave);
+    }
+    if constexpr (Cfg::STAGES >= 4) {
+      if (2 < KT) issue<2>(a_src, b_src, 2 * Cfg::BK, wave);
+    }
+    // tile 0 landed; younger prologue tiles may stay in flight
+    if constexpr (Cfg::STAGES == 2) {
+      wait_vmcnt<0>();
+    } else {
+      if (KT >= Cfg::STAGES - 1) {
+        wait_vmcnt<(Cfg::A_DMA + Cfg::B_DMA) * (Cfg::STAGES - 2)>();
+      } else {
+        wait_vmcnt<0>();
+      }
+    }
+    block_barrier();
+
+    for (int kt0 = 0; kt0 < KT; kt0 += Cfg::STAGES) {
+      Step<0>::run(acc, a_src, b_src, a_off, b_off, kt0 + 0, KT, wave);
+      Step<1>::run(acc, a_src, b_src, a_off, b_off, kt0 + 1, KT, wave);
+      if constexpr (Cfg::STAGES >= 3) Step<2>::run(acc, a_src, b_src, a_off, b_off, kt0 + 2, KT, wave);
+      if constexpr (Cfg::STAGES >= 4) Step<3>::run(acc, a_src, b_src, a_off, b_off, kt0 + 3, KT, wave);
+    }
+  }
+
+  // Tile row this lane fetches with its i-th A (or B) load, and the K-chunk.
+  static __device__ __forceinline__ int dma_row(int i) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    return (i * Cfg::NW + wave) * Cfg::ROWS_PER_DMA + lane / Cfg::CPR;
+  }
+  static __device__ __forceinline__ int dma_chunk(int row) {
+    const int lane = threadIdx.x & 63;
+    return (lane % Cfg::CPR) ^ swz<Cfg::CPR>(row);
+  }
+};
+
+// Accumulator element r of block (tm, tn) is C[row, col] with
+//   row = wm*WTM + tm*32 + 8*(r/4) + 4*(lane/32) + r%4
+//   col = wn*WTN + tn*32 + lane%32
+template <class Cfg>
+__device__ __forceinline__ int acc_row(int tm, int r) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  return (wave / Cfg::WN) * Cfg::WTM + tm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+}
+template <class Cfg>
+__device__ __forceinline__ int acc_col(int tn) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  return (wave % Cfg::WN) * Cfg::WTN + tn * 32 + (lane & 31);
+}
+
+}  // namespace ccf

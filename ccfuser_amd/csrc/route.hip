@@ -1,0 +1,325 @@
+// Expert count, offset scan and deterministic pos for gfx950.
+//
+// Replaces the reference's expert_count_kernel / assign_pos_kernel pair
+// (mix_moe/csrc/cuda/local_exchange.cu:6-17, 37-70) and the host-side cumsum,
+// .item() and planning between them (mix_moe/mix_moe/functions.py:83-105).
+// The reference fills each expert's segment of pos through an atomicSub race;
+// here the flat indices inside a segment ascend, which is one of the orders
+// that race can produce, and everything stays on the device.
+//
+// Three small launches over chunks of kChunk flat indices:
+//   hist   per chunk, per expert counts (wavefront match + LDS integer adds)
+//   scan   one workgroup: per expert running sums over chunks, capacity clamp,
+//          exclusive scan over experts
+//   pos    per chunk: rank of every index inside its expert = chunk base +
+//          earlier wavefront passes in the chunk + lanes before it in the
+//          wavefront (ballot / popcount), then the scatter of pos and friends
+// Integer adds commute, so the results do not depend on scheduling.
+#include "ccf_common.h"
+
+namespace ccf {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kPasses = 4;                       // indices per thread
+constexpr int kChunk = kThreads * kPasses;       // flat indices per workgroup
+constexpr int kSub = kPasses * (kThreads / 64);  // wavefront passes per chunk
+constexpr int kMaxExpert = 1024;
+
+__device__ inline uint64_t lanes_below() {
+  const int lane = threadIdx.x & 63;
+  return lane ? (~0ull >> (64 - lane)) : 0ull;
+}
+
+// Lanes of this wavefront that hold the same valid expert id as the caller.
+__device__ inline uint64_t peers_of(int e, bool valid, int nbits) {
+  uint64_t peers = __ballot(valid);
+  for (int b = 0; b < nbits; ++b) {
+    uint64_t m = __ballot((e >> b) & 1);
+    peers &= ((e >> b) & 1) ? m : ~m;
+  }
+  return valid ? peers : 0ull;
+}
+
+__device__ inline int load_expert(const int64_t *idx, int i, int n, int E) {
+  if (i >= n) return -1;
+  int64_t e = idx[i];
+  return (e >= 0 && e < E) ? static_cast<int>(e) : -1;
+}
+
+__global__ void __launch_bounds__(kThreads)
+hist_kernel(const int64_t *__restrict__ idx, int n, int E, int nbits,
+            int32_t *__restrict__ chunk_cnt /* [nchunk][E] or NULL */,
+            int32_t *__restrict__ accumulate /* [E] or NULL */) {
+  extern __shared__ int s_hist[];
+  for (int e = threadIdx.x; e < E; e += kThreads) s_hist[e] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * kChunk;
+#pragma unroll
+  for (int p = 0; p < kPasses; ++p) {
+    const int i = base + p * kThreads + threadIdx.x;
+    const int e = load_expert(idx, i, n, E);
+    const uint64_t peers = peers_of(e, e >= 0, nbits);
+    if (e >= 0 && (peers & lanes_below()) == 0) atomicAdd(&s_hist[e], __popcll(peers));
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kThreads) {
+    if (chunk_cnt) chunk_cnt[static_cast<size_t>(blockIdx.x) * E + e] = s_hist[e];
+    if (accumulate && s_hist[e]) atomicAdd(&accumulate[e], s_hist[e]);
+  }
+}
+
+// One workgroup.  chunk_cnt becomes, in place, the exclusive running sum over
+// chunks (the rank base of each chunk).  If cum_inout is given the segment
+// starts come from it (cum[e] - total[e]) and are written back there;
+// otherwise they are the exclusive scan of the kept counts.
+__global__ void __launch_bounds__(1024)
+scan_kernel(int32_t *__restrict__ chunk_cnt, int nchunk, int E, int capacity,
+            int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
+            int32_t *__restrict__ cum_inout) {
+  __shared__ int s_kept[kMaxExpert];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    int run = 0;
+    for (int c = 0; c < nchunk; ++c) {
+      int v = chunk_cnt[static_cast<size_t>(c) * E + e];
+      chunk_cnt[static_cast<size_t>(c) * E + e] = run;
+      run += v;
+    }
+    int kept = (capacity >= 0 && run > capacity) ? capacity : run;
+    s_kept[e] = kept;
+    if (counts) counts[e] = kept;
+    if (cum_inout) {
+      int start = cum_inout[e] - run;
+      cum_inout[e] = start;
+      offsets[e] = start;
+    }
+  }
+  __syncthreads();
+  if (!cum_inout && threadIdx.x < 64) {
+    // exclusive scan over experts by one wavefront, 64 at a time
+    int carry = 0;
+    const int lane = threadIdx.x;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      int v = (e0 + lane < E) ? s_kept[e0 + lane] : 0;
+      int inc = v;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        int o = __shfl_up(inc, off, 64);
+        if (lane >= off) inc += o;
+      }
+      if (e0 + lane < E) offsets[e0 + lane] = carry + inc - v;
+      carry += __shfl(inc, 63, 64);
+    }
+    if (lane == 0) offsets[E] = carry;
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+pos_kernel(const int64_t *__restrict__ idx, int n, int E, int nbits, int top_k, int capacity,
+           const int32_t *__restrict__ chunk_base, const int32_t *__restrict__ offsets,
+           int64_t *__restrict__ pos, int32_t *__restrict__ src_row,
+           int32_t *__restrict__ dst_row, int32_t *__restrict__ inv_pos,
+           int64_t *__restrict__ idx_kept) {
+  extern __shared__ int s_sub[];                 // [kSub][E]
+  for (int i = threadIdx.x; i < kSub * E; i += kThreads) s_sub[i] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * kChunk;
+  const int wave = threadIdx.x >> 6;
+  int my_e[kPasses];
+  int my_rank[kPasses];
+#pragma unroll
+  for (int p = 0; p < kPasses; ++p) {
+    const int i = base + p * kThreads + threadIdx.x;
+    const int e = load_expert(idx, i, n, E);
+    const uint64_t peers = peers_of(e, e >= 0, nbits);
+    const uint64_t below = peers & lanes_below();
+    my_e[p] = e;
+    my_rank[p] = __popcll(below);
+    if (e >= 0 && below == 0) s_sub[(p * (kThreads / 64) + wave) * E + e] = __popcll(peers);
+  }
+  __syncthreads();
+  // exclusive running sum over the kSub wavefront passes, per expert
+  for (int e = threadIdx.x; e < E; e += kThreads) {
+    int run = chunk_base[static_cast<size_t>(blockIdx.x) * E + e];
+#pragma unroll
+    for (int s = 0; s < kSub; ++s) {
+      int v = s_sub[s * E + e];
+      s_sub[s * E + e] = run;
+      run += v;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int p = 0; p < kPasses; ++p) {
+    const int i = base + p * kThreads + threadIdx.x;
+    if (i >= n) continue;
+    const int e = my_e[p];
+    int j = -1;
+    if (e >= 0) {
+      const int rank = s_sub[(p * (kThreads / 64) + wave) * E + e] + my_rank[p];
+      if (capacity < 0 || rank < capacity) j = offsets[e] + rank;
+      if (j >= n) j = -1;                         // inconsistent caller-given starts
+    }
+    if (j >= 0) {
+      pos[j] = i;
+      if (src_row) src_row[j] = i / top_k;
+      if (dst_row) dst_row[j] = i;
+    }
+    if (inv_pos) inv_pos[i] = j;
+    if (idx_kept) idx_kept[i] = (j >= 0) ? static_cast<int64_t>(e) : -1;
+  }
+}
+
+// (start, len, expert) triples -> counts, offsets, row list grouped by expert.
+// Inside an expert the rows keep the order of the triple list, then row order.
+__global__ void __launch_bounds__(1024)
+segments_kernel(const int32_t *__restrict__ seg_start, const int32_t *__restrict__ seg_len,
+                const int32_t *__restrict__ seg_expert, int n_seg, int E, int total_rows,
+                int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
+                int32_t *__restrict__ rows) {
+  __shared__ int s_cnt[kMaxExpert];
+  __shared__ int s_off[kMaxExpert + 1];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    int run = 0;
+    for (int s = 0; s < n_seg; ++s)
+      if (seg_expert[s] == e && seg_len[s] > 0) run += seg_len[s];
+    s_cnt[e] = run;
+    counts[e] = run;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      s_off[e] = run;
+      offsets[e] = run;
+      run += s_cnt[e];
+    }
+    s_off[E] = run;
+    offsets[E] = run;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
+  for (int s = wave; s < n_seg; s += nwave) {
+    const int e = seg_expert[s];
+    const int len = seg_len[s], st = seg_start[s];
+    if (e < 0 || e >= E || len <= 0) continue;     // uniform per wavefront
+    int before = 0;                                // rows of earlier triples of this expert
+    for (int q = lane; q < s; q += 64)
+      if (seg_expert[q] == e && seg_len[q] > 0) before += seg_len[q];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) before += __shfl_xor(before, off, 64);
+    const int dst = s_off[e] + before;
+    for (int r = lane; r < len; r += 64) {
+      int row = st + r;                            // keep malformed triples inside the buffer
+      row = row < 0 ? 0 : (row >= total_rows ? total_rows - 1 : row);
+      if (dst + r < total_rows) rows[dst + r] = row;
+    }
+  }
+}
+
+int ceil_log2(int v) {
+  int b = 0;
+  while ((1 << b) < v) ++b;
+  return b;
+}
+
+struct RouteWs {
+  int32_t *chunk_cnt;   // [nchunk][E]
+  int nchunk;
+};
+
+size_t route_ws_bytes(int n_flat, int E) {
+  int nchunk = (n_flat + kChunk - 1) / kChunk;
+  if (nchunk < 1) nchunk = 1;
+  return round_up(sizeof(int32_t) * static_cast<size_t>(nchunk) * E, 256);
+}
+
+int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capacity,
+               int32_t *counts, int32_t *offsets, int32_t *cum_inout, int64_t *pos,
+               int32_t *src_row, int32_t *dst_row, int32_t *inv_pos, int64_t *idx_kept,
+               void *ws, size_t ws_bytes, hipStream_t stream) {
+  CCF_REQUIRE(gate_idx && pos, CCF_ERR_ARG, "route: null pointer");
+  CCF_REQUIRE(n_flat >= 0 && E > 0 && top_k >= 1, CCF_ERR_ARG, "route: bad size");
+  CCF_REQUIRE(E <= kMaxExpert, CCF_ERR_SHAPE, "route: num_expert=%d exceeds %d", E, kMaxExpert);
+  CCF_REQUIRE(ws && ws_bytes >= route_ws_bytes(n_flat, E), CCF_ERR_WORKSPACE,
+              "route: workspace of %zu bytes needed, %zu given", route_ws_bytes(n_flat, E), ws_bytes);
+  const int nchunk = n_flat > 0 ? (n_flat + kChunk - 1) / kChunk : 1;
+  const int nbits = ceil_log2(E);
+  int32_t *chunk_cnt = static_cast<int32_t *>(ws);
+  hipLaunchKernelGGL(hist_kernel, dim3(nchunk), dim3(kThreads), sizeof(int) * E, stream, gate_idx,
+                     n_flat, E, nbits, chunk_cnt, static_cast<int32_t *>(nullptr));
+  if (int rc = check_launch("hist_kernel")) return rc;
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, chunk_cnt, nchunk, E, capacity,
+                     counts, offsets, cum_inout);
+  if (int rc = check_launch("scan_kernel")) return rc;
+  hipLaunchKernelGGL(pos_kernel, dim3(nchunk), dim3(kThreads), sizeof(int) * kSub * E, stream,
+                     gate_idx, n_flat, E, nbits, top_k, capacity, chunk_cnt, offsets, pos, src_row,
+                     dst_row, inv_pos, idx_kept);
+  return check_launch("pos_kernel");
+}
+
+}  // namespace
+}  // namespace ccf
+
+extern "C" size_t ccf_route_workspace_bytes(int n_flat, int num_expert) {
+  if (n_flat < 0 || num_expert <= 0) return 0;
+  // chunk counts + room for the offsets ccf_assign_pos keeps internally
+  return ccf::route_ws_bytes(n_flat, num_expert) +
+         ccf::round_up(sizeof(int32_t) * (static_cast<size_t>(num_expert) + 1), 256);
+}
+
+extern "C" int ccf_expert_count(const int64_t *gate_idx, int n_flat, int32_t *expert_count,
+                                int num_expert, ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(gate_idx && expert_count, CCF_ERR_ARG, "expert_count: null pointer");
+  CCF_REQUIRE(n_flat >= 0 && num_expert > 0, CCF_ERR_ARG, "expert_count: bad size");
+  CCF_REQUIRE(num_expert <= kMaxExpert, CCF_ERR_SHAPE, "expert_count: num_expert=%d exceeds %d",
+              num_expert, kMaxExpert);
+  if (n_flat == 0) return CCF_OK;
+  const int nchunk = (n_flat + kChunk - 1) / kChunk;
+  hipLaunchKernelGGL(hist_kernel, dim3(nchunk), dim3(kThreads), sizeof(int) * num_expert,
+                     as_stream(stream), gate_idx, n_flat, num_expert, ceil_log2(num_expert),
+                     static_cast<int32_t *>(nullptr), expert_count);
+  return check_launch("hist_kernel");
+}
+
+extern "C" int ccf_assign_pos(int32_t *cum_count, const int64_t *gate_idx, int n_flat,
+                              int num_expert, int64_t *pos, void *workspace,
+                              size_t workspace_bytes, ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(cum_count, CCF_ERR_ARG, "assign_pos: null cum_count");
+  CCF_REQUIRE(workspace && workspace_bytes >= ccf_route_workspace_bytes(n_flat, num_expert),
+              CCF_ERR_WORKSPACE, "assign_pos: workspace of %zu bytes needed, %zu given",
+              ccf_route_workspace_bytes(n_flat, num_expert), workspace_bytes);
+  const size_t head = route_ws_bytes(n_flat, num_expert);
+  int32_t *offsets = reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + head);
+  return route_impl(gate_idx, n_flat, num_expert, 1, -1, nullptr, offsets, cum_count, pos, nullptr,
+                    nullptr, nullptr, nullptr, workspace, head, as_stream(stream));
+}
+
+extern "C" int ccf_route(const int64_t *gate_idx, int n_flat, int num_expert, int top_k,
+                         int capacity, int32_t *counts, int32_t *offsets, int64_t *pos,
+                         int32_t *src_row, int32_t *dst_row, int32_t *inv_pos, int64_t *idx_kept,
+                         void *workspace, size_t workspace_bytes, ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(counts && offsets, CCF_ERR_ARG, "route: null counts/offsets");
+  return route_impl(gate_idx, n_flat, num_expert, top_k, capacity, counts, offsets, nullptr, pos,
+                    src_row, dst_row, inv_pos, idx_kept, workspace, workspace_bytes,
+                    as_stream(stream));
+}
+
+extern "C" int ccf_segments_to_rows(const int32_t *seg_start, const int32_t *seg_len,
+                                    const int32_t *seg_expert, int n_seg, int num_expert,
+                                    int total_rows, int32_t *counts, int32_t *offsets,
+                                    int32_t *rows, ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(seg_start && seg_len && seg_expert && counts && offsets && rows, CCF_ERR_ARG,
+              "segments_to_rows: null pointer");
+  CCF_REQUIRE(n_seg >= 0 && num_expert > 0 && total_rows >= 0, CCF_ERR_ARG,
+              "segments_to_rows: bad size");
+  CCF_REQUIRE(num_expert <= kMaxExpert, CCF_ERR_SHAPE, "segments_to_rows: num_expert=%d exceeds %d",
+              num_expert, kMaxExpert);
+  hipLaunchKernelGGL(segments_kernel, dim3(1), dim3(1024), 0, as_stream(stream), seg_start, seg_len,
+                     seg_expert, n_seg, num_expert, total_rows, counts, offsets, rows);
+  return check_launch("segments_kernel");
+}

@@ -1,0 +1,106 @@
+"""Expert linear layers (reference mix_moe/mix_moe/linear.py).
+
+``MixMOELinear1`` / ``MixMOELinear2`` keep the reference's call shape
+``apply(inp, pos, block_infos, weight, bias)`` (linear.py:60-86, 115-143) but
+hand the stored ``[E, out, in]`` weight straight to the grouped GEMM: the
+per-call ``weight.transpose(-2, -1).contiguous()`` of the reference
+(linear.py:74, 129) is gone.  Only the forward halves exist; calling backward
+raises.
+"""
+import math
+import threading
+
+import torch
+import torch.nn as nn
+from torch.autograd import Function
+
+from .. import mix_moe_hip, ops
+
+
+class MixMOEInstance(object):
+    """Process-wide holder of the extension object (reference linear.py:15-29)."""
+    _instance_lock = threading.Lock()
+
+    def __init__(self, total_batch_size, num_expert, top_k, d_model, ffn_hidden_size, block_size):
+        self.mix_moe = mix_moe_hip.MixMOE(1, total_batch_size, num_expert, top_k, d_model,
+                                          ffn_hidden_size, block_size)
+
+    @classmethod
+    def instance(cls, *args, **kwargs):
+        if not hasattr(MixMOEInstance, "_instance"):
+            with MixMOEInstance._instance_lock:
+                if not hasattr(MixMOEInstance, "_instance"):
+                    MixMOEInstance._instance = MixMOEInstance(*args, **kwargs)
+        return MixMOEInstance._instance
+
+
+def _routing(pos, block_infos, top_k_hint=None):
+    """(src_row, dst_row, offsets, max_rows, n_flat) for the grouped GEMMs."""
+    if "offsets" in block_infos:                      # planned by this package: all on device
+        return (block_infos["src_row"], block_infos["dst_row"], block_infos["offsets"],
+                block_infos["max_rows"], block_infos["n_flat"])
+    raise KeyError("block_infos lacks 'offsets': plan it with AsyncExpertAssignment.process_data, or "
+                   "use ccfuser_amd.mix_moe_hip.MixMOE for the reference's block arrays")
+
+
+class MixMOELinear1(Function):
+    """h = x[pos // k] @ W1[e]^T + b1[e] per expert segment, optionally with the
+    erf GELU fused (``fuse_gelu``); h is in expert order, [max_rows, d_ffn]."""
+
+    @staticmethod
+    def forward(ctx, input_buf, pos, moe_inp_block_infos, weight, bias=None, fuse_gelu=False):
+        src_row, _, offsets, max_rows, _ = _routing(pos, moe_inp_block_infos)
+        E = offsets.numel() - 1
+        return ops.ffn1(input_buf, src_row, offsets, max_rows, weight.detach()[:E],
+                        bias.detach()[:E], gelu=bool(fuse_gelu))
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        raise NotImplementedError("forward-only build: MixMOELinear1.backward is not implemented")
+
+
+class MixMOELinear2(Function):
+    """y_flat[pos[j]] = h[j] @ W2[e]^T + b2[e]; y_flat is [tokens*top_k, d_model]
+    in flat token order (the reference's index_copy_ after the second GEMM,
+    mix_moe/csrc/mix_moe.h:433, happens in the GEMM epilogue)."""
+
+    @staticmethod
+    def forward(ctx, input_buf, pos, moe_inp_block_infos, weight, bias=None):
+        _, dst_row, offsets, max_rows, n_flat = _routing(pos, moe_inp_block_infos)
+        E = offsets.numel() - 1
+        d = weight.shape[1]
+        alloc = torch.zeros if moe_inp_block_infos.get("may_drop", True) else torch.empty
+        y = alloc(n_flat, d, dtype=input_buf.dtype, device=input_buf.device)
+        return ops.ffn2(input_buf, dst_row, offsets, max_rows, weight.detach()[:E],
+                        bias.detach()[:E], y)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        raise NotImplementedError("forward-only build: MixMOELinear2.backward is not implemented")
+
+
+class FMoELinear(nn.Module):
+    """Parameter container for E experts: weight [E, out, in], bias [E, out]
+    (reference linear.py:177-233)."""
+
+    def __init__(self, num_expert: int, in_feat: int, out_feat: int, bias: bool = True, rank: int = 0):
+        super().__init__()
+        self.num_expert = num_expert
+        self.in_feat = in_feat
+        self.out_feat = out_feat
+        self.rank = rank
+        self.weight = nn.Parameter(torch.empty(num_expert, out_feat, in_feat))
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(num_expert, out_feat))
+        else:
+            self.register_parameter("bias", None)
+        self.reset_parameters()
+
+    def extra_repr(self) -> str:
+        return "num_expert={}, in_features={}, out_features={}, bias={}, rank={}".format(
+            self.num_expert, self.in_feat, self.out_feat, self.bias is not None, self.rank)
+
+    def reset_parameters(self):
+        torch.nn.init.kaiming_uniform_(self.weight, a=math.sqrt(0.9))
+        if self.bias is not None:
+            torch.nn.init.kaiming_uniform_(self.bias, a=math.sqrt(0.9))

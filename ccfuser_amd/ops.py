@@ -1,0 +1,322 @@
+"""Torch-tensor front end of the C ABI: argument checks, workspaces, streams.
+
+Every function takes CUDA (ROCm) tensors, launches on torch's current stream
+for the tensors' device and returns without a host synchronisation unless its
+docstring says otherwise.  Wrong dtypes, shapes or devices raise Python
+exceptions (the reference prints and returns an empty tensor,
+mix_moe/csrc/mix_moe.h:242-245, or asserts, mix_moe/csrc/cuda/utils.h:4-6).
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+CCF_F16, CCF_F32 = 0, 1
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _check(t: torch.Tensor, name: str, dtype=None, ndim=None) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a tensor")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if ndim is not None and t.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dimensions, got {tuple(t.shape)}")
+
+
+def _workspace(nbytes: int, like: torch.Tensor) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=like.device)
+
+
+def set_option(name: str, value: int) -> None:
+    _lib.call("ccf_set_option", name.encode(), int(value))
+
+
+# ------------------------------------------------------------------ gate
+def gate_topk_softmax(x: torch.Tensor, wg: torch.Tensor, bg: Optional[torch.Tensor], top_k: int,
+                      return_logits: bool = False):
+    """(idx int64 [T,k], score [T,k]) and optionally logits [T,E], all on x's device."""
+    _check(x, "x", ndim=2)
+    if x.dtype not in (torch.float16, torch.float32):
+        raise TypeError(f"gate input must be float16 or float32, got {x.dtype}")
+    _check(wg, "gate weight", dtype=x.dtype, ndim=2)
+    if bg is not None:
+        _check(bg, "gate bias", dtype=x.dtype, ndim=1)
+    T, d = x.shape
+    E = wg.shape[0]
+    if wg.shape[1] != d or (bg is not None and bg.shape[0] != E):
+        raise ValueError("gate weight/bias shapes do not match the input")
+    idx = torch.empty(T, top_k, dtype=torch.int64, device=x.device)
+    score = torch.empty(T, top_k, dtype=x.dtype, device=x.device)
+    logits = torch.empty(T, E, dtype=x.dtype, device=x.device) if return_logits else None
+    with torch.cuda.device(x.device):
+        _lib.call("ccf_gate_topk_softmax", _ptr(x), _ptr(wg), _ptr(bg), T, d, E, int(top_k),
+                  CCF_F16 if x.dtype == torch.float16 else CCF_F32, _ptr(idx), _ptr(score),
+                  _ptr(logits), _stream(x))
+    return (idx, score, logits) if return_logits else (idx, score)
+
+
+# --------------------------------------------------------------- routing
+def expert_count(gate_idx: torch.Tensor, expert_count_out: torch.Tensor) -> None:
+    """Accumulate the histogram of ``gate_idx`` into ``expert_count_out`` (int32)."""
+    _check(gate_idx, "gate_idx", dtype=torch.int64)
+    _check(expert_count_out, "expert_count", dtype=torch.int32, ndim=1)
+    with torch.cuda.device(gate_idx.device):
+        _lib.call("ccf_expert_count", _ptr(gate_idx), gate_idx.numel(), _ptr(expert_count_out),
+                  expert_count_out.numel(), _stream(gate_idx))
+
+
+def assign_pos(cum_count: torch.Tensor, gate: torch.Tensor, pos: torch.Tensor) -> None:
+    """Fill ``pos`` from the inclusive cumulative count; ``cum_count`` is consumed."""
+    _check(cum_count, "cum_count", dtype=torch.int32, ndim=1)
+    _check(gate, "gate", dtype=torch.int64)
+    _check(pos, "pos", dtype=torch.int64, ndim=1)
+    n, E = gate.numel(), cum_count.numel()
+    if pos.numel() > n:
+        raise ValueError("pos is longer than the gate index list")
+    with torch.cuda.device(gate.device):
+        nbytes = _lib.lib().ccf_route_workspace_bytes(n, E)
+        ws = _workspace(nbytes, gate)
+        # pos may be shorter than n (dropped entries); the kernel bounds writes by n, so hand it
+        # a full-length buffer when the caller's is shorter
+        full = pos if pos.numel() == n else torch.empty(n, dtype=torch.int64, device=gate.device)
+        _lib.call("ccf_assign_pos", _ptr(cum_count), _ptr(gate), n, E, _ptr(full), _ptr(ws),
+                  ws.numel(), _stream(gate))
+        if full is not pos:
+            pos.copy_(full[: pos.numel()])
+
+
+def route(gate_idx: torch.Tensor, num_expert: int, top_k: int, capacity: int = -1) -> Dict[str, torch.Tensor]:
+    """Counts, offsets, deterministic pos and the row maps, all on the device.
+
+    ``pos``/``src_row``/``dst_row`` have ``n_flat`` entries of which the first
+    ``offsets[num_expert]`` are valid; nothing is synchronised to find that count.
+    """
+    _check(gate_idx, "gate_idx", dtype=torch.int64)
+    n = gate_idx.numel()
+    dev = gate_idx.device
+    out = {
+        "counts": torch.empty(num_expert, dtype=torch.int32, device=dev),
+        "offsets": torch.empty(num_expert + 1, dtype=torch.int32, device=dev),
+        "pos": torch.empty(n, dtype=torch.int64, device=dev),
+        "src_row": torch.empty(n, dtype=torch.int32, device=dev),
+        "dst_row": torch.empty(n, dtype=torch.int32, device=dev),
+        "inv_pos": torch.empty(n, dtype=torch.int32, device=dev),
+        "idx_kept": torch.empty(n, dtype=torch.int64, device=dev),
+    }
+    with torch.cuda.device(dev):
+        ws = _workspace(_lib.lib().ccf_route_workspace_bytes(n, num_expert), gate_idx)
+        _lib.call("ccf_route", _ptr(gate_idx), n, int(num_expert), int(top_k), int(capacity),
+                  _ptr(out["counts"]), _ptr(out["offsets"]), _ptr(out["pos"]), _ptr(out["src_row"]),
+                  _ptr(out["dst_row"]), _ptr(out["inv_pos"]), _ptr(out["idx_kept"]), _ptr(ws),
+                  ws.numel(), _stream(gate_idx))
+    return out
+
+
+def segments_to_rows(seg_start, seg_len, seg_expert, num_expert: int, total_rows: int):
+    for t, nm in ((seg_start, "seg_start"), (seg_len, "seg_len"), (seg_expert, "seg_expert")):
+        _check(t, nm, dtype=torch.int32, ndim=1)
+    dev = seg_start.device
+    counts = torch.empty(num_expert, dtype=torch.int32, device=dev)
+    offsets = torch.empty(num_expert + 1, dtype=torch.int32, device=dev)
+    rows = torch.zeros(total_rows, dtype=torch.int32, device=dev)   # entries past offsets[-1] stay 0
+    with torch.cuda.device(dev):
+        _lib.call("ccf_segments_to_rows", _ptr(seg_start), _ptr(seg_len), _ptr(seg_expert),
+                  seg_start.numel(), int(num_expert), int(total_rows), _ptr(counts), _ptr(offsets),
+                  _ptr(rows), _stream(seg_start))
+    return counts, offsets, rows
+
+
+# ------------------------------------------------- row moves and combine
+def local_scatter(inp: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
+    """``out[j] = inp[pos[j]]``; pos int32."""
+    _check(inp, "inp", dtype=torch.float16, ndim=2)
+    _check(pos, "pos", dtype=torch.int32, ndim=1)
+    out = torch.empty(pos.numel(), inp.shape[1], dtype=inp.dtype, device=inp.device)
+    with torch.cuda.device(inp.device):
+        _lib.call("ccf_local_scatter", _ptr(inp), _ptr(out), _ptr(pos), pos.numel(), inp.shape[1],
+                  _stream(inp))
+    return out
+
+
+def local_gather(inp: torch.Tensor, pos: torch.Tensor, out_rows: int) -> torch.Tensor:
+    """``out[pos[j]] = inp[j]``; rows nothing maps to are zero."""
+    _check(inp, "inp", dtype=torch.float16, ndim=2)
+    _check(pos, "pos", dtype=torch.int32, ndim=1)
+    if pos.numel() != inp.shape[0]:
+        raise ValueError("pos and inp disagree on the number of rows")
+    out = torch.zeros(out_rows, inp.shape[1], dtype=inp.dtype, device=inp.device)
+    with torch.cuda.device(inp.device):
+        _lib.call("ccf_local_gather", _ptr(inp), _ptr(out), _ptr(pos), pos.numel(), inp.shape[1],
+                  _stream(inp))
+    return out
+
+
+def combine(y_flat: torch.Tensor, score: torch.Tensor, top_k: int,
+            inv_pos: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _check(y_flat, "y_flat", dtype=torch.float16, ndim=2)
+    _check(score, "score", dtype=torch.float16)
+    if inv_pos is not None:
+        _check(inv_pos, "inv_pos", dtype=torch.int32, ndim=1)
+    n, d = y_flat.shape
+    if n % top_k or score.numel() != n or (inv_pos is not None and inv_pos.numel() != n):
+        raise ValueError("combine: sizes do not match tokens*top_k")
+    out = torch.empty(n // top_k, d, dtype=y_flat.dtype, device=y_flat.device)
+    with torch.cuda.device(y_flat.device):
+        _lib.call("ccf_combine", _ptr(y_flat), _ptr(score), _ptr(inv_pos), _ptr(out), n // top_k,
+                  int(top_k), d, _stream(y_flat))
+    return out
+
+
+# ------------------------------------------------------------ expert FFN
+def _check_expert(w: torch.Tensor, b: torch.Tensor, name: str) -> None:
+    _check(w, f"{name} weight", dtype=torch.float16, ndim=3)
+    _check(b, f"{name} bias", dtype=torch.float16, ndim=2)
+    if b.shape[0] != w.shape[0] or b.shape[1] != w.shape[1]:
+        raise ValueError(f"{name}: bias {tuple(b.shape)} does not match weight {tuple(w.shape)}")
+
+
+def ffn1(x: torch.Tensor, src_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
+         w1: torch.Tensor, b1: torch.Tensor, gelu: bool = True,
+         out: Optional[torch.Tensor] = None, dst_row: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h [max_rows, f] (or ``out``); rows nothing maps to are left as they were."""
+    if x.dtype != torch.float16:
+        raise TypeError("moe input data type must be float 16")
+    _check(x, "x", dtype=torch.float16, ndim=2)
+    _check_expert(w1, b1, "ffn1")
+    _check(offsets, "offsets", dtype=torch.int32, ndim=1)
+    E, f, d = w1.shape
+    if x.shape[1] != d or offsets.numel() != E + 1:
+        raise ValueError("ffn1: x/offsets do not match the weight shape")
+    if src_row is not None:
+        _check(src_row, "src_row", dtype=torch.int32, ndim=1)
+        if src_row.numel() < max_rows:
+            raise ValueError("ffn1: src_row shorter than max_rows")
+    elif x.shape[0] < max_rows:
+        raise ValueError("ffn1: x has fewer rows than max_rows")
+    if dst_row is not None:
+        _check(dst_row, "dst_row", dtype=torch.int32, ndim=1)
+        if out is None or dst_row.numel() < max_rows:
+            raise ValueError("ffn1: dst_row needs an explicit `out` and max_rows entries")
+    h = out if out is not None else torch.empty(max_rows, f, dtype=x.dtype, device=x.device)
+    _check(h, "h", dtype=torch.float16, ndim=2)
+    if h.shape[1] != f or (dst_row is None and h.shape[0] < max_rows):
+        raise ValueError("ffn1: output buffer too small")
+    with torch.cuda.device(x.device):
+        ws = _workspace(_lib.lib().ccf_ffn_workspace_bytes(max_rows, E, d, f), x)
+        _lib.call("ccf_ffn1_forward", _ptr(x), _ptr(src_row), _ptr(dst_row), _ptr(offsets), int(max_rows), E, d, f,
+                  _ptr(w1), _ptr(b1), int(bool(gelu)), _ptr(h), _ptr(ws), ws.numel(), _stream(x))
+    return h
+
+
+def ffn2(h: torch.Tensor, dst_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
+         w2: torch.Tensor, b2: torch.Tensor, y: torch.Tensor,
+         row_scale: Optional[torch.Tensor] = None,
+         src_row: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Writes ``y[dst_row[j]]`` for the routed rows and returns ``y``."""
+    _check(h, "h", dtype=torch.float16, ndim=2)
+    _check_expert(w2, b2, "ffn2")
+    _check(offsets, "offsets", dtype=torch.int32, ndim=1)
+    _check(y, "y", dtype=torch.float16, ndim=2)
+    E, d, f = w2.shape
+    if h.shape[1] != f or offsets.numel() != E + 1 or y.shape[1] != d:
+        raise ValueError("ffn2: h/offsets/y do not match the weight shape")
+    if src_row is not None:
+        _check(src_row, "src_row", dtype=torch.int32, ndim=1)
+        if src_row.numel() < max_rows:
+            raise ValueError("ffn2: src_row shorter than max_rows")
+    elif h.shape[0] < max_rows:
+        raise ValueError("ffn2: h has fewer rows than max_rows")
+    if dst_row is not None:
+        _check(dst_row, "dst_row", dtype=torch.int32, ndim=1)
+        if dst_row.numel() < max_rows:
+            raise ValueError("ffn2: dst_row shorter than max_rows")
+    elif y.shape[0] < max_rows:
+        raise ValueError("ffn2: y has fewer rows than max_rows")
+    if row_scale is not None:
+        _check(row_scale, "row_scale", dtype=torch.float16, ndim=1)
+    with torch.cuda.device(h.device):
+        ws = _workspace(_lib.lib().ccf_ffn_workspace_bytes(max_rows, E, d, f), h)
+        _lib.call("ccf_ffn2_forward", _ptr(h), _ptr(src_row), _ptr(dst_row), _ptr(offsets), int(max_rows), E, d, f,
+                  _ptr(w2), _ptr(b2), _ptr(row_scale), _ptr(y), _ptr(ws), ws.numel(), _stream(h))
+    return y
+
+
+# ------------------------------------------------------- the whole layer
+def moe_forward(x, wg, bg, w1, b1, w2, b2, top_k: int, capacity: int = -1,
+                return_routing: bool = False, workspace: Optional[torch.Tensor] = None):
+    """The fused layer forward: out [T, d] fp16 (and the routing tensors on request)."""
+    if x.dtype != torch.float16:
+        raise TypeError("moe input data type must be float 16")
+    _check(x, "x", dtype=torch.float16, ndim=2)
+    _check(wg, "gate weight", dtype=torch.float16, ndim=2)
+    if bg is not None:
+        _check(bg, "gate bias", dtype=torch.float16, ndim=1)
+    _check_expert(w1, b1, "ffn1")
+    _check_expert(w2, b2, "ffn2")
+    T, d = x.shape
+    E, f, d1 = w1.shape
+    if d1 != d or tuple(w2.shape) != (E, d, f) or tuple(wg.shape) != (E, d):
+        raise ValueError("moe_forward: weight shapes do not match (one GPU: the gate scores the local experts)")
+    dev = x.device
+    out = torch.empty(T, d, dtype=x.dtype, device=dev)
+    n = T * top_k
+    extra = {}
+    if return_routing:
+        extra = {"idx": torch.empty(T, top_k, dtype=torch.int64, device=dev),
+                 "score": torch.empty(T, top_k, dtype=x.dtype, device=dev),
+                 "pos": torch.empty(n, dtype=torch.int64, device=dev),
+                 "counts": torch.empty(E, dtype=torch.int32, device=dev),
+                 "offsets": torch.empty(E + 1, dtype=torch.int32, device=dev)}
+    with torch.cuda.device(dev):
+        need = _lib.lib().ccf_moe_workspace_bytes(T, d, f, E, int(top_k))
+        ws = workspace if workspace is not None else _workspace(need, x)
+        _lib.call("ccf_moe_forward", _ptr(x), _ptr(wg), _ptr(bg), _ptr(w1), _ptr(b1), _ptr(w2),
+                  _ptr(b2), T, d, f, E, int(top_k), int(capacity), _ptr(out), _ptr(extra.get("idx")),
+                  _ptr(extra.get("score")), _ptr(extra.get("pos")), _ptr(extra.get("counts")),
+                  _ptr(extra.get("offsets")), _ptr(ws), ws.numel(), _stream(x))
+    return (out, extra) if return_routing else out
+
+
+def moe_workspace(tokens: int, d_model: int, d_ffn: int, num_expert: int, top_k: int,
+                  device) -> torch.Tensor:
+    """A reusable workspace for ``moe_forward`` (one layer call at a time per workspace)."""
+    need = _lib.lib().ccf_moe_workspace_bytes(tokens, d_model, d_ffn, num_expert, top_k)
+    return torch.empty(max(need, 256), dtype=torch.uint8, device=device)
+
+
+def moe_ffn_segments(x, seg_start, seg_len, seg_expert, w1, b1, w2, b2,
+                     y: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Expert FFN over an inbound buffer addressed by (start, len, expert) triples."""
+    if x.dtype != torch.float16:
+        raise TypeError("moe input data type must be float 16")
+    _check(x, "x", dtype=torch.float16, ndim=2)
+    for t, nm in ((seg_start, "seg_start"), (seg_len, "seg_len"), (seg_expert, "seg_expert")):
+        _check(t, nm, dtype=torch.int32, ndim=1)
+    _check_expert(w1, b1, "ffn1")
+    _check_expert(w2, b2, "ffn2")
+    R, d = x.shape
+    E, f, _ = w1.shape
+    if y is None:
+        y = torch.zeros(R, d, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        need = _lib.lib().ccf_segments_workspace_bytes(R, seg_start.numel(), E, d, f)
+        ws = _workspace(need, x)
+        _lib.call("ccf_moe_ffn_segments", _ptr(x), _ptr(seg_start), _ptr(seg_len), _ptr(seg_expert),
+                  seg_start.numel(), R, d, f, E, _ptr(w1), _ptr(b1), _ptr(w2), _ptr(b2), _ptr(y),
+                  _ptr(ws), ws.numel(), _stream(x))
+    return y

@@ -1,0 +1,263 @@
+/*
+ * ccfuser_moe.h -- C ABI of the MI355X (gfx950) MoE layer forward.
+ *
+ * One shared library, libccfuser_moe.so, exports the functions below.  They
+ * take raw device pointers, sizes and a HIP stream, enqueue kernels on that
+ * stream and return without synchronising the host.  No torch types cross
+ * this boundary.  Every function returns 0 on success or a CCF_ERR_* code; the
+ * text of the last error on the calling thread is available from
+ * ccf_last_error().  Nothing here calls exit().
+ *
+ * Each declaration names the reference interface it replaces; paths are
+ * relative to the reference repository root.
+ *
+ * Conventions
+ *   - fp16 tensors are IEEE binary16, row-major, rows 16-byte aligned
+ *     (d_model and d_ffn multiples of 8; the grouped GEMMs need multiples of 64).
+ *   - expert weights keep the layout of the reference's parameter containers
+ *     (mix_moe/mix_moe/linear.py:198-202): w1 [E, d_ffn, d_model],
+ *     b1 [E, d_ffn], w2 [E, d_model, d_ffn], b2 [E, d_model].  The reference
+ *     transposes them to [E, K, N] on every call (linear.py:74, 129); this
+ *     library consumes the stored layout directly.
+ *   - "flat index" i = token * top_k + slot, as in the reference's pos vector.
+ *   - workspaces are caller-owned device memory, 256-byte aligned; the
+ *     *_workspace_bytes functions give the size to allocate.
+ */
+#ifndef CCFUSER_MOE_H
+#define CCFUSER_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *ccf_stream_t; /* a hipStream_t; NULL is the null stream */
+
+enum {
+  CCF_OK = 0,
+  CCF_ERR_ARG = 1,         /* null pointer, negative size, bad enum            */
+  CCF_ERR_SHAPE = 2,       /* a size the kernels do not support                */
+  CCF_ERR_WORKSPACE = 3,   /* workspace missing or too small                   */
+  CCF_ERR_HIP = 4,         /* a HIP runtime call or a launch failed            */
+  CCF_ERR_UNSUPPORTED = 5  /* dtype or option not implemented                  */
+};
+
+enum { CCF_F16 = 0, CCF_F32 = 1 };
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ccf_version(void);
+
+/* Text of the last error raised on this thread ("" if none). */
+const char *ccf_last_error(void);
+
+/*
+ * Tuning knobs (no counterpart in the reference).  "gemm_variant" selects the
+ * grouped-GEMM tile configuration used by the FFN entry points; 0 is the
+ * default.  Process-wide; not meant to be changed while work is in flight.
+ */
+int ccf_set_option(const char *name, int value);
+
+/* ------------------------------------------------------------------ gate */
+
+/*
+ * Top-k gate: logits = x * wg^T + bg (fp32 accumulation in a fixed order,
+ * rounded once to the input dtype), top-k per token (slot 0 = largest, ties to
+ * the lower expert id), softmax over the k selected logits.
+ * Replaces NaiveGate.forward, mix_moe/mix_moe/gates/naive_gate.py:26-45.
+ *   x [tokens, d_model], wg [tot_expert, d_model], bg [tot_expert] or NULL,
+ *   idx_out int64 [tokens, top_k], score_out [tokens, top_k] in the input
+ *   dtype, logits_out [tokens, tot_expert] in the input dtype or NULL.
+ *   dtype is CCF_F16 or CCF_F32.  d_model % 8 == 0, 1 <= top_k <= 8,
+ *   top_k <= tot_expert <= 1024.
+ */
+int ccf_gate_topk_softmax(const void *x, const void *wg, const void *bg,
+                          int tokens, int d_model, int tot_expert, int top_k,
+                          int dtype, int64_t *idx_out, void *score_out,
+                          void *logits_out, ccf_stream_t stream);
+
+/* --------------------------------------------------------------- routing */
+
+/* Bytes of workspace ccf_route / ccf_assign_pos need for n_flat indices. */
+size_t ccf_route_workspace_bytes(int n_flat, int num_expert);
+
+/*
+ * Histogram of gate indices, accumulated into expert_count (the caller zero
+ * fills, as mix_moe/mix_moe/functions.py:85-88 does).  Entries < 0 or
+ * >= num_expert are skipped.
+ * Replaces _expert_count / expert_count_kernel,
+ * mix_moe/csrc/cuda/local_exchange.cu:37-79, 98-108.
+ */
+int ccf_expert_count(const int64_t *gate_idx, int n_flat, int32_t *expert_count,
+                     int num_expert, ccf_stream_t stream);
+
+/*
+ * pos from an inclusive cumulative count: the flat indices routed to expert e
+ * fill pos[cum[e]-count[e] .. cum[e]) in ascending order; on return
+ * cum_count[e] holds the start of that segment (the reference decrements it
+ * once per routed index, so it ends at the same value).
+ * Replaces _assign_pos / assign_pos_kernel,
+ * mix_moe/csrc/cuda/local_exchange.cu:6-27, 81-96, whose order inside a
+ * segment is left to an atomic race.
+ */
+int ccf_assign_pos(int32_t *cum_count, const int64_t *gate_idx, int n_flat,
+                   int num_expert, int64_t *pos, void *workspace,
+                   size_t workspace_bytes, ccf_stream_t stream);
+
+/*
+ * Count + exclusive scan + deterministic pos in one call, with optional
+ * capacity limiting, all on the device and without a host synchronisation.
+ * Replaces perpare_expert_assignment at world_size 1,
+ * mix_moe/mix_moe/functions.py:83-105.
+ *   gate_idx int64 [n_flat] (-1 = already dropped)
+ *   capacity  rows an expert keeps (first come in flat order), < 0 = no limit
+ *   counts  int32 [num_expert]      kept rows per expert
+ *   offsets int32 [num_expert + 1]  exclusive scan; offsets[num_expert] = R
+ *   pos     int64 [n_flat]          first R entries valid
+ *   src_row int32 [n_flat] or NULL  pos[j] / top_k  (row of x to read)
+ *   dst_row int32 [n_flat] or NULL  pos[j]          (row of y_flat to write)
+ *   inv_pos int32 [n_flat] or NULL  j for kept flat index i, else -1
+ *   idx_kept int64 [n_flat] or NULL gate_idx with dropped entries set to -1
+ */
+int ccf_route(const int64_t *gate_idx, int n_flat, int num_expert, int top_k,
+              int capacity, int32_t *counts, int32_t *offsets, int64_t *pos,
+              int32_t *src_row, int32_t *dst_row, int32_t *inv_pos,
+              int64_t *idx_kept, void *workspace, size_t workspace_bytes,
+              ccf_stream_t stream);
+
+/*
+ * Rows addressed by (start, len, expert) triples -> per-expert counts,
+ * offsets and a row list grouped by expert (segment order, then row order).
+ * The triple is what the reference plans per block
+ * (mix_moe/mix_moe/transformer.py:242-250: start_addrs, lens, expert_ids) and
+ * its kernels address blocks with (mix_moe/csrc/cuda/mix_gemm.cu:296-301).
+ *   rows int32 [total_rows] out; counts int32 [E]; offsets int32 [E+1].
+ */
+int ccf_segments_to_rows(const int32_t *seg_start, const int32_t *seg_len,
+                         const int32_t *seg_expert, int n_seg, int num_expert,
+                         int total_rows, int32_t *counts, int32_t *offsets,
+                         int32_t *rows, ccf_stream_t stream);
+
+/* ------------------------------------------------- row moves and combine */
+
+/*
+ * out[j, :] = in[pos[j], :] for j < pos_len (fp16 rows of `hidden`).
+ * Replaces _local_scatter_launch, mix_moe/csrc/cuda/mix_moe_kernel.cu:18-42
+ * (which needs pos_len % 32 == 0; this one does not).
+ */
+int ccf_local_scatter(const void *in, void *out, const int32_t *pos,
+                      int pos_len, int hidden, ccf_stream_t stream);
+
+/*
+ * out[pos[j], :] = in[j, :].
+ * Replaces _local_gather_launch, mix_moe/csrc/cuda/mix_moe_kernel.cu:56-79.
+ */
+int ccf_local_gather(const void *in, void *out, const int32_t *pos,
+                     int pos_len, int hidden, ccf_stream_t stream);
+
+/*
+ * out[t, :] = sum_s score[t, s] * y_flat[t*top_k + s, :], fp32 accumulation,
+ * one rounding to fp16.  If inv_pos is not NULL, slots with inv_pos < 0
+ * (dropped) contribute zero and their y_flat rows are never read.
+ * Replaces the bmm combine of MixMOE.forward, mix_moe/mix_moe/layers.py:550-559.
+ */
+int ccf_combine(const void *y_flat, const void *score, const int32_t *inv_pos,
+                void *out, int tokens, int top_k, int hidden,
+                ccf_stream_t stream);
+
+/* ------------------------------------------------------------ expert FFN */
+
+/* Bytes of workspace the FFN entry points need (the device-built tile plan). */
+size_t ccf_ffn_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn);
+
+/*
+ * FFN1 as a grouped GEMM with the scatter fused into the A-tile loads:
+ *   h[dst_row[j], :] = gelu(x[src_row[j], :] * w1[e]^T + b1[e])   for offsets[e] <= j < offsets[e+1]
+ * erf-form GELU, fp16 operands, fp32 MFMA accumulation, fp16 h.
+ * src_row / dst_row NULL mean row j.  offsets lives on the device; max_rows
+ * bounds offsets[num_expert].  apply_gelu = 0 stores the pre-activation instead.
+ * Replaces _MixMOE::first_gemm_forward -> first_mix_gemm -> moe_first_mm,
+ * mix_moe/csrc/mix_moe.h:236-298, mix_moe/csrc/cuda/mix_gemm.cu:282-436, 557-610,
+ * together with the activation the reference runs as a separate kernel
+ * (mix_moe/mix_moe/transformer.py:88).
+ */
+int ccf_ffn1_forward(const void *x, const int32_t *src_row, const int32_t *dst_row,
+                     const int32_t *offsets, int max_rows, int num_expert,
+                     int d_model, int d_ffn, const void *w1, const void *b1,
+                     int apply_gelu, void *h, void *workspace,
+                     size_t workspace_bytes, ccf_stream_t stream);
+
+/*
+ * FFN2 as a grouped GEMM with the un-permute fused into the epilogue:
+ *   y[dst_row[j], :] = (h[src_row[j], :] * w2[e]^T + b2[e]) * (row_scale ? row_scale[j] : 1)
+ * src_row / dst_row NULL mean row j.  Rows of y that no j maps to are left
+ * untouched.
+ * Replaces _MixMOE::second_gemm_forward -> second_mix_gemm -> moe_second_mm and
+ * the index_copy_ that follows it, mix_moe/csrc/mix_moe.h:390-437,
+ * mix_moe/csrc/cuda/mix_gemm.cu:439-555, 668-720.
+ */
+int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row,
+                     const int32_t *offsets, int max_rows, int num_expert,
+                     int d_model, int d_ffn, const void *w2, const void *b2,
+                     const void *row_scale, void *y, void *workspace,
+                     size_t workspace_bytes, ccf_stream_t stream);
+
+/* ------------------------------------------------------- the whole layer */
+
+/* Bytes of workspace ccf_moe_forward needs. */
+size_t ccf_moe_workspace_bytes(int tokens, int d_model, int d_ffn, int num_expert, int top_k);
+
+/*
+ * The MoE layer forward on one GPU: gate -> count/scan/pos (with optional
+ * capacity) -> FFN1 (gather fused) -> GELU -> FFN2 (un-permute fused) ->
+ * gate-weighted combine.  out [tokens, d_model] fp16.
+ * Replaces MixMOETransformerMLP.forward, mix_moe/mix_moe/transformer.py:475-497,
+ * i.e. AsyncExpertAssignment.process_data (376-402) followed by MixMOE.forward
+ * (mix_moe/mix_moe/layers.py:501-559); its single-call C++ form is
+ * _MixMOE::forward, mix_moe/csrc/mix_moe.h:507-598.
+ * Optional outputs (NULL to skip): idx_out int64 [tokens*top_k] (after
+ * capacity), score_out fp16 [tokens*top_k], pos_out int64 [tokens*top_k],
+ * counts_out int32 [num_expert], offsets_out int32 [num_expert+1].
+ */
+int ccf_moe_forward(const void *x, const void *wg, const void *bg,
+                    const void *w1, const void *b1, const void *w2, const void *b2,
+                    int tokens, int d_model, int d_ffn, int num_expert, int top_k,
+                    int capacity, void *out, int64_t *idx_out, void *score_out,
+                    int64_t *pos_out, int32_t *counts_out, int32_t *offsets_out,
+                    void *workspace, size_t workspace_bytes, ccf_stream_t stream);
+
+/*
+ * Profiling hook (no counterpart in the reference).  Gives up to six hipEvent_t
+ * handles; every later ccf_moe_forward on this thread records them on its
+ * stream: [0] before the gate, then after the gate, the count/scan/pos, FFN1,
+ * FFN2 and the combine.  count = 0 switches the recording off.
+ */
+int ccf_moe_forward_set_events(void *const *events, int count);
+
+/* Bytes of workspace ccf_moe_ffn_segments needs. */
+size_t ccf_segments_workspace_bytes(int total_rows, int n_seg, int num_expert,
+                                    int d_model, int d_ffn);
+
+/*
+ * One GPU's expert-parallel share: the expert FFN over an inbound buffer whose
+ * rows are addressed by (start, len, expert) triples; y[r, :] is the FFN
+ * output of inbound row r (same layout as x, ready to be returned to the
+ * senders).  Rows no triple covers are left untouched.
+ * Replaces the block-addressed form of the two fused kernels, where each
+ * block carries (expert_ids, start_addrs, lens),
+ * mix_moe/csrc/cuda/mix_gemm.cu:282-345, 439-490, as called from
+ * _MixMOE::forward, mix_moe/csrc/mix_moe.h:539-575.
+ */
+int ccf_moe_ffn_segments(const void *x, const int32_t *seg_start,
+                         const int32_t *seg_len, const int32_t *seg_expert,
+                         int n_seg, int total_rows, int d_model, int d_ffn,
+                         int num_expert, const void *w1, const void *b1,
+                         const void *w2, const void *b2, void *y,
+                         void *workspace, size_t workspace_bytes,
+                         ccf_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CCFUSER_MOE_H */

@@ -1,0 +1,44 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+def _has_gpu():
+    try:
+        import torch
+        return torch.cuda.is_available()
+    except Exception:
+        return False
+
+
+def pytest_collection_modifyitems(config, items):
+    if _has_gpu():
+        return
+    skip = pytest.mark.skip(reason="no GPU in this container")
+    for item in items:
+        if "gpu" in item.keywords:
+            item.add_marker(skip)
+
+
+@pytest.fixture(scope="session")
+def workloads():
+    """Cache of generated workloads (generation of the big ones takes seconds)."""
+    from ccfuser_amd.workloads import make_workload
+    cache = {}
+
+    def get(name, scale_rows=None):
+        key = (name, scale_rows)
+        if key not in cache:
+            cache[key] = make_workload(name, scale_rows=scale_rows)
+        return cache[key]
+
+    return get

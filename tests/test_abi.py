@@ -1,0 +1,84 @@
+"""The C-ABI library loads and exports every function include/ccfuser_moe.h declares;
+argument checks that need no GPU return error codes instead of crashing."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ccfuser_moe.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ccf_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from ccfuser_amd import _lib
+    if not _lib.LIB_PATH.exists():
+        from ccfuser_amd import build
+        build.build(verbose=False)
+    return _lib.lib()
+
+
+def test_header_and_binding_agree(lib):
+    from ccfuser_amd import _lib
+    names = declared_functions()
+    assert len(names) >= 18
+    assert set(names) == set(_lib.SIGNATURES), "binding table and header differ"
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared but not exported"
+
+
+def test_every_declaration_cites_the_reference_or_says_it_has_none():
+    text = open(HEADER).read()
+    blocks = re.findall(r"/\*(.*?)\*/\s*(?:int|size_t|const char \*)\s*(ccf_[a-z0-9_]+)\s*\(", text, flags=re.S)
+    assert blocks
+    for comment, name in blocks:
+        ok = ("mix_moe/" in comment) or ("no counterpart" in comment) or name in (
+            "ccf_version", "ccf_last_error", "ccf_route_workspace_bytes", "ccf_ffn_workspace_bytes",
+            "ccf_moe_workspace_bytes", "ccf_segments_workspace_bytes")
+        assert ok, f"{name}: declaration comment names no reference interface"
+
+
+def test_version_and_sizes(lib):
+    assert lib.ccf_version() >= 100
+    assert lib.ccf_route_workspace_bytes(32768, 32) > 0
+    assert lib.ccf_ffn_workspace_bytes(8192, 8, 4096, 14336) > 0
+    need = lib.ccf_moe_workspace_bytes(4096, 4096, 14336, 8, 2)
+    # dominated by h [8192, 14336] and y_flat [8192, 4096] in fp16
+    assert 8192 * (14336 + 4096) * 2 <= need <= 8192 * (14336 + 4096) * 2 + (1 << 21)
+    assert lib.ccf_moe_workspace_bytes(-1, 64, 64, 2, 1) == 0
+
+
+def test_argument_errors_are_codes_not_crashes(lib):
+    # null pointers and bad sizes are rejected before anything touches the GPU
+    rc = lib.ccf_gate_topk_softmax(None, None, None, 4, 64, 4, 2, 0, None, None, None, None)
+    assert rc == 1 and b"null" in lib.ccf_last_error()
+    rc = lib.ccf_set_option(b"gemm_variant", 999)
+    assert rc == 1
+    rc = lib.ccf_set_option(b"no_such_option", 0)
+    assert rc == 1 and b"unknown option" in lib.ccf_last_error()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    rc = lib.ccf_gate_topk_softmax(p, p, None, 4, 60, 4, 2, 0, p, p, None, None)
+    assert rc == 2 and b"multiple of 8" in lib.ccf_last_error()
+    rc = lib.ccf_combine(p, p, None, p, 4, 9, 64, None)
+    assert rc == 2
+    rc = lib.ccf_ffn1_forward(p, None, None, p, 8, 2, 64, 64, p, p, 1, p, None, 0, None)
+    assert rc == 3 and b"workspace" in lib.ccf_last_error()
+    rc = lib.ccf_moe_forward(p, p, p, p, p, p, p, 4, 64, 64, 2, 1, -1, p, None, None, None, None,
+                             None, p, 16, None)
+    assert rc == 3
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from ccfuser_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libccfuser_moe.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.lib()
