@@ -86,28 +86,47 @@ struct GroupedArgs {
 
 constexpr int kGroupM = 4;
 
+// erf-form GELU, 0.5*v*(1+erf(v/sqrt2)), with erf from Abramowitz-Stegun 7.1.26
+// (|error| <= 1.5e-7, far below one fp16 ulp of the result):
+//   erf(z) = 1 - (a1 t + .. + a5 t^5) exp(-z^2),  t = 1/(1 + p z),  z >= 0
+// and 0.5*v*(1 + sign(v) erf(|z|)) = 0.5*(v + |v| erf(|z|)).  About 14
+// instructions instead of the library erff's ~40.
 __device__ __forceinline__ float gelu_erf(float v) {
-  return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+  const float az = fabsf(v) * 0.70710678118654752440f;
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, az, 1.0f));
+  float poly = fmaf(1.061405429f, t, -1.453152027f);
+  poly = fmaf(poly, t, 1.421413741f);
+  poly = fmaf(poly, t, -0.284496736f);
+  poly = fmaf(poly, t, 0.254829592f);
+  poly *= t;
+  const float ex = __builtin_amdgcn_exp2f(-1.4426950408889634f * az * az);
+  const float erf_abs = fmaf(-poly, ex, 1.0f);
+  return 0.5f * fmaf(fabsf(v), erf_abs, v);
 }
 
 template <class Cfg, bool kGelu>
-__global__ void __launch_bounds__(Cfg::THREADS)
+__global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_kernel(GroupedArgs p) {
   using ML = GemmMainloop<Cfg>;
-  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn; undo that so
-  // that one XCD (one L2) works on a contiguous run of logical tile ids.
-  const int per_xcd = gridDim.x >> 3;               // grid is a multiple of 8
-  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn.  Undo that
+  // so one XCD (one L2) works on a contiguous run of logical tile ids, and cut
+  // the REAL tiles (known only on the device) into eight equal runs: the grid
+  // is sized for the worst case, and surplus workgroups must not pile up on
+  // the last XCDs.
+  const PlanView pv = plan_view(p.plan, p.max_tiles);
+  const int n_m = pv.n_tiles[0];
+  const int total = n_m * p.n_tiles_n;
+  const int per_xcd = (total + 7) >> 3;
+  const int slot = blockIdx.x >> 3;
+  const int logical = (blockIdx.x & 7) * per_xcd + slot;
+  if (slot >= per_xcd || logical >= total) return;
   // Runs of kGroupM M tiles x all N tiles: neighbours share A rows and B rows.
   const int group_sz = kGroupM * p.n_tiles_n;
   const int first_m = (logical / group_sz) * kGroupM;
-  const int gm = (p.max_tiles - first_m) < kGroupM ? (p.max_tiles - first_m) : kGroupM;
-  if (gm <= 0) return;
+  const int gm = (n_m - first_m) < kGroupM ? (n_m - first_m) : kGroupM;
   const int in_group = logical % group_sz;
   const int tile_m = first_m + in_group % gm;
   const int tile_n = in_group / gm;
-  const PlanView pv = plan_view(p.plan, p.max_tiles);
-  if (tile_m >= pv.n_tiles[0] || tile_n >= p.n_tiles_n) return;
 
   const int e = pv.expert[tile_m];
   const int row0 = pv.row0[tile_m];
@@ -139,44 +158,70 @@ grouped_gemm_kernel(GroupedArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
 
-  ML::run(acc, a_src, b_src, p.K);
-
-  // Epilogue: bias (+ GELU) (+ row scale), fp16 store through the row index.
-  const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
-  float bias_v[Cfg::TN];
-  int col[Cfg::TN];
-#pragma unroll
-  for (int tn = 0; tn < Cfg::TN; ++tn) {
-    col[tn] = n0 + acc_col<Cfg>(tn);
-    bias_v[tn] = col[tn] < p.N ? static_cast<float>(bias_e[col[tn]]) : 0.0f;
+  if constexpr (Cfg::SCHED == 0) {
+    ML::run(acc, a_src, b_src, p.K);
+  } else {
+    ML::run_pingpong(acc, a_src, b_src, p.K);
   }
+
+  // Epilogue: bias (+ GELU) (+ row scale), fp16, 8-byte stores through the row index.
+  const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
+  float bias_v[Cfg::TN][4][4];
+  int col[Cfg::TN][4];
+#pragma unroll
+  for (int tn = 0; tn < Cfg::TN; ++tn)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      col[tn][q] = n0 + acc_col4<Cfg>(tn, q);
+      half4 bv = {0, 0, 0, 0};
+      if (col[tn][q] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn][q]);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) bias_v[tn][q][c] = static_cast<float>(bv[c]);
+    }
 #pragma unroll
   for (int tm = 0; tm < Cfg::TM; ++tm) {
+    const int lr = acc_row<Cfg>(tm);
+    if (lr < rows) {
+      const int j = row0 + lr;
+      const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
+      const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
+      half_t *dst = p.C + crow * p.N;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int lr = acc_row<Cfg>(tm, r);
-      if (lr < rows) {
-        const int j = row0 + lr;
-        const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
-        const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
-        half_t *dst = p.C + crow * p.N;
+      for (int tn = 0; tn < Cfg::TN; ++tn)
 #pragma unroll
-        for (int tn = 0; tn < Cfg::TN; ++tn) {
-          float v = acc[tm][tn][r] + bias_v[tn];
-          if (kGelu) v = gelu_erf(v);
-          v *= sc;
-          if (col[tn] < p.N) dst[col[tn]] = static_cast<half_t>(v);
+        for (int q = 0; q < 4; ++q) {
+          half4 o;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            float v = acc[tm][tn][4 * q + c] + bias_v[tn][q][c];
+            if (kGelu) v = gelu_erf(v);
+            o[c] = static_cast<half_t>(v * sc);
+          }
+          if (col[tn][q] < p.N) *reinterpret_cast<half4 *>(dst + col[tn][q]) = o;
         }
-      }
     }
   }
 }
 
 // ---- variants -------------------------------------------------------------------
 using CfgA = GemmCfg<256, 256, 64, 2, 4, 2>;   // 8 wavefronts, 128x64 each, 128 KB LDS
-using CfgB = GemmCfg<256, 128, 64, 2, 2, 3>;   // 4 wavefronts, 128x64 each, 144 KB LDS
-using CfgC = GemmCfg<128, 128, 64, 2, 2, 2>;   // 4 wavefronts, 64x64 each, 64 KB LDS (2 per CU)
+using CfgB = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1>; // as 0 but tile loads behind every MFMA
+using CfgC = GemmCfg<256, 256, 64, 2, 4, 2, 1, 4>; // as 0 but tile loads behind every 4th MFMA
 using CfgD = GemmCfg<256, 256, 64, 4, 2, 2>;   // 8 wavefronts, 64x128 each
+using CfgE = GemmCfg<256, 256, 32, 2, 4, 4>;   // BK=32, 4 stages, 128 KB LDS
+using CfgF = GemmCfg<256, 256, 32, 2, 4, 5>;   // BK=32, 5 stages, 160 KB LDS
+using CfgG = GemmCfg<256, 128, 32, 2, 2, 3, 2>;   // 4 wavefronts, 72 KB LDS: two workgroups per CU
+using CfgH = GemmCfg<128, 256, 32, 1, 4, 3, 2>;   // 4 wavefronts 128x64, 72 KB LDS: two per CU
+using CfgI = GemmCfg<256, 256, 32, 2, 2, 4>;   // 4 wavefronts, 128x128 each, 128 KB LDS
+using CfgP1 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 0, 1>;   // ping-pong, groups by wave/4, 4 stages
+using CfgP2 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 0, 2>;   // ping-pong, groups by wave%2
+using CfgP3 = GemmCfg<256, 256, 32, 2, 4, 5, 1, 2, 0, 1>;   // ping-pong, 5 stages
+using CfgP4 = GemmCfg<256, 256, 32, 4, 2, 4, 1, 2, 0, 1>;   // ping-pong, 64x128 wavefront tiles
+using CfgX1 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 1>;   // timing experiments on variant 1
+using CfgX2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 2>;
+using CfgX3 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 3>;
+using CfgX4 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 4>;
+using CfgX7 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 7>;
 
 int g_variant = 0;
 
@@ -191,6 +236,20 @@ const Launch kVariants[] = {
     {CfgB::BM, CfgB::BN, CfgB::THREADS, grouped_gemm_kernel<CfgB, false>, grouped_gemm_kernel<CfgB, true>},
     {CfgC::BM, CfgC::BN, CfgC::THREADS, grouped_gemm_kernel<CfgC, false>, grouped_gemm_kernel<CfgC, true>},
     {CfgD::BM, CfgD::BN, CfgD::THREADS, grouped_gemm_kernel<CfgD, false>, grouped_gemm_kernel<CfgD, true>},
+    {CfgE::BM, CfgE::BN, CfgE::THREADS, grouped_gemm_kernel<CfgE, false>, grouped_gemm_kernel<CfgE, true>},
+    {CfgF::BM, CfgF::BN, CfgF::THREADS, grouped_gemm_kernel<CfgF, false>, grouped_gemm_kernel<CfgF, true>},
+    {CfgG::BM, CfgG::BN, CfgG::THREADS, grouped_gemm_kernel<CfgG, false>, grouped_gemm_kernel<CfgG, true>},
+    {CfgH::BM, CfgH::BN, CfgH::THREADS, grouped_gemm_kernel<CfgH, false>, grouped_gemm_kernel<CfgH, true>},
+    {CfgI::BM, CfgI::BN, CfgI::THREADS, grouped_gemm_kernel<CfgI, false>, grouped_gemm_kernel<CfgI, true>},
+    {CfgP1::BM, CfgP1::BN, CfgP1::THREADS, grouped_gemm_kernel<CfgP1, false>, grouped_gemm_kernel<CfgP1, true>},
+    {CfgP2::BM, CfgP2::BN, CfgP2::THREADS, grouped_gemm_kernel<CfgP2, false>, grouped_gemm_kernel<CfgP2, true>},
+    {CfgP3::BM, CfgP3::BN, CfgP3::THREADS, grouped_gemm_kernel<CfgP3, false>, grouped_gemm_kernel<CfgP3, true>},
+    {CfgP4::BM, CfgP4::BN, CfgP4::THREADS, grouped_gemm_kernel<CfgP4, false>, grouped_gemm_kernel<CfgP4, true>},
+    {CfgX1::BM, CfgX1::BN, CfgX1::THREADS, grouped_gemm_kernel<CfgX1, false>, grouped_gemm_kernel<CfgX1, true>},
+    {CfgX2::BM, CfgX2::BN, CfgX2::THREADS, grouped_gemm_kernel<CfgX2, false>, grouped_gemm_kernel<CfgX2, true>},
+    {CfgX3::BM, CfgX3::BN, CfgX3::THREADS, grouped_gemm_kernel<CfgX3, false>, grouped_gemm_kernel<CfgX3, true>},
+    {CfgX4::BM, CfgX4::BN, CfgX4::THREADS, grouped_gemm_kernel<CfgX4, false>, grouped_gemm_kernel<CfgX4, true>},
+    {CfgX7::BM, CfgX7::BN, CfgX7::THREADS, grouped_gemm_kernel<CfgX7, false>, grouped_gemm_kernel<CfgX7, true>},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kMinBM = 128;
@@ -210,7 +269,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   CCF_REQUIRE(E <= 1024, CCF_ERR_SHAPE, "%s: num_expert=%d exceeds 1024", what, E);
   CCF_REQUIRE(K % 64 == 0, CCF_ERR_SHAPE, "%s: K=%d is not a multiple of 64", what, K);
   CCF_REQUIRE(N % 8 == 0, CCF_ERR_SHAPE, "%s: N=%d is not a multiple of 8", what, N);
-  CCF_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C), CCF_ERR_ARG,
+  CCF_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C) && aligned16(bias), CCF_ERR_ARG,
               "%s: operands must be 16-byte aligned", what);
   if (max_rows == 0) return CCF_OK;
   const Launch &v = kVariants[g_variant];

@@ -31,8 +31,15 @@ namespace ccf {
 // a wavefront differ by compile-time constants.
 template <int CPR>
 __device__ __forceinline__ int swz(int r) {
-  static_assert(CPR == 8, "swizzle written for BK = 64");
-  return (r & 7) ^ ((r >> 3) & 1);
+  static_assert(CPR == 8 || CPR == 4, "swizzle written for BK = 64 and BK = 32");
+  if constexpr (CPR == 8) {
+    // 128-byte rows: 8 (and 16) consecutive rows spread over all 16-byte bank groups
+    return (r & 7) ^ ((r >> 3) & 1);
+  } else {
+    // 64-byte rows: two rows per 128 bytes; bits of the result are
+    // (r>>2)&1 and ((r>>3)^(r>>1))&1
+    return (((r >> 2) & 1) << 1) | (((r >> 3) ^ (r >> 1)) & 1);
+  }
 }
 
 typedef __attribute__((address_space(3))) char lds_char;
@@ -93,10 +100,24 @@ __device__ __forceinline__ void lds_dma16(const void *gptr, lds_char *lds_wave_b
                                    (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
 }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WGS_PER_CU_ = 1,
+          int DMA_EVERY_ = 2, int ABLATE_ = 0, int SCHED_ = 0>
 struct GemmCfg {
+  // 0: every wavefront interleaves MFMAs, LDS reads and tile loads.
+  // 1, 2: ping-pong.  The wavefronts form two groups (1: by wave/4, the two that
+  // share a SIMD; 2: by wave%2) that alternate between a memory phase (LDS
+  // fragment reads + tile loads) and a compute phase (a burst of MFMAs on
+  // fragments already in registers), one workgroup barrier per phase, so that
+  // a stall while issuing memory instructions never delays an MFMA.
+  static constexpr int SCHED = SCHED_;
+  // Timing experiments only (results are wrong when set): 1 = no tile loads,
+  // 2 = no LDS fragment reads, 4 = no workgroup barriers.
+  static constexpr int ABLATE = ABLATE_;
+  static constexpr int DMA_EVERY = DMA_EVERY_;         // one tile load behind every n-th MFMA
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
   static constexpr int NW = WM * WN;
+  static constexpr int WGS_PER_CU = WGS_PER_CU_;
+  static constexpr int MIN_WAVES_PER_SIMD = (NW * WGS_PER_CU + 3) / 4;   // register budget
   static constexpr int THREADS = NW * 64;
   static constexpr int WTM = BM / WM, WTN = BN / WN;   // wavefront tile
   static constexpr int TM = WTM / 32, TN = WTN / 32;   // 32x32 MFMA blocks per wavefront
@@ -109,7 +130,7 @@ struct GemmCfg {
   static constexpr int KSTEPS = BK / 16;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wavefront tile");
   static_assert(BM % (ROWS_PER_DMA * NW) == 0 && BN % (ROWS_PER_DMA * NW) == 0, "dma split");
-  static_assert(STAGES >= 2 && STAGES <= 4, "stages");
+  static_assert(STAGES >= 2 && STAGES <= 6, "stages");
 };
 
 // One workgroup's main loop.  a_row_ptr(r) / b_row_ptr(r) give the global
@@ -149,7 +170,9 @@ struct GemmMainloop {
                                                    const int (&a_off)[Cfg::KSTEPS],
                                                    const int (&b_off)[Cfg::KSTEPS]) {
     const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage<S>()));
-    if constexpr (I == 0) {
+    if constexpr ((Cfg::ABLATE & 2) != 0) {
+      return;
+    } else if constexpr (I == 0) {
       a[0] = lds_read_b128<0>(base + a_off[KS]);
     } else if constexpr (I <= Cfg::TN) {
       b[I - 1] = lds_read_b128<Cfg::A_BYTES + (I - 1) * 32 * Cfg::CPR * 16>(base + b_off[KS]);
@@ -158,35 +181,75 @@ struct GemmMainloop {
     }
   }
 
+  // The i-th tile load of this wavefront (A loads first, then B) into stage S.
+  template <int S, int I>
+  static __device__ __forceinline__ void issue_one(const half_t *const (&a_src)[Cfg::A_DMA],
+                                                   const half_t *const (&b_src)[Cfg::B_DMA],
+                                                   int k_elem, int wave) {
+    lds_char *base = stage<S>();
+    if constexpr ((Cfg::ABLATE & 1) != 0) {
+      return;
+    } else if constexpr (I < Cfg::A_DMA) {
+      lds_dma16(a_src[I] + k_elem, base + (I * Cfg::NW + wave) * 1024);
+    } else {
+      lds_dma16(b_src[I - Cfg::A_DMA] + k_elem,
+                base + Cfg::A_BYTES + ((I - Cfg::A_DMA) * Cfg::NW + wave) * 1024);
+    }
+  }
+
   // MFMAs over the K tile held in stage S.  The fragments of K step ks+1 are
-  // read between the MFMAs of step ks into a second register set.  The LDS
+  // read between the MFMAs of step ks into a second register set, and (PREFETCH)
+  // the loads of a later K tile into stage NEXT are issued between MFMAs too,
+  // one behind every DMA_EVERY-th MFMA from the start of the tile: a wavefront
+  // issues in order, so a tile load that waits for a free slot in the texture
+  // address queue would otherwise hold up every MFMA behind it, while issued in
+  // the shadow of an MFMA (32 clocks in the pipe) it costs nothing.  The LDS
   // reads are inline asm (the compiler would otherwise make every LDS read
   // wait for the tile loads in flight), so the lgkmcnt waits are placed here:
   // LDS reads return in order, and before MFMA i of a step the reads still
   // allowed in flight are the later fragments of this step plus the fragments
   // of the next step issued so far.  Scheduling fences keep the source order.
-  template <int S>
+  template <int S, int NEXT, bool PREFETCH>
   static __device__ __forceinline__ void compute(acc_t (&acc)[Cfg::TM][Cfg::TN],
+                                                 const half_t *const (&a_src)[Cfg::A_DMA],
+                                                 const half_t *const (&b_src)[Cfg::B_DMA],
                                                  const int (&a_off)[Cfg::KSTEPS],
-                                                 const int (&b_off)[Cfg::KSTEPS]) {
+                                                 const int (&b_off)[Cfg::KSTEPS], int k_pre,
+                                                 int wave) {
+    constexpr int PER_STEP = Cfg::TM * Cfg::TN;
+    constexpr int PER_TILE = Cfg::A_DMA + Cfg::B_DMA;
     half8 a[2][Cfg::TM], b[2][Cfg::TN];
+    if constexpr ((Cfg::ABLATE & 2) != 0) {
+      static_for<0, Cfg::TM>([&](auto I) { a[0][I.value] = a[1][I.value] = half8{1, 2, 3, 4, 5, 6, 7, 8}; });
+      static_for<0, Cfg::TN>([&](auto I) { b[0][I.value] = b[1][I.value] = half8{1, 1, 2, 2, 3, 3, 4, 4}; });
+    }
     static_for<0, FRAGS>([&](auto I) { read_frag<S, 0, I.value>(a[0], b[0], a_off, b_off); });
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, Cfg::KSTEPS>([&](auto KS) {
       constexpr int ks = KS.value;
       constexpr int cur = ks & 1;
       constexpr bool more = ks + 1 < Cfg::KSTEPS;
-      static_for<0, Cfg::TM * Cfg::TN>([&](auto II) {
+      static_for<0, PER_STEP>([&](auto II) {
         constexpr int i = II.value;
         constexpr int tm = i / Cfg::TN, tn = i % Cfg::TN;
         constexpr int need = a_seq(tm) > b_seq(tn) ? a_seq(tm) : b_seq(tn);
         constexpr int next_issued = more ? (i < FRAGS ? i : FRAGS) : 0;
-        wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
-        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
+        if constexpr ((Cfg::ABLATE & 2) == 0)
+          wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
         if constexpr (more && i < FRAGS) read_frag<S, ks + 1, i>(a[cur ^ 1], b[cur ^ 1], a_off, b_off);
+        constexpr int m = ks * PER_STEP + i;                 // MFMA index within the tile
+        if constexpr (PREFETCH && m % Cfg::DMA_EVERY == 0 && m / Cfg::DMA_EVERY < PER_TILE)
+          issue_one<NEXT, m / Cfg::DMA_EVERY>(a_src, b_src, k_pre, wave);
         __builtin_amdgcn_sched_barrier(0);
       });
     });
+    // a tile with fewer MFMAs than load slots: issue the rest now
+    if constexpr (PREFETCH) {
+      constexpr int slots = (Cfg::KSTEPS * PER_STEP + Cfg::DMA_EVERY - 1) / Cfg::DMA_EVERY;
+      static_for<(slots < PER_TILE ? slots : PER_TILE), PER_TILE>(
+          [&](auto I) { issue_one<NEXT, I.value>(a_src, b_src, k_pre, wave); });
+    }
   }
 
   template <int S>
@@ -200,17 +263,15 @@ struct GemmMainloop {
       constexpr int NEXT = (S + Cfg::STAGES - 1) % Cfg::STAGES;   // stage of tile kt+STAGES-1
       constexpr int PER_TILE = Cfg::A_DMA + Cfg::B_DMA;
       if (kt >= KT) return;                                        // uniform
-      const int kpre = kt + Cfg::STAGES - 1;
-      if (kpre < KT) issue<NEXT>(a_src, b_src, kpre * Cfg::BK, wave);
-      compute<S>(acc, a_off, b_off);
+      // Past the end the prefetch re-reads the last K tile into a stage nobody
+      // reads any more: the loop stays free of branches and the wait counts fixed.
+      int kpre = kt + Cfg::STAGES - 1;
+      kpre = kpre < KT ? kpre : KT - 1;
+      compute<S, NEXT, true>(acc, a_src, b_src, a_off, b_off, kpre * Cfg::BK, wave);
       // tile kt+1 must have landed before anyone reads it: leave at most the
       // loads of the STAGES-2 younger tiles in flight.
-      if (kpre < KT) {
-        wait_vmcnt<PER_TILE *(Cfg::STAGES - 2)>();
-      } else {
-        wait_vmcnt<0>();
-      }
-      block_barrier();
+      wait_vmcnt<PER_TILE *(Cfg::STAGES - 2)>();
+      if constexpr ((Cfg::ABLATE & 4) == 0) block_barrier();
     }
   };
 
@@ -237,31 +298,118 @@ struct GemmMainloop {
     }
 
     // Prologue: tiles 0 .. STAGES-2.
-    if (0 < KT) issue<0>(a_src, b_src, 0, wave);
-    if constexpr (Cfg::STAGES >= 3) {
-      if (1 < KT) issue<1>(a_src, b_src, Cfg::BK, wave);
-    }
-    if constexpr (Cfg::STAGES >= 4) {
-      if (2 < KT) issue<2>(a_src, b_src, 2 * Cfg::BK, wave);
-    }
+    static_for<0, Cfg::STAGES - 1>([&](auto S) {
+      if (S.value < KT) issue<S.value>(a_src, b_src, S.value * Cfg::BK, wave);
+    });
     // tile 0 landed; younger prologue tiles may stay in flight
-    if constexpr (Cfg::STAGES == 2) {
-      wait_vmcnt<0>();
+    if (KT >= Cfg::STAGES - 1) {
+      wait_vmcnt<(Cfg::A_DMA + Cfg::B_DMA) * (Cfg::STAGES - 2)>();
     } else {
-      if (KT >= Cfg::STAGES - 1) {
-        wait_vmcnt<(Cfg::A_DMA + Cfg::B_DMA) * (Cfg::STAGES - 2)>();
-      } else {
-        wait_vmcnt<0>();
-      }
+      wait_vmcnt<0>();
     }
     block_barrier();
 
     for (int kt0 = 0; kt0 < KT; kt0 += Cfg::STAGES) {
-      Step<0>::run(acc, a_src, b_src, a_off, b_off, kt0 + 0, KT, wave);
-      Step<1>::run(acc, a_src, b_src, a_off, b_off, kt0 + 1, KT, wave);
-      if constexpr (Cfg::STAGES >= 3) Step<2>::run(acc, a_src, b_src, a_off, b_off, kt0 + 2, KT, wave);
-      if constexpr (Cfg::STAGES >= 4) Step<3>::run(acc, a_src, b_src, a_off, b_off, kt0 + 3, KT, wave);
+      static_for<0, Cfg::STAGES>([&](auto S) {
+        Step<S.value>::run(acc, a_src, b_src, a_off, b_off, kt0 + S.value, KT, wave);
+      });
     }
+    wait_vmcnt<0>();      // the redundant tail prefetches
+  }
+
+  // ---- ping-pong schedule ---------------------------------------------------
+  // Barrier that first waits for every LDS read in flight; the fragment
+  // registers are tied to the wait so no MFMA can be scheduled above it.
+  static __device__ __forceinline__ void pp_barrier_after_reads(half8 (&a)[Cfg::KSTEPS][Cfg::TM],
+                                                                half8 (&b)[Cfg::KSTEPS][Cfg::TN]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int ks = 0; ks < Cfg::KSTEPS; ++ks) {
+#pragma unroll
+      for (int i = 0; i < Cfg::TM; ++i) asm volatile("" : "+v"(a[ks][i]));
+#pragma unroll
+      for (int i = 0; i < Cfg::TN; ++i) asm volatile("" : "+v"(b[ks][i]));
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  template <int S>
+  struct PingPong {
+    // memory phase of K slice kt (held in stage S), then compute phase
+    static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
+                                               const half_t *const (&a_src)[Cfg::A_DMA],
+                                               const half_t *const (&b_src)[Cfg::B_DMA],
+                                               const int (&a_off)[Cfg::KSTEPS],
+                                               const int (&b_off)[Cfg::KSTEPS], int kt, int KT,
+                                               int wave) {
+      constexpr int NEXT = (S + Cfg::STAGES - 1) % Cfg::STAGES;
+      constexpr int PER_TILE = Cfg::A_DMA + Cfg::B_DMA;
+      if (kt >= KT) return;                                        // uniform
+      int kpre = kt + Cfg::STAGES - 1;
+      kpre = kpre < KT ? kpre : KT - 1;
+      half8 a[Cfg::KSTEPS][Cfg::TM], b[Cfg::KSTEPS][Cfg::TN];
+      // --- memory phase
+      static_for<0, Cfg::KSTEPS>([&](auto KS) {
+        static_for<0, FRAGS>([&](auto I) {
+          read_frag<S, KS.value, I.value>(a[KS.value], b[KS.value], a_off, b_off);
+        });
+      });
+      static_for<0, PER_TILE>([&](auto I) { issue_one<NEXT, I.value>(a_src, b_src, kpre * Cfg::BK, wave); });
+      __builtin_amdgcn_sched_barrier(0);
+      wait_vmcnt<PER_TILE *(Cfg::STAGES - 2)>();
+      pp_barrier_after_reads(a, b);
+      // --- compute phase
+      static_for<0, Cfg::KSTEPS>([&](auto KS) {
+        static_for<0, Cfg::TM * Cfg::TN>([&](auto II) {
+          constexpr int tm = II.value / Cfg::TN, tn = II.value % Cfg::TN;
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[KS.value][tn], a[KS.value][tm],
+                                                               acc[tm][tn], 0, 0, 0);
+        });
+      });
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  static __device__ __forceinline__ void run_pingpong(acc_t (&acc)[Cfg::TM][Cfg::TN],
+                                                      const half_t *const (&a_src)[Cfg::A_DMA],
+                                                      const half_t *const (&b_src)[Cfg::B_DMA],
+                                                      int K) {
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+    const int KT = K / Cfg::BK;
+    const int group = Cfg::SCHED == 1 ? (wave >> 2) & 1 : wave & 1;
+    int a_off[Cfg::KSTEPS], b_off[Cfg::KSTEPS];
+    {
+      const int ra = wm * Cfg::WTM + (lane & 31);
+      const int rb = wn * Cfg::WTN + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < Cfg::KSTEPS; ++ks) {
+        const int c = ks * 2 + (lane >> 5);
+        a_off[ks] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
+        b_off[ks] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
+      }
+    }
+    // Prologue: slices 0 .. STAGES-2 (past the end: the last slice again).
+    static_for<0, Cfg::STAGES - 1>([&](auto S) {
+      const int k = S.value < KT ? S.value : KT - 1;
+      issue<S.value>(a_src, b_src, k * Cfg::BK, wave);
+    });
+    wait_vmcnt<(Cfg::A_DMA + Cfg::B_DMA) * (Cfg::STAGES - 2)>();
+    block_barrier();
+    // The second group runs one phase behind the first.
+    if (group == 1) __builtin_amdgcn_s_barrier();
+    for (int kt0 = 0; kt0 < KT; kt0 += Cfg::STAGES) {
+      static_for<0, Cfg::STAGES>([&](auto S) {
+        PingPong<S.value>::run(acc, a_src, b_src, a_off, b_off, kt0 + S.value, KT, wave);
+      });
+    }
+    if (group == 0) __builtin_amdgcn_s_barrier();
+    wait_vmcnt<0>();
   }
 
   // Tile row this lane fetches with its i-th A (or B) load, and the K-chunk.
@@ -275,18 +423,22 @@ struct GemmMainloop {
   }
 };
 
-// Accumulator element r of block (tm, tn) is C[row, col] with
-//   row = wm*WTM + tm*32 + 8*(r/4) + 4*(lane/32) + r%4
-//   col = wn*WTN + tn*32 + lane%32
+// The weight fragment is the first MFMA operand and the token fragment the
+// second, so a lane owns ONE token row per 32x32 block and, per group of four
+// accumulator registers, four consecutive output columns:
+//   row = wm*WTM + tm*32 + lane%32
+//   col = wn*WTN + tn*32 + 8*(r/4) + 4*(lane/32) + r%4
+// which lets the epilogue look up row data once per block and store 8 bytes at
+// a time.
 template <class Cfg>
-__device__ __forceinline__ int acc_row(int tm, int r) {
+__device__ __forceinline__ int acc_row(int tm) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  return (wave / Cfg::WN) * Cfg::WTM + tm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+  return (wave / Cfg::WN) * Cfg::WTM + tm * 32 + (lane & 31);
 }
 template <class Cfg>
-__device__ __forceinline__ int acc_col(int tn) {
+__device__ __forceinline__ int acc_col4(int tn, int q) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  return (wave % Cfg::WN) * Cfg::WTN + tn * 32 + (lane & 31);
+  return (wave % Cfg::WN) * Cfg::WTN + tn * 32 + 8 * q + 4 * (lane >> 5);
 }
 
 }  // namespace ccf
