@@ -160,6 +160,8 @@ grouped_gemm_kernel(GroupedArgs p) {
 
   if constexpr (Cfg::SCHED == 0) {
     ML::run(acc, a_src, b_src, p.K);
+  } else if constexpr (Cfg::SCHED == 3) {
+    RingMainloop<Cfg>::run(acc, a_src, b_src, p.K);
   } else {
     ML::run_pingpong(acc, a_src, b_src, p.K);
   }
@@ -217,11 +219,25 @@ using CfgP1 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 0, 1>;   // ping-pong, groups
 using CfgP2 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 0, 2>;   // ping-pong, groups by wave%2
 using CfgP3 = GemmCfg<256, 256, 32, 2, 4, 5, 1, 2, 0, 1>;   // ping-pong, 5 stages
 using CfgP4 = GemmCfg<256, 256, 32, 4, 2, 4, 1, 2, 0, 1>;   // ping-pong, 64x128 wavefront tiles
+using CfgR2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 2, 0, 3>;   // five-slot ring, a load behind every 2nd MFMA
+using CfgR4 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 4, 0, 3>;   // five-slot ring, every 4th
+using CfgR1 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 0, 3>;   // five-slot ring, every MFMA
+using CfgR3 = GemmCfg<256, 256, 64, 4, 2, 2, 1, 4, 0, 3>;   // five-slot ring, 64x128 wavefront tiles
+using CfgQ0 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 0, 0>;   // 4 wavefronts of 128x128, two stages
+using CfgQ3 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 0, 3>;   // 4 wavefronts of 128x128, five-slot ring
+using CfgQ2 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 2, 0, 3>;   // same, a load behind every 2nd MFMA
 using CfgX1 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 1>;   // timing experiments on variant 1
 using CfgX2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 2>;
 using CfgX3 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 3>;
 using CfgX4 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 4>;
 using CfgX7 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 7>;
+using CfgY0 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 0, 2>;   // loads only: up front / every 2nd / every 4th MFMA
+using CfgY2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 2, 2>;
+using CfgY4 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 4, 2>;
+using CfgZ0 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 0, 0>;   // full kernel, all loads up front
+using CfgW0 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 0, 10>;  // tile loads only (no MFMA, no LDS reads)
+using CfgW1 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 0, 10>;  // same, BK=32 x 4 stages
+using CfgW2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 0, 8>;   // tile loads + LDS reads, no MFMA
 
 int g_variant = 0;
 
@@ -245,11 +261,25 @@ const Launch kVariants[] = {
     {CfgP2::BM, CfgP2::BN, CfgP2::THREADS, grouped_gemm_kernel<CfgP2, false>, grouped_gemm_kernel<CfgP2, true>},
     {CfgP3::BM, CfgP3::BN, CfgP3::THREADS, grouped_gemm_kernel<CfgP3, false>, grouped_gemm_kernel<CfgP3, true>},
     {CfgP4::BM, CfgP4::BN, CfgP4::THREADS, grouped_gemm_kernel<CfgP4, false>, grouped_gemm_kernel<CfgP4, true>},
+    {CfgR2::BM, CfgR2::BN, CfgR2::THREADS, grouped_gemm_kernel<CfgR2, false>, grouped_gemm_kernel<CfgR2, true>},
+    {CfgR4::BM, CfgR4::BN, CfgR4::THREADS, grouped_gemm_kernel<CfgR4, false>, grouped_gemm_kernel<CfgR4, true>},
+    {CfgR1::BM, CfgR1::BN, CfgR1::THREADS, grouped_gemm_kernel<CfgR1, false>, grouped_gemm_kernel<CfgR1, true>},
+    {CfgR3::BM, CfgR3::BN, CfgR3::THREADS, grouped_gemm_kernel<CfgR3, false>, grouped_gemm_kernel<CfgR3, true>},
+    {CfgQ0::BM, CfgQ0::BN, CfgQ0::THREADS, grouped_gemm_kernel<CfgQ0, false>, grouped_gemm_kernel<CfgQ0, true>},
+    {CfgQ3::BM, CfgQ3::BN, CfgQ3::THREADS, grouped_gemm_kernel<CfgQ3, false>, grouped_gemm_kernel<CfgQ3, true>},
+    {CfgQ2::BM, CfgQ2::BN, CfgQ2::THREADS, grouped_gemm_kernel<CfgQ2, false>, grouped_gemm_kernel<CfgQ2, true>},
     {CfgX1::BM, CfgX1::BN, CfgX1::THREADS, grouped_gemm_kernel<CfgX1, false>, grouped_gemm_kernel<CfgX1, true>},
     {CfgX2::BM, CfgX2::BN, CfgX2::THREADS, grouped_gemm_kernel<CfgX2, false>, grouped_gemm_kernel<CfgX2, true>},
     {CfgX3::BM, CfgX3::BN, CfgX3::THREADS, grouped_gemm_kernel<CfgX3, false>, grouped_gemm_kernel<CfgX3, true>},
     {CfgX4::BM, CfgX4::BN, CfgX4::THREADS, grouped_gemm_kernel<CfgX4, false>, grouped_gemm_kernel<CfgX4, true>},
     {CfgX7::BM, CfgX7::BN, CfgX7::THREADS, grouped_gemm_kernel<CfgX7, false>, grouped_gemm_kernel<CfgX7, true>},
+    {CfgY0::BM, CfgY0::BN, CfgY0::THREADS, grouped_gemm_kernel<CfgY0, false>, grouped_gemm_kernel<CfgY0, true>},
+    {CfgY2::BM, CfgY2::BN, CfgY2::THREADS, grouped_gemm_kernel<CfgY2, false>, grouped_gemm_kernel<CfgY2, true>},
+    {CfgY4::BM, CfgY4::BN, CfgY4::THREADS, grouped_gemm_kernel<CfgY4, false>, grouped_gemm_kernel<CfgY4, true>},
+    {CfgZ0::BM, CfgZ0::BN, CfgZ0::THREADS, grouped_gemm_kernel<CfgZ0, false>, grouped_gemm_kernel<CfgZ0, true>},
+    {CfgW0::BM, CfgW0::BN, CfgW0::THREADS, grouped_gemm_kernel<CfgW0, false>, grouped_gemm_kernel<CfgW0, true>},
+    {CfgW1::BM, CfgW1::BN, CfgW1::THREADS, grouped_gemm_kernel<CfgW1, false>, grouped_gemm_kernel<CfgW1, true>},
+    {CfgW2::BM, CfgW2::BN, CfgW2::THREADS, grouped_gemm_kernel<CfgW2, false>, grouped_gemm_kernel<CfgW2, true>},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kMinBM = 128;

@@ -22,29 +22,47 @@ namespace ccf {
 namespace {
 
 constexpr int kMaxTopK = 8;
-constexpr int kGateTT = 4;   // tokens per wavefront
 constexpr int kGateEG = 8;   // experts accumulated per pass over x
 
+// Eight consecutive K elements as loaded, and acc += x[j] * w[j] for j = 0..7 in
+// order.  For fp16 the product is exact in fp32, so a fused multiply-add on the
+// fp16 operands (v_fma_mix_f32, no conversions) gives the same bits as a
+// multiply followed by an add; for fp32 the two stay separate.
 template <typename T>
-__device__ inline void load8(const T *p, float (&v)[8]);
+struct Chunk;
 
 template <>
-__device__ inline void load8<half_t>(const half_t *p, float (&v)[8]) {
-  half8 h = *reinterpret_cast<const half8 *>(p);
+struct Chunk<half_t> {
+  half8 v;
+  __device__ inline void load(const half_t *p) { v = *reinterpret_cast<const half8 *>(p); }
+  __device__ inline void mac(const Chunk &w, float &acc) const {
 #pragma unroll
-  for (int j = 0; j < 8; ++j) v[j] = static_cast<float>(h[j]);
-}
-
-template <>
-__device__ inline void load8<float>(const float *p, float (&v)[8]) {
-  float4v a = reinterpret_cast<const float4v *>(p)[0];
-  float4v b = reinterpret_cast<const float4v *>(p)[1];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    v[j] = a[j];
-    v[4 + j] = b[j];
+    for (int j = 0; j < 8; ++j)
+      acc = __builtin_fmaf(static_cast<float>(v[j]), static_cast<float>(w.v[j]), acc);
   }
-}
+};
+
+template <>
+struct Chunk<float> {
+  float4v lo, hi;
+  __device__ inline void load(const float *p) {
+    lo = reinterpret_cast<const float4v *>(p)[0];
+    hi = reinterpret_cast<const float4v *>(p)[1];
+  }
+  __device__ inline void mac(const Chunk &w, float &acc) const {
+#pragma clang fp contract(off)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float p = lo[j] * w.lo[j];
+      acc = acc + p;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float p = hi[j] * w.hi[j];
+      acc = acc + p;
+    }
+  }
+};
 
 template <typename T>
 __device__ inline float round_to(float v) {
@@ -55,126 +73,221 @@ __device__ inline bool better(float v, int id, float bv, int bid) {
   return v > bv || (v == bv && id < bid);
 }
 
-template <typename T>
+// One level of the lane fold (see gate_kernel): LIVE values remain, partner lane
+// is lane ^ OFF.  Everything is resolved at compile time so v stays in registers.
+template <int LIVE, int OFF, int N>
+__device__ inline void fold_level(float (&v)[N], int lane) {
+  if constexpr (OFF >= 1) {
+    if constexpr (LIVE > 1) {
+      constexpr int HALF = LIVE / 2;
+      const bool upper = (lane & OFF) != 0;
+#pragma unroll
+      for (int j = 0; j < HALF; ++j) {
+        const float keep = upper ? v[j + HALF] : v[j];
+        const float send = upper ? v[j] : v[j + HALF];
+        v[j] = keep + __shfl_xor(send, OFF, kWave);
+      }
+      fold_level<HALF, OFF / 2, N>(v, lane);
+    } else {
+      v[0] = v[0] + __shfl_xor(v[0], OFF, kWave);
+      fold_level<1, OFF / 2, N>(v, lane);
+    }
+  }
+}
+
+template <int N, int OFF>
+__device__ inline void fold_lanes(float (&v)[N], int lane) {
+  fold_level<N, OFF, N>(v, lane);
+}
+
+// Workgroups are persistent: each stages an expert group's weight rows in LDS
+// once (when they fit, kWLds) and then walks over its share of the tokens, one
+// wavefront scoring TT tokens at a time.  The x chunks of up to kBatch passes
+// are requested together before any arithmetic (one memory round trip for
+// d_model <= 4096).  Logits of all experts are parked in LDS until the last
+// expert group is done, then each wavefront picks the top-k of its tokens.
+// None of this changes the order of the additions.
+template <typename T, int TT, bool kWLds>
 __global__ void __launch_bounds__(256)
 gate_kernel(const T *__restrict__ x, const T *__restrict__ wg, const T *__restrict__ bg,
-            int tokens, int d, int E, int k, int64_t *__restrict__ idx_out,
+            int tokens, int d, int E, int k, int groups_per_block, int64_t *__restrict__ idx_out,
             T *__restrict__ score_out, T *__restrict__ logits_out) {
 #pragma clang fp contract(off)
-  extern __shared__ float s_logit[];               // [4 waves][kGateTT][E]
+  constexpr int kBatch = 8 / TT;                   // x chunks requested together per lane
+  extern __shared__ float s_logit[];               // [groups_per_block][4 waves][TT][E], then weights
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
-  const int t0 = (blockIdx.x * 4 + wave) * kGateTT;
   const int nchunk = d >> 3;
-  float *mine = s_logit + static_cast<size_t>(wave) * kGateTT * E;
-
-  const T *xrow[kGateTT];
-#pragma unroll
-  for (int tt = 0; tt < kGateTT; ++tt) {
-    int t = t0 + tt;
-    if (t > tokens - 1) t = tokens - 1;            // tail waves re-read the last token
-    xrow[tt] = x + static_cast<size_t>(t) * d;
-  }
+  const int niter = (nchunk + kWave - 1) / kWave;
+  const int n_groups = (tokens + 4 * TT - 1) / (4 * TT);
+  T *w_lds = reinterpret_cast<T *>(s_logit + static_cast<size_t>(groups_per_block) * 4 * TT * E);
 
   for (int e0 = 0; e0 < E; e0 += kGateEG) {
-    float acc[kGateTT][kGateEG];
+    const int ng = (E - e0) < kGateEG ? (E - e0) : kGateEG;
+    if (kWLds) {
+      __syncthreads();                             // previous group fully consumed
+      // always kGateEG rows (rows past E repeat the last expert and are discarded),
+      // 16-byte pieces, 8 loads in flight per lane
+      const int per_row = static_cast<int>(static_cast<size_t>(d) * sizeof(T) / 16);
+      const int total = kGateEG * per_row;
+      int4v *dst = reinterpret_cast<int4v *>(w_lds);
+      for (int i0 = threadIdx.x; i0 < total; i0 += 256 * 8) {
+        int4v tmp[8];
 #pragma unroll
-    for (int tt = 0; tt < kGateTT; ++tt)
+        for (int u = 0; u < 8; ++u) {
+          const int i = i0 + u * 256;
+          if (i < total) {
+            int row = e0 + i / per_row;
+            row = row < E ? row : E - 1;
+            tmp[u] = reinterpret_cast<const int4v *>(wg + static_cast<size_t>(row) * d)[i % per_row];
+          }
+        }
 #pragma unroll
-      for (int g = 0; g < kGateEG; ++g) acc[tt][g] = 0.0f;
+        for (int u = 0; u < 8; ++u)
+          if (i0 + u * 256 < total) dst[i0 + u * 256] = tmp[u];
+      }
+      __syncthreads();
+    }
+    const T *wbase = kWLds ? w_lds : wg + static_cast<size_t>(e0) * d;
 
-    for (int c = lane; c < nchunk; c += kWave) {
-      float xv[kGateTT][8];
+    for (int gi = 0; gi < groups_per_block; ++gi) {
+      const int grp = blockIdx.x + gi * gridDim.x;
+      if (grp >= n_groups) break;                  // uniform per workgroup
+      const int t0 = (grp * 4 + wave) * TT;
+      float *mine = s_logit + (static_cast<size_t>(gi) * 4 + wave) * TT * E;
+      const T *xrow[TT];
 #pragma unroll
-      for (int tt = 0; tt < kGateTT; ++tt) load8<T>(xrow[tt] + c * 8, xv[tt]);
+      for (int tt = 0; tt < TT; ++tt) {
+        int t = t0 + tt;
+        if (t > tokens - 1) t = tokens - 1;        // tail waves re-read the last token
+        xrow[tt] = x + static_cast<size_t>(t) * d;
+      }
+      float acc[TT][kGateEG];
 #pragma unroll
-      for (int g = 0; g < kGateEG; ++g) {
-        if (e0 + g < E) {
-          float wv[8];
-          load8<T>(wg + static_cast<size_t>(e0 + g) * d + c * 8, wv);
+      for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-          for (int tt = 0; tt < kGateTT; ++tt)
+        for (int g = 0; g < kGateEG; ++g) acc[tt][g] = 0.0f;
+
+      for (int it0 = 0; it0 < niter; it0 += kBatch) {
+        Chunk<T> xv[kBatch][TT];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              float p = xv[tt][j] * wv[j];
-              acc[tt][g] = acc[tt][g] + p;
+        for (int i = 0; i < kBatch; ++i) {
+          const int c = lane + (it0 + i) * kWave;
+          if (c < nchunk) {
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) xv[i][tt].load(xrow[tt] + c * 8);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+          const int c = lane + (it0 + i) * kWave;
+          if (c < nchunk) {                        // lanes past the end of K skip the whole chunk
+#pragma unroll
+            for (int g = 0; g < kGateEG; ++g) {
+              Chunk<T> wv;
+              if (kWLds) {
+                wv.load(wbase + static_cast<size_t>(g) * d + c * 8);
+              } else {
+                const int row = (e0 + g) < E ? g : (E - 1 - e0);
+                wv.load(wbase + static_cast<size_t>(row) * d + c * 8);
+              }
+#pragma unroll
+              for (int tt = 0; tt < TT; ++tt) xv[i][tt].mac(wv, acc[tt][g]);
             }
+          }
+        }
+      }
+      // Fold the 64 lane sums of all TT*kGateEG accumulators at once.  Level by
+      // level (xor 32, 16, ...) a lane keeps the half of the values its lane bit
+      // selects and adds the partner's copy of them, so N values cost N-1
+      // exchanges instead of 6N; the pairs added at each level, and therefore
+      // the bits of the result, are those of the plain butterfly.  Value i ends
+      // up in the lanes whose top log2(N) lane bits spell i.
+      constexpr int N = TT * kGateEG;
+      float v[N];
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+        for (int g = 0; g < kGateEG; ++g) v[tt * kGateEG + g] = acc[tt][g];
+      fold_lanes<N, 32>(v, lane);
+      {
+        constexpr int kBits = N == 32 ? 5 : (N == 16 ? 4 : 3);
+        static_assert(N == 8 || N == 16 || N == 32, "TT*kGateEG");
+        const int i = lane >> (6 - kBits);                      // value this lane holds
+        const int tt = i / kGateEG, g = i % kGateEG;
+        if ((lane & ((1 << (6 - kBits)) - 1)) == 0 && g < ng) {
+          float b = bg ? static_cast<float>(bg[e0 + g]) : 0.0f;
+          mine[tt * E + e0 + g] = round_to<T>(v[0] + b);
         }
       }
     }
-#pragma unroll
-    for (int tt = 0; tt < kGateTT; ++tt)
-#pragma unroll
-      for (int g = 0; g < kGateEG; ++g) {
-        float v = acc[tt][g];
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, kWave);
-        if (lane == 0 && e0 + g < E) {
-          float b = bg ? static_cast<float>(bg[e0 + g]) : 0.0f;
-          mine[tt * E + e0 + g] = round_to<T>(v + b);
-        }
-      }
   }
   __syncthreads();
 
+  for (int gi = 0; gi < groups_per_block; ++gi) {
+    const int grp = blockIdx.x + gi * gridDim.x;
+    if (grp >= n_groups) break;
+    const int t0 = (grp * 4 + wave) * TT;
+    const float *mine = s_logit + (static_cast<size_t>(gi) * 4 + wave) * TT * E;
 #pragma unroll 1
-  for (int tt = 0; tt < kGateTT; ++tt) {
-    const int t = t0 + tt;
-    if (t >= tokens) break;                        // uniform per wave
-    const float *lg = mine + tt * E;
-    if (logits_out)
-      for (int e = lane; e < E; e += kWave)
-        logits_out[static_cast<size_t>(t) * E + e] = static_cast<T>(lg[e]);
+    for (int tt = 0; tt < TT; ++tt) {
+      const int t = t0 + tt;
+      if (t >= tokens) break;                      // uniform per wave
+      const float *lg = mine + tt * E;
+      if (logits_out)
+        for (int e = lane; e < E; e += kWave)
+          logits_out[static_cast<size_t>(t) * E + e] = static_cast<T>(lg[e]);
 
-    float sel_v[kMaxTopK];
-    int sel_id[kMaxTopK];
-#pragma unroll
-    for (int s = 0; s < kMaxTopK; ++s) {
-      sel_v[s] = 0.0f;
-      sel_id[s] = -1;
-    }
-#pragma unroll
-    for (int s = 0; s < kMaxTopK; ++s) {
-      if (s < k) {
-        float bv = -INFINITY;
-        int bid = INT_MAX;
-        for (int e = lane; e < E; e += kWave) {
-          bool taken = false;
-#pragma unroll
-          for (int q = 0; q < kMaxTopK; ++q) taken = taken || (q < s && sel_id[q] == e);
-          float v = lg[e];
-          if (!taken && better(v, e, bv, bid)) {
-            bv = v;
-            bid = e;
-          }
-        }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-          float ov = __shfl_xor(bv, off, kWave);
-          int oi = __shfl_xor(bid, off, kWave);
-          if (better(ov, oi, bv, bid)) {
-            bv = ov;
-            bid = oi;
-          }
-        }
-        sel_v[s] = bv;
-        sel_id[s] = bid;
-      }
-    }
-    if (lane == 0) {
-      // softmax over the k selected logits; slot 0 holds the maximum
-      float ex[kMaxTopK];
-      float sum = 0.0f;
+      float sel_v[kMaxTopK];
+      int sel_id[kMaxTopK];
 #pragma unroll
       for (int s = 0; s < kMaxTopK; ++s) {
-        ex[s] = (s < k) ? expf(sel_v[s] - sel_v[0]) : 0.0f;
-        sum += ex[s];
+        sel_v[s] = 0.0f;
+        sel_id[s] = -1;
       }
 #pragma unroll
       for (int s = 0; s < kMaxTopK; ++s) {
         if (s < k) {
-          idx_out[static_cast<size_t>(t) * k + s] = static_cast<int64_t>(sel_id[s]);
-          score_out[static_cast<size_t>(t) * k + s] = static_cast<T>(ex[s] / sum);
+          float bv = -INFINITY;
+          int bid = INT_MAX;
+          for (int e = lane; e < E; e += kWave) {
+            bool taken = false;
+#pragma unroll
+            for (int q = 0; q < kMaxTopK; ++q) taken = taken || (q < s && sel_id[q] == e);
+            float v = lg[e];
+            if (!taken && better(v, e, bv, bid)) {
+              bv = v;
+              bid = e;
+            }
+          }
+#pragma unroll
+          for (int off = 32; off >= 1; off >>= 1) {
+            float ov = __shfl_xor(bv, off, kWave);
+            int oi = __shfl_xor(bid, off, kWave);
+            if (better(ov, oi, bv, bid)) {
+              bv = ov;
+              bid = oi;
+            }
+          }
+          sel_v[s] = bv;
+          sel_id[s] = bid;
+        }
+      }
+      if (lane == 0) {
+        // softmax over the k selected logits; slot 0 holds the maximum
+        float ex[kMaxTopK];
+        float sum = 0.0f;
+#pragma unroll
+        for (int s = 0; s < kMaxTopK; ++s) {
+          ex[s] = (s < k) ? expf(sel_v[s] - sel_v[0]) : 0.0f;
+          sum += ex[s];
+        }
+#pragma unroll
+        for (int s = 0; s < kMaxTopK; ++s) {
+          if (s < k) {
+            idx_out[static_cast<size_t>(t) * k + s] = static_cast<int64_t>(sel_id[s]);
+            score_out[static_cast<size_t>(t) * k + s] = static_cast<T>(ex[s] / sum);
+          }
         }
       }
     }
@@ -198,19 +311,47 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
   CCF_REQUIRE(dtype == CCF_F16 || dtype == CCF_F32, CCF_ERR_UNSUPPORTED, "gate: dtype %d", dtype);
   CCF_REQUIRE(aligned16(x) && aligned16(wg), CCF_ERR_ARG, "gate: x and wg must be 16-byte aligned");
   if (tokens == 0) return CCF_OK;
-  const int tokens_per_block = 4 * kGateTT;
-  dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block), block(256);
-  size_t lds = sizeof(float) * 4 * kGateTT * static_cast<size_t>(tot_expert);
+  // Enough wavefronts to hide HBM latency: fewer tokens per wavefront when the batch is small.
+  const int tt = tokens >= 32768 ? 4 : (tokens >= 8192 ? 2 : 1);
+  const int group = tot_expert < kGateEG ? tot_expert : kGateEG;
+  const size_t esz = dtype == CCF_F16 ? 2 : 4;
+  const size_t w_bytes = static_cast<size_t>(group) * d_model * esz;
+  const bool w_lds = w_bytes <= 65536;             // one expert group of weights fits next to the logits
+  const int n_groups = (tokens + 4 * tt - 1) / (4 * tt);
+  const int max_blocks = 512;                      // two persistent workgroups per CU
+  const int blocks = n_groups < max_blocks ? n_groups : max_blocks;
+  const int groups_per_block = (n_groups + blocks - 1) / blocks;
+  dim3 grid(blocks), block(256);
+  const size_t lds = sizeof(float) * 4 * tt * static_cast<size_t>(tot_expert) * groups_per_block +
+                     (w_lds ? w_bytes : 0);
+  CCF_REQUIRE(lds <= 160 * 1024, CCF_ERR_SHAPE, "gate: %zu bytes of LDS needed", lds);
+#define CCF_GATE_LAUNCH(TYPE, TT, WL)                                                              \
+  do {                                                                                             \
+    auto kern = gate_kernel<TYPE, TT, WL>;                                                         \
+    if (lds > 65536) {                                                                             \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                     \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,               \
+                                         static_cast<int>(lds));                                   \
+      if (e != hipSuccess) return fail(CCF_ERR_HIP, "gate: LDS attribute: %s", hipGetErrorString(e)); \
+    }                                                                                              \
+    hipLaunchKernelGGL(kern, grid, block, lds, as_stream(stream), static_cast<const TYPE *>(x),    \
+                       static_cast<const TYPE *>(wg), static_cast<const TYPE *>(bg), tokens,      \
+                       d_model, tot_expert, top_k, groups_per_block, idx_out,                      \
+                       static_cast<TYPE *>(score_out),                                             \
+                       static_cast<TYPE *>(logits_out));                                           \
+  } while (0)
+#define CCF_GATE_TT(TYPE, WL)                    \
+  do {                                           \
+    if (tt == 4) CCF_GATE_LAUNCH(TYPE, 4, WL);   \
+    else if (tt == 2) CCF_GATE_LAUNCH(TYPE, 2, WL); \
+    else CCF_GATE_LAUNCH(TYPE, 1, WL);           \
+  } while (0)
   if (dtype == CCF_F16) {
-    hipLaunchKernelGGL(gate_kernel<half_t>, grid, block, lds, as_stream(stream),
-                       static_cast<const half_t *>(x), static_cast<const half_t *>(wg),
-                       static_cast<const half_t *>(bg), tokens, d_model, tot_expert, top_k, idx_out,
-                       static_cast<half_t *>(score_out), static_cast<half_t *>(logits_out));
+    if (w_lds) CCF_GATE_TT(half_t, true); else CCF_GATE_TT(half_t, false);
   } else {
-    hipLaunchKernelGGL(gate_kernel<float>, grid, block, lds, as_stream(stream),
-                       static_cast<const float *>(x), static_cast<const float *>(wg),
-                       static_cast<const float *>(bg), tokens, d_model, tot_expert, top_k, idx_out,
-                       static_cast<float *>(score_out), static_cast<float *>(logits_out));
+    if (w_lds) CCF_GATE_TT(float, true); else CCF_GATE_TT(float, false);
   }
+#undef CCF_GATE_TT
+#undef CCF_GATE_LAUNCH
   return check_launch("gate_kernel");
 }

@@ -81,8 +81,14 @@ __device__ __forceinline__ void static_for(F &&f) {
 // scheduled ahead of it.
 template <int N>
 __device__ __forceinline__ void wait_lgkmcnt(half8 &x, half8 &y) {
-  static_assert(N >= 0 && N < 15, "lgkmcnt");
-  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+  static_assert(N >= 0, "lgkmcnt");
+  if constexpr (N < 15) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+  } else {
+    // the counter has four bits: more than 15 LDS reads are never in flight,
+    // so "at most 15" always holds; keep the ordering tie only
+    asm volatile("" : "+v"(x), "+v"(y));
+  }
 }
 
 // 16 bytes per lane from LDS byte address addr + OFF.
@@ -111,7 +117,7 @@ struct GemmCfg {
   // a stall while issuing memory instructions never delays an MFMA.
   static constexpr int SCHED = SCHED_;
   // Timing experiments only (results are wrong when set): 1 = no tile loads,
-  // 2 = no LDS fragment reads, 4 = no workgroup barriers.
+  // 2 = no LDS fragment reads, 4 = no workgroup barriers, 8 = no MFMAs.
   static constexpr int ABLATE = ABLATE_;
   static constexpr int DMA_EVERY = DMA_EVERY_;         // one tile load behind every n-th MFMA
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
@@ -219,9 +225,24 @@ struct GemmMainloop {
     constexpr int PER_STEP = Cfg::TM * Cfg::TN;
     constexpr int PER_TILE = Cfg::A_DMA + Cfg::B_DMA;
     half8 a[2][Cfg::TM], b[2][Cfg::TN];
+    if constexpr (PREFETCH && Cfg::DMA_EVERY == 0) {       // all tile loads up front
+      static_for<0, PER_TILE>([&](auto I) { issue_one<NEXT, I.value>(a_src, b_src, k_pre, wave); });
+      __builtin_amdgcn_sched_barrier(0);
+    }
     if constexpr ((Cfg::ABLATE & 2) != 0) {
-      static_for<0, Cfg::TM>([&](auto I) { a[0][I.value] = a[1][I.value] = half8{1, 2, 3, 4, 5, 6, 7, 8}; });
-      static_for<0, Cfg::TN>([&](auto I) { b[0][I.value] = b[1][I.value] = half8{1, 1, 2, 2, 3, 3, 4, 4}; });
+      // stand-in operands with realistic bit toggling (timing experiments only)
+      unsigned x = threadIdx.x * 2654435761u + 12345u;
+      auto rnd = [&](float scale) {
+        half8 v;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+          v[j] = static_cast<half_t>((static_cast<int>(x & 0xffff) - 32768) / 32768.0f * scale);
+        }
+        return v;
+      };
+      static_for<0, Cfg::TM>([&](auto I) { a[0][I.value] = rnd(1.0f); a[1][I.value] = rnd(1.0f); });
+      static_for<0, Cfg::TN>([&](auto I) { b[0][I.value] = rnd(0.03f); b[1][I.value] = rnd(0.03f); });
     }
     static_for<0, FRAGS>([&](auto I) { read_frag<S, 0, I.value>(a[0], b[0], a_off, b_off); });
     __builtin_amdgcn_sched_barrier(0);
@@ -236,17 +257,21 @@ struct GemmMainloop {
         constexpr int next_issued = more ? (i < FRAGS ? i : FRAGS) : 0;
         if constexpr ((Cfg::ABLATE & 2) == 0)
           wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
-        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
+        if constexpr ((Cfg::ABLATE & 8) == 0)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
         if constexpr (more && i < FRAGS) read_frag<S, ks + 1, i>(a[cur ^ 1], b[cur ^ 1], a_off, b_off);
         constexpr int m = ks * PER_STEP + i;                 // MFMA index within the tile
-        if constexpr (PREFETCH && m % Cfg::DMA_EVERY == 0 && m / Cfg::DMA_EVERY < PER_TILE)
-          issue_one<NEXT, m / Cfg::DMA_EVERY>(a_src, b_src, k_pre, wave);
+        if constexpr (PREFETCH && Cfg::DMA_EVERY > 0) {
+          if constexpr (m % (Cfg::DMA_EVERY > 0 ? Cfg::DMA_EVERY : 1) == 0 &&
+                        m / (Cfg::DMA_EVERY > 0 ? Cfg::DMA_EVERY : 1) < PER_TILE)
+            issue_one<NEXT, m / (Cfg::DMA_EVERY > 0 ? Cfg::DMA_EVERY : 1)>(a_src, b_src, k_pre, wave);
+        }
         __builtin_amdgcn_sched_barrier(0);
       });
     });
     // a tile with fewer MFMAs than load slots: issue the rest now
-    if constexpr (PREFETCH) {
-      constexpr int slots = (Cfg::KSTEPS * PER_STEP + Cfg::DMA_EVERY - 1) / Cfg::DMA_EVERY;
+    if constexpr (PREFETCH && Cfg::DMA_EVERY > 0) {
+      constexpr int slots = (Cfg::KSTEPS * PER_STEP + Cfg::DMA_EVERY - 1) / (Cfg::DMA_EVERY > 0 ? Cfg::DMA_EVERY : 1);
       static_for<(slots < PER_TILE ? slots : PER_TILE), PER_TILE>(
           [&](auto I) { issue_one<NEXT, I.value>(a_src, b_src, k_pre, wave); });
     }
@@ -420,6 +445,135 @@ struct GemmMainloop {
   static __device__ __forceinline__ int dma_chunk(int row) {
     const int lane = threadIdx.x & 63;
     return (lane % Cfg::CPR) ^ swz<Cfg::CPR>(row);
+  }
+};
+
+// ---- five-slot ring ------------------------------------------------------------
+// 256x256x64 tiles need 64 KB of LDS per K tile, so only two whole tiles fit in
+// the CU's 160 KB, and with two stages a tile's loads must all have landed
+// before the next tile's can be issued: the memory pipe drains once per K tile
+// (measured: 12 TB/s into LDS against 16 TB/s when loads of two tiles overlap).
+// Here the A half and the B half of a K tile are separate 32 KB slots of a ring
+// of five.  While tile k is computed, A(k+1) is resident, B(k+1) and A(k+2) are
+// in flight; at the end of the step only B(k+1) must have landed, A(k+2) keeps
+// flying across the barrier.  Every load is a whole 128-byte line and there is
+// still one barrier per K tile.
+template <class Cfg>
+struct RingMainloop {
+  using acc_t = float16v;
+  using Base = GemmMainloop<Cfg>;
+  static_assert(Cfg::A_BYTES == Cfg::B_BYTES, "ring slots are one size");
+  static constexpr int NSLOT = 5;
+  static constexpr int FRAGS = Cfg::TM + Cfg::TN;
+
+  template <int S>
+  static __device__ __forceinline__ lds_char *slot() {
+    return stage_buf<100 + S, Cfg::A_BYTES>();
+  }
+
+  template <int SLOT, int N>
+  static __device__ __forceinline__ void issue_all(const half_t *const (&src)[N], int k_elem, int wave) {
+    static_for<0, N>([&](auto I) {
+      lds_dma16(src[I.value] + k_elem, slot<SLOT>() + (I.value * Cfg::NW + wave) * 1024);
+    });
+  }
+
+  template <int SA, int SB, int KS, int I>
+  static __device__ __forceinline__ void read_frag(half8 (&a)[Cfg::TM], half8 (&b)[Cfg::TN],
+                                                   const int (&a_off)[Cfg::KSTEPS],
+                                                   const int (&b_off)[Cfg::KSTEPS]) {
+    const uint32_t base_a = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(slot<SA>()));
+    const uint32_t base_b = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(slot<SB>()));
+    if constexpr (I == 0) {
+      a[0] = lds_read_b128<0>(base_a + a_off[KS]);
+    } else if constexpr (I <= Cfg::TN) {
+      b[I - 1] = lds_read_b128<(I - 1) * 32 * Cfg::CPR * 16>(base_b + b_off[KS]);
+    } else {
+      a[I - Cfg::TN] = lds_read_b128<(I - Cfg::TN) * 32 * Cfg::CPR * 16>(base_a + a_off[KS]);
+    }
+  }
+
+  template <int U>
+  struct Step {
+    static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
+                                               const half_t *const (&a_src)[Cfg::A_DMA],
+                                               const half_t *const (&b_src)[Cfg::B_DMA],
+                                               const int (&a_off)[Cfg::KSTEPS],
+                                               const int (&b_off)[Cfg::KSTEPS], int kt, int KT,
+                                               int wave) {
+      constexpr int SA = (2 * U) % NSLOT, SB = (2 * U + 1) % NSLOT;       // tile kt
+      constexpr int WB = (2 * U + 3) % NSLOT, WA = (2 * U + 4) % NSLOT;   // B(kt+1), A(kt+2)
+      constexpr int PER_STEP = Cfg::TM * Cfg::TN;
+      constexpr int LOADS = Cfg::A_DMA + Cfg::B_DMA;
+      if (kt >= KT) return;                                               // uniform
+      // past the end the last K tile is fetched again into slots nobody reads
+      const int kb = ((kt + 1 < KT) ? kt + 1 : KT - 1) * Cfg::BK;
+      const int ka = ((kt + 2 < KT) ? kt + 2 : KT - 1) * Cfg::BK;
+      half8 a[2][Cfg::TM], b[2][Cfg::TN];
+      static_for<0, FRAGS>([&](auto I) { read_frag<SA, SB, 0, I.value>(a[0], b[0], a_off, b_off); });
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<0, Cfg::KSTEPS>([&](auto KS) {
+        constexpr int ks = KS.value;
+        constexpr int cur = ks & 1;
+        constexpr bool more = ks + 1 < Cfg::KSTEPS;
+        static_for<0, PER_STEP>([&](auto II) {
+          constexpr int i = II.value;
+          constexpr int tm = i / Cfg::TN, tn = i % Cfg::TN;
+          constexpr int need = Base::a_seq(tm) > Base::b_seq(tn) ? Base::a_seq(tm) : Base::b_seq(tn);
+          constexpr int next_issued = more ? (i < FRAGS ? i : FRAGS) : 0;
+          wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
+          if constexpr (more && i < FRAGS) read_frag<SA, SB, ks + 1, i>(a[cur ^ 1], b[cur ^ 1], a_off, b_off);
+          constexpr int m = ks * PER_STEP + i;
+          if constexpr (m % Cfg::DMA_EVERY == 0 && m / Cfg::DMA_EVERY < LOADS) {
+            constexpr int l = m / Cfg::DMA_EVERY;                         // B loads first, then A
+            if constexpr (l < Cfg::B_DMA) {
+              lds_dma16(b_src[l] + kb, slot<WB>() + (l * Cfg::NW + wave) * 1024);
+            } else {
+              lds_dma16(a_src[l - Cfg::B_DMA] + ka, slot<WA>() + ((l - Cfg::B_DMA) * Cfg::NW + wave) * 1024);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      });
+      static_assert((Cfg::KSTEPS * PER_STEP + Cfg::DMA_EVERY - 1) / Cfg::DMA_EVERY >= LOADS,
+                    "not enough MFMA slots for the tile loads");
+      // B(kt+1) and everything older have landed; A(kt+2) may stay in flight
+      wait_vmcnt<Cfg::A_DMA>();
+      block_barrier();
+    }
+  };
+
+  static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
+                                             const half_t *const (&a_src)[Cfg::A_DMA],
+                                             const half_t *const (&b_src)[Cfg::B_DMA], int K) {
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+    const int KT = K / Cfg::BK;
+    int a_off[Cfg::KSTEPS], b_off[Cfg::KSTEPS];
+    {
+      const int ra = wm * Cfg::WTM + (lane & 31);
+      const int rb = wn * Cfg::WTN + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < Cfg::KSTEPS; ++ks) {
+        const int c = ks * 2 + (lane >> 5);
+        a_off[ks] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
+        b_off[ks] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
+      }
+    }
+    // Prologue: A(0) -> slot 0, B(0) -> slot 1, A(1) -> slot 2.
+    issue_all<0>(a_src, 0, wave);
+    issue_all<1>(b_src, 0, wave);
+    issue_all<2>(a_src, (KT > 1 ? 1 : 0) * Cfg::BK, wave);
+    wait_vmcnt<Cfg::A_DMA>();
+    block_barrier();
+    for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
+      static_for<0, NSLOT>([&](auto U) {
+        Step<U.value>::run(acc, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave);
+      });
+    }
+    wait_vmcnt<0>();
   }
 };
 
