@@ -39,28 +39,47 @@ __device__ inline PlanView plan_view(const int32_t *plan, int max_tiles) {
 __global__ void __launch_bounds__(256)
 plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, int max_rows,
             int32_t *__restrict__ plan) {
+  __shared__ int s_off[1025];
   __shared__ int s_base[1025];
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int e = 0; e < E; ++e) {
-      s_base[e] = run;
-      int lo = offsets[e], hi = offsets[e + 1];
-      if (hi > max_rows) hi = max_rows;              // never plan past the caller's bound
-      int cnt = hi > lo ? hi - lo : 0;
-      run += (cnt + BM - 1) / BM;
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) {
+    int v = offsets[e];
+    s_off[e] = v < max_rows ? v : max_rows;          // never plan past the caller's bound
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    // exclusive scan of the per-expert tile counts by one wavefront
+    const int lane = threadIdx.x;
+    int carry = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      const int e = e0 + lane;
+      int cnt = e < E ? s_off[e + 1] - s_off[e] : 0;
+      cnt = cnt > 0 ? cnt : 0;
+      const int nt = (cnt + BM - 1) / BM;
+      int inc = nt;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        int o = __shfl_up(inc, off, 64);
+        if (lane >= off) inc += o;
+      }
+      if (e < E) s_base[e] = carry + inc - nt;
+      carry += __shfl(inc, 63, 64);
     }
-    s_base[E] = run;
-    plan[0] = run < max_tiles ? run : max_tiles;
+    if (lane == 0) {
+      s_base[E] = carry;
+      plan[0] = carry < max_tiles ? carry : max_tiles;
+    }
   }
   __syncthreads();
   int32_t *expert = plan + 64, *row0 = expert + max_tiles, *rows = row0 + max_tiles;
-  for (int e = threadIdx.x; e < E; e += blockDim.x) {
-    int lo = offsets[e], hi = offsets[e + 1];
-    if (hi > max_rows) hi = max_rows;
-    int cnt = hi > lo ? hi - lo : 0;
-    int nt = s_base[e + 1] - s_base[e];
-    for (int i = 0; i < nt; ++i) {
-      int t = s_base[e] + i;
+  // one wavefront per expert, one lane per tile
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
+  for (int e = wave; e < E; e += nwave) {
+    const int lo = s_off[e];
+    int cnt = s_off[e + 1] - lo;
+    cnt = cnt > 0 ? cnt : 0;
+    const int nt = s_base[e + 1] - s_base[e];
+    for (int i = lane; i < nt; i += 64) {
+      const int t = s_base[e] + i;
       if (t >= max_tiles) break;
       expert[t] = e;
       row0[t] = lo + i * BM;
@@ -161,7 +180,7 @@ grouped_gemm_kernel(GroupedArgs p) {
   if constexpr (Cfg::SCHED == 0) {
     ML::run(acc, a_src, b_src, p.K);
   } else if constexpr (Cfg::SCHED == 3) {
-    RingMainloop<Cfg>::run(acc, a_src, b_src, p.K);
+    RingMainloop<Cfg>::run(acc, a_src, b_src, p.K, rows);
   } else {
     ML::run_pingpong(acc, a_src, b_src, p.K);
   }
@@ -206,38 +225,15 @@ grouped_gemm_kernel(GroupedArgs p) {
 }
 
 // ---- variants -------------------------------------------------------------------
-using CfgA = GemmCfg<256, 256, 64, 2, 4, 2>;   // 8 wavefronts, 128x64 each, 128 KB LDS
-using CfgB = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1>; // as 0 but tile loads behind every MFMA
-using CfgC = GemmCfg<256, 256, 64, 2, 4, 2, 1, 4>; // as 0 but tile loads behind every 4th MFMA
-using CfgD = GemmCfg<256, 256, 64, 4, 2, 2>;   // 8 wavefronts, 64x128 each
-using CfgE = GemmCfg<256, 256, 32, 2, 4, 4>;   // BK=32, 4 stages, 128 KB LDS
-using CfgF = GemmCfg<256, 256, 32, 2, 4, 5>;   // BK=32, 5 stages, 160 KB LDS
-using CfgG = GemmCfg<256, 128, 32, 2, 2, 3, 2>;   // 4 wavefronts, 72 KB LDS: two workgroups per CU
-using CfgH = GemmCfg<128, 256, 32, 1, 4, 3, 2>;   // 4 wavefronts 128x64, 72 KB LDS: two per CU
-using CfgI = GemmCfg<256, 256, 32, 2, 2, 4>;   // 4 wavefronts, 128x128 each, 128 KB LDS
-using CfgP1 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 0, 1>;   // ping-pong, groups by wave/4, 4 stages
-using CfgP2 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 0, 2>;   // ping-pong, groups by wave%2
-using CfgP3 = GemmCfg<256, 256, 32, 2, 4, 5, 1, 2, 0, 1>;   // ping-pong, 5 stages
-using CfgP4 = GemmCfg<256, 256, 32, 4, 2, 4, 1, 2, 0, 1>;   // ping-pong, 64x128 wavefront tiles
-using CfgR2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 2, 0, 3>;   // five-slot ring, a load behind every 2nd MFMA
-using CfgR4 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 4, 0, 3>;   // five-slot ring, every 4th
-using CfgR1 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 0, 3>;   // five-slot ring, every MFMA
-using CfgR3 = GemmCfg<256, 256, 64, 4, 2, 2, 1, 4, 0, 3>;   // five-slot ring, 64x128 wavefront tiles
-using CfgQ0 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 0, 0>;   // 4 wavefronts of 128x128, two stages
-using CfgQ3 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 0, 3>;   // 4 wavefronts of 128x128, five-slot ring
-using CfgQ2 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 2, 0, 3>;   // same, a load behind every 2nd MFMA
-using CfgX1 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 1>;   // timing experiments on variant 1
-using CfgX2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 2>;
-using CfgX3 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 3>;
-using CfgX4 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 4>;
-using CfgX7 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 7>;
-using CfgY0 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 0, 2>;   // loads only: up front / every 2nd / every 4th MFMA
-using CfgY2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 2, 2>;
-using CfgY4 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 4, 2>;
-using CfgZ0 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 0, 0>;   // full kernel, all loads up front
-using CfgW0 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 0, 10>;  // tile loads only (no MFMA, no LDS reads)
-using CfgW1 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 0, 10>;  // same, BK=32 x 4 stages
-using CfgW2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 0, 8>;   // tile loads + LDS reads, no MFMA
+// 256x256x64 tiles throughout (the most flop per byte pulled from L2 that the
+// register file allows).  What differs is how the tile loads are pipelined and
+// how the wavefronts split the tile; variant 0 is the default, the others are
+// kept for measurement (ccf_set_option("gemm_variant", n)).
+using Cfg0 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 2, 3>;   // 8 wavefronts of 128x64, five-slot ring
+using Cfg1 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 3>;   // 4 wavefronts of 128x128, five-slot ring
+using Cfg2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 0>;   // 8 wavefronts, two whole-tile stages
+using Cfg3 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 1>;   // 8 wavefronts, BK=32 x 4 stages, ping-pong
+using Cfg4 = GemmCfg<256, 128, 32, 2, 2, 3, 2, 2, 0>;   // 4 wavefronts, 72 KB LDS: two workgroups per CU
 
 int g_variant = 0;
 
@@ -247,40 +243,10 @@ struct Launch {
   void (*gelu)(GroupedArgs);
 };
 
-const Launch kVariants[] = {
-    {CfgA::BM, CfgA::BN, CfgA::THREADS, grouped_gemm_kernel<CfgA, false>, grouped_gemm_kernel<CfgA, true>},
-    {CfgB::BM, CfgB::BN, CfgB::THREADS, grouped_gemm_kernel<CfgB, false>, grouped_gemm_kernel<CfgB, true>},
-    {CfgC::BM, CfgC::BN, CfgC::THREADS, grouped_gemm_kernel<CfgC, false>, grouped_gemm_kernel<CfgC, true>},
-    {CfgD::BM, CfgD::BN, CfgD::THREADS, grouped_gemm_kernel<CfgD, false>, grouped_gemm_kernel<CfgD, true>},
-    {CfgE::BM, CfgE::BN, CfgE::THREADS, grouped_gemm_kernel<CfgE, false>, grouped_gemm_kernel<CfgE, true>},
-    {CfgF::BM, CfgF::BN, CfgF::THREADS, grouped_gemm_kernel<CfgF, false>, grouped_gemm_kernel<CfgF, true>},
-    {CfgG::BM, CfgG::BN, CfgG::THREADS, grouped_gemm_kernel<CfgG, false>, grouped_gemm_kernel<CfgG, true>},
-    {CfgH::BM, CfgH::BN, CfgH::THREADS, grouped_gemm_kernel<CfgH, false>, grouped_gemm_kernel<CfgH, true>},
-    {CfgI::BM, CfgI::BN, CfgI::THREADS, grouped_gemm_kernel<CfgI, false>, grouped_gemm_kernel<CfgI, true>},
-    {CfgP1::BM, CfgP1::BN, CfgP1::THREADS, grouped_gemm_kernel<CfgP1, false>, grouped_gemm_kernel<CfgP1, true>},
-    {CfgP2::BM, CfgP2::BN, CfgP2::THREADS, grouped_gemm_kernel<CfgP2, false>, grouped_gemm_kernel<CfgP2, true>},
-    {CfgP3::BM, CfgP3::BN, CfgP3::THREADS, grouped_gemm_kernel<CfgP3, false>, grouped_gemm_kernel<CfgP3, true>},
-    {CfgP4::BM, CfgP4::BN, CfgP4::THREADS, grouped_gemm_kernel<CfgP4, false>, grouped_gemm_kernel<CfgP4, true>},
-    {CfgR2::BM, CfgR2::BN, CfgR2::THREADS, grouped_gemm_kernel<CfgR2, false>, grouped_gemm_kernel<CfgR2, true>},
-    {CfgR4::BM, CfgR4::BN, CfgR4::THREADS, grouped_gemm_kernel<CfgR4, false>, grouped_gemm_kernel<CfgR4, true>},
-    {CfgR1::BM, CfgR1::BN, CfgR1::THREADS, grouped_gemm_kernel<CfgR1, false>, grouped_gemm_kernel<CfgR1, true>},
-    {CfgR3::BM, CfgR3::BN, CfgR3::THREADS, grouped_gemm_kernel<CfgR3, false>, grouped_gemm_kernel<CfgR3, true>},
-    {CfgQ0::BM, CfgQ0::BN, CfgQ0::THREADS, grouped_gemm_kernel<CfgQ0, false>, grouped_gemm_kernel<CfgQ0, true>},
-    {CfgQ3::BM, CfgQ3::BN, CfgQ3::THREADS, grouped_gemm_kernel<CfgQ3, false>, grouped_gemm_kernel<CfgQ3, true>},
-    {CfgQ2::BM, CfgQ2::BN, CfgQ2::THREADS, grouped_gemm_kernel<CfgQ2, false>, grouped_gemm_kernel<CfgQ2, true>},
-    {CfgX1::BM, CfgX1::BN, CfgX1::THREADS, grouped_gemm_kernel<CfgX1, false>, grouped_gemm_kernel<CfgX1, true>},
-    {CfgX2::BM, CfgX2::BN, CfgX2::THREADS, grouped_gemm_kernel<CfgX2, false>, grouped_gemm_kernel<CfgX2, true>},
-    {CfgX3::BM, CfgX3::BN, CfgX3::THREADS, grouped_gemm_kernel<CfgX3, false>, grouped_gemm_kernel<CfgX3, true>},
-    {CfgX4::BM, CfgX4::BN, CfgX4::THREADS, grouped_gemm_kernel<CfgX4, false>, grouped_gemm_kernel<CfgX4, true>},
-    {CfgX7::BM, CfgX7::BN, CfgX7::THREADS, grouped_gemm_kernel<CfgX7, false>, grouped_gemm_kernel<CfgX7, true>},
-    {CfgY0::BM, CfgY0::BN, CfgY0::THREADS, grouped_gemm_kernel<CfgY0, false>, grouped_gemm_kernel<CfgY0, true>},
-    {CfgY2::BM, CfgY2::BN, CfgY2::THREADS, grouped_gemm_kernel<CfgY2, false>, grouped_gemm_kernel<CfgY2, true>},
-    {CfgY4::BM, CfgY4::BN, CfgY4::THREADS, grouped_gemm_kernel<CfgY4, false>, grouped_gemm_kernel<CfgY4, true>},
-    {CfgZ0::BM, CfgZ0::BN, CfgZ0::THREADS, grouped_gemm_kernel<CfgZ0, false>, grouped_gemm_kernel<CfgZ0, true>},
-    {CfgW0::BM, CfgW0::BN, CfgW0::THREADS, grouped_gemm_kernel<CfgW0, false>, grouped_gemm_kernel<CfgW0, true>},
-    {CfgW1::BM, CfgW1::BN, CfgW1::THREADS, grouped_gemm_kernel<CfgW1, false>, grouped_gemm_kernel<CfgW1, true>},
-    {CfgW2::BM, CfgW2::BN, CfgW2::THREADS, grouped_gemm_kernel<CfgW2, false>, grouped_gemm_kernel<CfgW2, true>},
-};
+#define CCF_VARIANT(C) {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>}
+const Launch kVariants[] = {CCF_VARIANT(Cfg0), CCF_VARIANT(Cfg1), CCF_VARIANT(Cfg2), CCF_VARIANT(Cfg3),
+                            CCF_VARIANT(Cfg4)};
+#undef CCF_VARIANT
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kMinBM = 128;
 

@@ -107,7 +107,7 @@ __device__ __forceinline__ void lds_dma16(const void *gptr, lds_char *lds_wave_b
 }
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WGS_PER_CU_ = 1,
-          int DMA_EVERY_ = 2, int ABLATE_ = 0, int SCHED_ = 0>
+          int DMA_EVERY_ = 2, int SCHED_ = 0>
 struct GemmCfg {
   // 0: every wavefront interleaves MFMAs, LDS reads and tile loads.
   // 1, 2: ping-pong.  The wavefronts form two groups (1: by wave/4, the two that
@@ -115,10 +115,8 @@ struct GemmCfg {
   // fragment reads + tile loads) and a compute phase (a burst of MFMAs on
   // fragments already in registers), one workgroup barrier per phase, so that
   // a stall while issuing memory instructions never delays an MFMA.
+  // 3: as 0, with the K tiles held in the five-slot ring (RingMainloop).
   static constexpr int SCHED = SCHED_;
-  // Timing experiments only (results are wrong when set): 1 = no tile loads,
-  // 2 = no LDS fragment reads, 4 = no workgroup barriers, 8 = no MFMAs.
-  static constexpr int ABLATE = ABLATE_;
   static constexpr int DMA_EVERY = DMA_EVERY_;         // one tile load behind every n-th MFMA
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
   static constexpr int NW = WM * WN;
@@ -176,9 +174,7 @@ struct GemmMainloop {
                                                    const int (&a_off)[Cfg::KSTEPS],
                                                    const int (&b_off)[Cfg::KSTEPS]) {
     const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage<S>()));
-    if constexpr ((Cfg::ABLATE & 2) != 0) {
-      return;
-    } else if constexpr (I == 0) {
+    if constexpr (I == 0) {
       a[0] = lds_read_b128<0>(base + a_off[KS]);
     } else if constexpr (I <= Cfg::TN) {
       b[I - 1] = lds_read_b128<Cfg::A_BYTES + (I - 1) * 32 * Cfg::CPR * 16>(base + b_off[KS]);
@@ -193,9 +189,7 @@ struct GemmMainloop {
                                                    const half_t *const (&b_src)[Cfg::B_DMA],
                                                    int k_elem, int wave) {
     lds_char *base = stage<S>();
-    if constexpr ((Cfg::ABLATE & 1) != 0) {
-      return;
-    } else if constexpr (I < Cfg::A_DMA) {
+    if constexpr (I < Cfg::A_DMA) {
       lds_dma16(a_src[I] + k_elem, base + (I * Cfg::NW + wave) * 1024);
     } else {
       lds_dma16(b_src[I - Cfg::A_DMA] + k_elem,
@@ -229,21 +223,6 @@ struct GemmMainloop {
       static_for<0, PER_TILE>([&](auto I) { issue_one<NEXT, I.value>(a_src, b_src, k_pre, wave); });
       __builtin_amdgcn_sched_barrier(0);
     }
-    if constexpr ((Cfg::ABLATE & 2) != 0) {
-      // stand-in operands with realistic bit toggling (timing experiments only)
-      unsigned x = threadIdx.x * 2654435761u + 12345u;
-      auto rnd = [&](float scale) {
-        half8 v;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
-          v[j] = static_cast<half_t>((static_cast<int>(x & 0xffff) - 32768) / 32768.0f * scale);
-        }
-        return v;
-      };
-      static_for<0, Cfg::TM>([&](auto I) { a[0][I.value] = rnd(1.0f); a[1][I.value] = rnd(1.0f); });
-      static_for<0, Cfg::TN>([&](auto I) { b[0][I.value] = rnd(0.03f); b[1][I.value] = rnd(0.03f); });
-    }
     static_for<0, FRAGS>([&](auto I) { read_frag<S, 0, I.value>(a[0], b[0], a_off, b_off); });
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, Cfg::KSTEPS>([&](auto KS) {
@@ -255,10 +234,8 @@ struct GemmMainloop {
         constexpr int tm = i / Cfg::TN, tn = i % Cfg::TN;
         constexpr int need = a_seq(tm) > b_seq(tn) ? a_seq(tm) : b_seq(tn);
         constexpr int next_issued = more ? (i < FRAGS ? i : FRAGS) : 0;
-        if constexpr ((Cfg::ABLATE & 2) == 0)
-          wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
-        if constexpr ((Cfg::ABLATE & 8) == 0)
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
+        wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
         if constexpr (more && i < FRAGS) read_frag<S, ks + 1, i>(a[cur ^ 1], b[cur ^ 1], a_off, b_off);
         constexpr int m = ks * PER_STEP + i;                 // MFMA index within the tile
         if constexpr (PREFETCH && Cfg::DMA_EVERY > 0) {
@@ -296,7 +273,7 @@ struct GemmMainloop {
       // tile kt+1 must have landed before anyone reads it: leave at most the
       // loads of the STAGES-2 younger tiles in flight.
       wait_vmcnt<PER_TILE *(Cfg::STAGES - 2)>();
-      if constexpr ((Cfg::ABLATE & 4) == 0) block_barrier();
+      block_barrier();
     }
   };
 
@@ -493,14 +470,17 @@ struct RingMainloop {
     }
   }
 
-  template <int U>
+  // FULL: every 32-row block of this wavefront holds real rows.  Otherwise only
+  // the first live_m blocks do (the tail tile of an expert), and the MFMAs of
+  // the padded blocks are skipped: they would only burn power.
+  template <int U, bool FULL>
   struct Step {
     static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
                                                const half_t *const (&a_src)[Cfg::A_DMA],
                                                const half_t *const (&b_src)[Cfg::B_DMA],
                                                const int (&a_off)[Cfg::KSTEPS],
                                                const int (&b_off)[Cfg::KSTEPS], int kt, int KT,
-                                               int wave) {
+                                               int wave, int live_m) {
       constexpr int SA = (2 * U) % NSLOT, SB = (2 * U + 1) % NSLOT;       // tile kt
       constexpr int WB = (2 * U + 3) % NSLOT, WA = (2 * U + 4) % NSLOT;   // B(kt+1), A(kt+2)
       constexpr int PER_STEP = Cfg::TM * Cfg::TN;
@@ -522,7 +502,8 @@ struct RingMainloop {
           constexpr int need = Base::a_seq(tm) > Base::b_seq(tn) ? Base::a_seq(tm) : Base::b_seq(tn);
           constexpr int next_issued = more ? (i < FRAGS ? i : FRAGS) : 0;
           wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
+          if (FULL || tm < live_m)
+            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
           if constexpr (more && i < FRAGS) read_frag<SA, SB, ks + 1, i>(a[cur ^ 1], b[cur ^ 1], a_off, b_off);
           constexpr int m = ks * PER_STEP + i;
           if constexpr (m % Cfg::DMA_EVERY == 0 && m / Cfg::DMA_EVERY < LOADS) {
@@ -544,13 +525,18 @@ struct RingMainloop {
     }
   };
 
+  // rows: real rows of this M tile (1..BM).
   static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
                                              const half_t *const (&a_src)[Cfg::A_DMA],
-                                             const half_t *const (&b_src)[Cfg::B_DMA], int K) {
+                                             const half_t *const (&b_src)[Cfg::B_DMA], int K,
+                                             int rows) {
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
     const int KT = K / Cfg::BK;
+    int live_m = (rows - wm * Cfg::WTM + 31) / 32;       // 32-row blocks of this wavefront with real rows
+    live_m = live_m < 0 ? 0 : (live_m > Cfg::TM ? Cfg::TM : live_m);
+    live_m = __builtin_amdgcn_readfirstlane(live_m);
     int a_off[Cfg::KSTEPS], b_off[Cfg::KSTEPS];
     {
       const int ra = wm * Cfg::WTM + (lane & 31);
@@ -568,10 +554,18 @@ struct RingMainloop {
     issue_all<2>(a_src, (KT > 1 ? 1 : 0) * Cfg::BK, wave);
     wait_vmcnt<Cfg::A_DMA>();
     block_barrier();
-    for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
-      static_for<0, NSLOT>([&](auto U) {
-        Step<U.value>::run(acc, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave);
-      });
+    if (live_m == Cfg::TM) {
+      for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
+        static_for<0, NSLOT>([&](auto U) {
+          Step<U.value, true>::run(acc, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave, live_m);
+        });
+      }
+    } else {
+      for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
+        static_for<0, NSLOT>([&](auto U) {
+          Step<U.value, false>::run(acc, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave, live_m);
+        });
+      }
     }
     wait_vmcnt<0>();
   }

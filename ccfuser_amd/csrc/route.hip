@@ -72,18 +72,37 @@ hist_kernel(const int64_t *__restrict__ idx, int n, int E, int nbits,
 // One workgroup.  chunk_cnt becomes, in place, the exclusive running sum over
 // chunks (the rank base of each chunk).  If cum_inout is given the segment
 // starts come from it (cum[e] - total[e]) and are written back there;
-// otherwise they are the exclusive scan of the kept counts.
+// otherwise they are the exclusive scan of the kept counts.  The table is
+// pulled into LDS with parallel loads first when it fits, so that the per
+// expert running sum is not a chain of dependent global loads.
+constexpr int kScanLdsEntries = 8192;
+
 __global__ void __launch_bounds__(1024)
 scan_kernel(int32_t *__restrict__ chunk_cnt, int nchunk, int E, int capacity,
             int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
             int32_t *__restrict__ cum_inout) {
   __shared__ int s_kept[kMaxExpert];
+  __shared__ int s_tab[kScanLdsEntries];
+  const int entries = nchunk * E;
+  const bool in_lds = entries <= kScanLdsEntries;
+  if (in_lds) {
+    for (int i = threadIdx.x; i < entries; i += blockDim.x) s_tab[i] = chunk_cnt[i];
+    __syncthreads();
+  }
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     int run = 0;
-    for (int c = 0; c < nchunk; ++c) {
-      int v = chunk_cnt[static_cast<size_t>(c) * E + e];
-      chunk_cnt[static_cast<size_t>(c) * E + e] = run;
-      run += v;
+    if (in_lds) {
+      for (int c = 0; c < nchunk; ++c) {
+        int v = s_tab[c * E + e];
+        s_tab[c * E + e] = run;
+        run += v;
+      }
+    } else {
+      for (int c = 0; c < nchunk; ++c) {
+        int v = chunk_cnt[static_cast<size_t>(c) * E + e];
+        chunk_cnt[static_cast<size_t>(c) * E + e] = run;
+        run += v;
+      }
     }
     int kept = (capacity >= 0 && run > capacity) ? capacity : run;
     s_kept[e] = kept;
@@ -95,6 +114,8 @@ scan_kernel(int32_t *__restrict__ chunk_cnt, int nchunk, int E, int capacity,
     }
   }
   __syncthreads();
+  if (in_lds)
+    for (int i = threadIdx.x; i < entries; i += blockDim.x) chunk_cnt[i] = s_tab[i];
   if (!cum_inout && threadIdx.x < 64) {
     // exclusive scan over experts by one wavefront, 64 at a time
     int carry = 0;
