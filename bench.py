@@ -89,6 +89,9 @@ def main():
     ap.add_argument("--workload", default="c3_mixtral")
     ap.add_argument("--gemm-variant", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies (a known HBM traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU's share only: this build has no collectives or sharding "
@@ -165,6 +168,13 @@ def main():
         for row in events:
             for e in row:
                 ev.destroy(e)
+
+    if a.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     ms = wall / K * 1e3
     flops = wl.flops(routed)

@@ -22,23 +22,31 @@ namespace ccf {
 namespace {
 
 // ---- tile plan ---------------------------------------------------------------
-// plan[0] = number of M tiles, then three arrays of max_tiles entries.
+// plan[0] = number of M tiles, then three arrays of max_tiles entries (expert,
+// first row, rows of each M tile), then the launch order: for every logical
+// tile id its (M tile, N tile) pair.
 struct PlanView {
   const int32_t *n_tiles;
   const int32_t *expert;
   const int32_t *row0;
   const int32_t *rows;
+  const int32_t *order;   // [max_tiles * n_tiles_n][2]
 };
 
-__host__ __device__ inline size_t plan_ints(int max_tiles) { return 64 + 3 * static_cast<size_t>(max_tiles); }
-
-__device__ inline PlanView plan_view(const int32_t *plan, int max_tiles) {
-  return PlanView{plan, plan + 64, plan + 64 + max_tiles, plan + 64 + 2 * max_tiles};
+__host__ __device__ inline size_t plan_ints(int max_tiles, int n_tiles_n) {
+  return 64 + 3 * static_cast<size_t>(max_tiles) + 2 * static_cast<size_t>(max_tiles) * n_tiles_n;
 }
 
-__global__ void __launch_bounds__(256)
+__device__ inline PlanView plan_view(const int32_t *plan, int max_tiles) {
+  return PlanView{plan, plan + 64, plan + 64 + max_tiles, plan + 64 + 2 * max_tiles,
+                  plan + 64 + 3 * static_cast<size_t>(max_tiles)};
+}
+
+constexpr int kOrderGroupM = 8;
+
+__global__ void __launch_bounds__(1024)
 plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, int max_rows,
-            int32_t *__restrict__ plan) {
+            int n_tiles_n, int32_t *__restrict__ plan) {
   __shared__ int s_off[1025];
   __shared__ int s_base[1025];
   for (int e = threadIdx.x; e <= E; e += blockDim.x) {
@@ -71,19 +79,35 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
   }
   __syncthreads();
   int32_t *expert = plan + 64, *row0 = expert + max_tiles, *rows = row0 + max_tiles;
+  int32_t *order = rows + max_tiles;
   // one wavefront per expert, one lane per tile
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
   for (int e = wave; e < E; e += nwave) {
     const int lo = s_off[e];
     int cnt = s_off[e + 1] - lo;
     cnt = cnt > 0 ? cnt : 0;
-    const int nt = s_base[e + 1] - s_base[e];
+    int nt = s_base[e + 1] - s_base[e];
+    if (s_base[e] + nt > max_tiles) nt = max_tiles - s_base[e];
     for (int i = lane; i < nt; i += 64) {
       const int t = s_base[e] + i;
-      if (t >= max_tiles) break;
       expert[t] = e;
       row0[t] = lo + i * BM;
       rows[t] = (cnt - i * BM) < BM ? (cnt - i * BM) : BM;
+    }
+    // Launch order inside an expert: runs of up to kOrderGroupM M tiles, and
+    // inside a run the M tile varies fastest.  The ~32 workgroups an XCD runs at
+    // a time (consecutive logical ids) then form a patch of a M tiles x 32/a N
+    // tiles of ONE expert: a weight tile is pulled from HBM once for a M tiles,
+    // a token tile once for 32/a N tiles, and HBM traffic per patch, which goes
+    // as 1/a + a/32, is near its minimum for a = 4..8.
+    const long long first = static_cast<long long>(s_base[e]) * n_tiles_n;
+    for (int l = lane; l < nt * n_tiles_n; l += 64) {
+      const int run = l / (kOrderGroupM * n_tiles_n);            // which run of M tiles
+      const int run_first = run * kOrderGroupM;
+      const int run_size = (nt - run_first) < kOrderGroupM ? (nt - run_first) : kOrderGroupM;
+      const int in_run = l - run * kOrderGroupM * n_tiles_n;
+      order[2 * (first + l)] = s_base[e] + run_first + in_run % run_size;
+      order[2 * (first + l) + 1] = in_run / run_size;
     }
   }
 }
@@ -102,8 +126,6 @@ struct GroupedArgs {
   int n_tiles_n;
   int N, K;
 };
-
-constexpr int kGroupM = 4;
 
 // erf-form GELU, 0.5*v*(1+erf(v/sqrt2)), with erf from Abramowitz-Stegun 7.1.26
 // (|error| <= 1.5e-7, far below one fp16 ulp of the result):
@@ -139,13 +161,8 @@ grouped_gemm_kernel(GroupedArgs p) {
   const int slot = blockIdx.x >> 3;
   const int logical = (blockIdx.x & 7) * per_xcd + slot;
   if (slot >= per_xcd || logical >= total) return;
-  // Runs of kGroupM M tiles x all N tiles: neighbours share A rows and B rows.
-  const int group_sz = kGroupM * p.n_tiles_n;
-  const int first_m = (logical / group_sz) * kGroupM;
-  const int gm = (n_m - first_m) < kGroupM ? (n_m - first_m) : kGroupM;
-  const int in_group = logical % group_sz;
-  const int tile_m = first_m + in_group % gm;
-  const int tile_n = in_group / gm;
+  const int tile_m = pv.order[2 * static_cast<size_t>(logical)];
+  const int tile_n = pv.order[2 * static_cast<size_t>(logical) + 1];
 
   const int e = pv.expert[tile_m];
   const int row0 = pv.row0[tile_m];
@@ -252,8 +269,11 @@ constexpr int kMinBM = 128;
 
 int max_tiles_for(int max_rows, int E, int bm) { return (max_rows + bm - 1) / bm + E; }
 
-size_t plan_bytes(int max_rows, int E) {
-  return round_up(sizeof(int32_t) * plan_ints(max_tiles_for(max_rows, E, kMinBM)), 256);
+constexpr int kMinBN = 128;
+
+size_t plan_bytes(int max_rows, int E, int n_max) {
+  return round_up(sizeof(int32_t) * plan_ints(max_tiles_for(max_rows, E, kMinBM),
+                                              (n_max + kMinBN - 1) / kMinBN), 256);
 }
 
 int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets, int max_rows, int E,
@@ -270,8 +290,9 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   if (max_rows == 0) return CCF_OK;
   const Launch &v = kVariants[g_variant];
   const int max_tiles = max_tiles_for(max_rows, E, v.bm);
-  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(256), 0, stream, offsets, E, v.bm, max_tiles,
-                     max_rows, plan);
+  const int n_tiles_n = (N + v.bn - 1) / v.bn;
+  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, offsets, E, v.bm, max_tiles,
+                     max_rows, n_tiles_n, plan);
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
   p.A = A;
@@ -283,12 +304,11 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.row_scale = row_scale;
   p.plan = plan;
   p.max_tiles = max_tiles;
-  p.n_tiles_n = (N + v.bn - 1) / v.bn;
+  p.n_tiles_n = n_tiles_n;
   p.N = N;
   p.K = K;
-  // whole groups of kGroupM M tiles, rounded to a multiple of 8 workgroups
-  const long long groups = (max_tiles + kGroupM - 1) / kGroupM;
-  long long wgs = groups * kGroupM * p.n_tiles_n;
+  // worst-case tile count, rounded to a multiple of 8 workgroups (one share per XCD)
+  long long wgs = static_cast<long long>(max_tiles) * p.n_tiles_n;
   wgs = (wgs + 7) / 8 * 8;
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   hipLaunchKernelGGL(gelu ? v.gelu : v.plain, dim3(static_cast<unsigned>(wgs)), dim3(v.threads), 0,
@@ -313,7 +333,7 @@ extern "C" int ccf_set_option(const char *name, int value) {
 
 extern "C" size_t ccf_ffn_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn) {
   if (max_rows < 0 || num_expert <= 0 || d_model <= 0 || d_ffn <= 0) return 0;
-  return ccf::plan_bytes(max_rows, num_expert);
+  return ccf::plan_bytes(max_rows, num_expert, d_model > d_ffn ? d_model : d_ffn);
 }
 
 extern "C" int ccf_ffn1_forward(const void *x, const int32_t *src_row, const int32_t *dst_row,
@@ -321,9 +341,9 @@ extern "C" int ccf_ffn1_forward(const void *x, const int32_t *src_row, const int
                                 int d_ffn, const void *w1, const void *b1, int apply_gelu, void *h,
                                 void *workspace, size_t workspace_bytes, ccf_stream_t stream) {
   using namespace ccf;
-  CCF_REQUIRE(workspace && workspace_bytes >= plan_bytes(max_rows, num_expert), CCF_ERR_WORKSPACE,
-              "ffn1: workspace of %zu bytes needed, %zu given", plan_bytes(max_rows, num_expert),
-              workspace_bytes);
+  const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
+  CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
+              "ffn1: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   return grouped_gemm(static_cast<const half_t *>(x), src_row, offsets, max_rows, num_expert, d_ffn,
                       d_model, static_cast<const half_t *>(w1), static_cast<const half_t *>(b1),
                       apply_gelu != 0, static_cast<half_t *>(h), dst_row, nullptr,
@@ -336,9 +356,9 @@ extern "C" int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int
                                 void *y, void *workspace, size_t workspace_bytes,
                                 ccf_stream_t stream) {
   using namespace ccf;
-  CCF_REQUIRE(workspace && workspace_bytes >= plan_bytes(max_rows, num_expert), CCF_ERR_WORKSPACE,
-              "ffn2: workspace of %zu bytes needed, %zu given", plan_bytes(max_rows, num_expert),
-              workspace_bytes);
+  const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
+  CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
+              "ffn2: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   return grouped_gemm(static_cast<const half_t *>(h), src_row, offsets, max_rows, num_expert, d_model,
                       d_ffn, static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), false,
                       static_cast<half_t *>(y), dst_row, static_cast<const half_t *>(row_scale),
