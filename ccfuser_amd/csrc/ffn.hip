@@ -22,24 +22,15 @@ namespace ccf {
 namespace {
 
 // ---- tile plan ---------------------------------------------------------------
-// plan[0] = number of M tiles, then three arrays of max_tiles entries (expert,
-// first row, rows of each M tile), then the launch order: for every logical
-// tile id its (M tile, N tile) pair.
-struct PlanView {
-  const int32_t *n_tiles;
-  const int32_t *expert;
-  const int32_t *row0;
-  const int32_t *rows;
-  const int32_t *order;   // [max_tiles * n_tiles_n][2]
-};
+// The plan is one 16-byte entry per launched workgroup, indexed by the hardware
+// workgroup id: {expert, first sorted row, rows in the M tile, N tile}, expert
+// = -1 for workgroups with nothing to do.  A workgroup learns its whole
+// assignment from a single load.
+__host__ __device__ inline size_t plan_ints(long long wgs) { return 4 * static_cast<size_t>(wgs); }
 
-__host__ __device__ inline size_t plan_ints(int max_tiles, int n_tiles_n) {
-  return 64 + 3 * static_cast<size_t>(max_tiles) + 2 * static_cast<size_t>(max_tiles) * n_tiles_n;
-}
-
-__device__ inline PlanView plan_view(const int32_t *plan, int max_tiles) {
-  return PlanView{plan, plan + 64, plan + 64 + max_tiles, plan + 64 + 2 * max_tiles,
-                  plan + 64 + 3 * static_cast<size_t>(max_tiles)};
+__host__ __device__ inline long long launched_wgs(int max_tiles, int n_tiles_n) {
+  long long w = static_cast<long long>(max_tiles) * n_tiles_n;
+  return (w + 7) / 8 * 8;                         // one equal share per XCD
 }
 
 constexpr int kOrderGroupM = 8;
@@ -72,15 +63,23 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
       if (e < E) s_base[e] = carry + inc - nt;
       carry += __shfl(inc, 63, 64);
     }
-    if (lane == 0) {
-      s_base[E] = carry;
-      plan[0] = carry < max_tiles ? carry : max_tiles;
-    }
+    if (lane == 0) s_base[E] = carry;
   }
   __syncthreads();
-  int32_t *expert = plan + 64, *row0 = expert + max_tiles, *rows = row0 + max_tiles;
-  int32_t *order = rows + max_tiles;
-  // one wavefront per expert, one lane per tile
+  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn.  Logical
+  // tile ids are cut into eight equal contiguous runs, one per XCD (one L2), so
+  // hardware id b works on logical id (b % 8) * per_xcd + b / 8.
+  int n_m = s_base[E] < max_tiles ? s_base[E] : max_tiles;
+  const long long total = static_cast<long long>(n_m) * n_tiles_n;
+  const long long per_xcd = (total + 7) / 8;
+  const long long wgs = launched_wgs(max_tiles, n_tiles_n);
+  int4v *entry = reinterpret_cast<int4v *>(plan);
+  for (long long b = threadIdx.x; b < wgs; b += blockDim.x) {
+    const long long slot = b >> 3;
+    const long long logical = (b & 7) * per_xcd + slot;
+    if (slot >= per_xcd || logical >= total) entry[b] = int4v{-1, 0, 0, 0};
+  }
+  // one wavefront per expert
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
   for (int e = wave; e < E; e += nwave) {
     const int lo = s_off[e];
@@ -88,12 +87,6 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
     cnt = cnt > 0 ? cnt : 0;
     int nt = s_base[e + 1] - s_base[e];
     if (s_base[e] + nt > max_tiles) nt = max_tiles - s_base[e];
-    for (int i = lane; i < nt; i += 64) {
-      const int t = s_base[e] + i;
-      expert[t] = e;
-      row0[t] = lo + i * BM;
-      rows[t] = (cnt - i * BM) < BM ? (cnt - i * BM) : BM;
-    }
     // Launch order inside an expert: runs of up to kOrderGroupM M tiles, and
     // inside a run the M tile varies fastest.  The ~32 workgroups an XCD runs at
     // a time (consecutive logical ids) then form a patch of a M tiles x 32/a N
@@ -106,8 +99,12 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
       const int run_first = run * kOrderGroupM;
       const int run_size = (nt - run_first) < kOrderGroupM ? (nt - run_first) : kOrderGroupM;
       const int in_run = l - run * kOrderGroupM * n_tiles_n;
-      order[2 * (first + l)] = s_base[e] + run_first + in_run % run_size;
-      order[2 * (first + l) + 1] = in_run / run_size;
+      const int i = run_first + in_run % run_size;               // M tile within the expert
+      const int tn = in_run / run_size;
+      const long long logical = first + l;
+      const long long b = (logical % per_xcd) * 8 + logical / per_xcd;   // hardware id
+      const int rows = (cnt - i * BM) < BM ? (cnt - i * BM) : BM;
+      entry[b] = int4v{e, lo + i * BM, rows, tn};
     }
   }
 }
@@ -122,8 +119,6 @@ struct GroupedArgs {
   const int32_t *c_rows;    // row of C for sorted row j, or NULL (identity)
   const half_t *row_scale;  // [rows] or NULL
   const int32_t *plan;
-  int max_tiles;
-  int n_tiles_n;
   int N, K;
 };
 
@@ -149,24 +144,12 @@ template <class Cfg, bool kGelu>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_kernel(GroupedArgs p) {
   using ML = GemmMainloop<Cfg>;
-  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn.  Undo that
-  // so one XCD (one L2) works on a contiguous run of logical tile ids, and cut
-  // the REAL tiles (known only on the device) into eight equal runs: the grid
-  // is sized for the worst case, and surplus workgroups must not pile up on
-  // the last XCDs.
-  const PlanView pv = plan_view(p.plan, p.max_tiles);
-  const int n_m = pv.n_tiles[0];
-  const int total = n_m * p.n_tiles_n;
-  const int per_xcd = (total + 7) >> 3;
-  const int slot = blockIdx.x >> 3;
-  const int logical = (blockIdx.x & 7) * per_xcd + slot;
-  if (slot >= per_xcd || logical >= total) return;
-  const int tile_m = pv.order[2 * static_cast<size_t>(logical)];
-  const int tile_n = pv.order[2 * static_cast<size_t>(logical) + 1];
-
-  const int e = pv.expert[tile_m];
-  const int row0 = pv.row0[tile_m];
-  const int rows = pv.rows[tile_m];
+  const int4v ent = reinterpret_cast<const int4v *>(p.plan)[blockIdx.x];
+  const int e = ent[0];
+  if (e < 0) return;                                 // surplus workgroup of the worst-case grid
+  const int row0 = ent[1];
+  const int rows = ent[2];
+  const int tile_n = ent[3];
   const int n0 = tile_n * Cfg::BN;
   const half_t *Be = p.B + static_cast<size_t>(e) * p.N * p.K;
 
@@ -272,8 +255,8 @@ int max_tiles_for(int max_rows, int E, int bm) { return (max_rows + bm - 1) / bm
 constexpr int kMinBN = 128;
 
 size_t plan_bytes(int max_rows, int E, int n_max) {
-  return round_up(sizeof(int32_t) * plan_ints(max_tiles_for(max_rows, E, kMinBM),
-                                              (n_max + kMinBN - 1) / kMinBN), 256);
+  return round_up(sizeof(int32_t) * plan_ints(launched_wgs(max_tiles_for(max_rows, E, kMinBM),
+                                                            (n_max + kMinBN - 1) / kMinBN)), 256);
 }
 
 int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets, int max_rows, int E,
@@ -303,13 +286,9 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.c_rows = c_rows;
   p.row_scale = row_scale;
   p.plan = plan;
-  p.max_tiles = max_tiles;
-  p.n_tiles_n = n_tiles_n;
   p.N = N;
   p.K = K;
-  // worst-case tile count, rounded to a multiple of 8 workgroups (one share per XCD)
-  long long wgs = static_cast<long long>(max_tiles) * p.n_tiles_n;
-  wgs = (wgs + 7) / 8 * 8;
+  const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   hipLaunchKernelGGL(gelu ? v.gelu : v.plain, dim3(static_cast<unsigned>(wgs)), dim3(v.threads), 0,
                      stream, p);
