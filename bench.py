@@ -24,6 +24,25 @@ sys.path.insert(0, ROOT)
 PEAK_FP16_TFLOPS = 2500.0          # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 
+# Bytes moved between L2 and the memory fabric per launch of the grouped GEMM, from two
+# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each
+# scaled by what the counter reads for a plain 256 MiB device copy in the same run (FETCH_SIZE
+# reads half the copied bytes: factor 2.0; WRITE_SIZE factor 1.0).  The summaries are in
+# profiles/grouped_gemm_<workload>_hbm_traffic.txt.  Counters cannot be read from inside a
+# normal run, so a workload without a profile reports null.
+MEASURED_TRAFFIC_KIB = {
+    ("c3_mixtral", "ffn1"): {"FETCH_SIZE": 1456019.8, "WRITE_SIZE": 231244.9},
+    ("c3_mixtral", "ffn2"): {"FETCH_SIZE": 1364172.0, "WRITE_SIZE": 65936.3},
+}
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+
+
+def measured_traffic(workload, stage):
+    m = MEASURED_TRAFFIC_KIB.get((workload, stage))
+    if m is None:
+        return None
+    return (m["FETCH_SIZE"] * FETCH_SCALE + m["WRITE_SIZE"] * WRITE_SCALE) * 1024.0
+
 
 class HipEvents:
     """hipEvent_t handles through the HIP runtime (torch's events hide the handle)."""
@@ -194,7 +213,8 @@ def main():
         ach = (flops / 2) / (stage_ms[dom] * 1e-3) / 1e12
         line["roofline"] = {"kernel": f"grouped_gemm_kernel ({dom})", "bound": "mfma",
                             "achieved": ach, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                            "frac": ach / PEAK_FP16_TFLOPS, "traffic": None,
+                            "frac": ach / PEAK_FP16_TFLOPS,
+                            "traffic": measured_traffic(wl.name, dom), "traffic_unit": "bytes/launch",
                             "flop_per_launch": flops / 2, "avg_launch_ms": stage_ms[dom]}
         hbm_bytes = T * d * 2 + E * d * 2 + T * k * 10
         line["gate_gbs"] = hbm_bytes / (stage_ms["gate"] * 1e-3) / 1e9
