@@ -30,81 +30,100 @@ __host__ __device__ inline size_t plan_ints(long long wgs) { return 4 * static_c
 
 __host__ __device__ inline long long launched_wgs(int max_tiles, int n_tiles_n) {
   long long w = static_cast<long long>(max_tiles) * n_tiles_n;
-  return (w + 7) / 8 * 8;                         // one equal share per XCD
+  return ((w + 7) / 8 + 2) * 8;                   // per XCD: a share of each of the two tile classes, rounded up
 }
 
 constexpr int kOrderGroupM = 8;
 
+// Tiles come in two classes.  A "long" M tile holds more than BM/2 rows and
+// takes a full tile's time; a "short" one (an expert's last tile with at most
+// BM/2 rows) skips most of its MFMAs and ends early.  Workgroups that share an
+// XCD share weight and token tiles through its L2 only while they walk K in
+// step, and a workgroup that ends early puts every later one on its CU out of
+// step, so all long tiles are launched first and the short ones after them,
+// where they also even out the end of the launch.
 __global__ void __launch_bounds__(1024)
 plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, int max_rows,
             int n_tiles_n, int32_t *__restrict__ plan) {
   __shared__ int s_off[1025];
-  __shared__ int s_base[1025];
+  __shared__ int s_long[1025];     // exclusive scan of long M tiles per expert
+  __shared__ int s_short[1025];    // exclusive scan of short M tiles per expert (0 or 1 each)
   for (int e = threadIdx.x; e <= E; e += blockDim.x) {
     int v = offsets[e];
     s_off[e] = v < max_rows ? v : max_rows;          // never plan past the caller's bound
   }
   __syncthreads();
   if (threadIdx.x < 64) {
-    // exclusive scan of the per-expert tile counts by one wavefront
     const int lane = threadIdx.x;
-    int carry = 0;
+    int carry_l = 0, carry_s = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
       int cnt = e < E ? s_off[e + 1] - s_off[e] : 0;
       cnt = cnt > 0 ? cnt : 0;
       const int nt = (cnt + BM - 1) / BM;
-      int inc = nt;
+      const int ns = (nt > 0 && cnt - (nt - 1) * BM <= BM / 2) ? 1 : 0;
+      const int nl = nt - ns;
+      int inc_l = nl, inc_s = ns;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
-        int o = __shfl_up(inc, off, 64);
-        if (lane >= off) inc += o;
+        int ol = __shfl_up(inc_l, off, 64);
+        int os = __shfl_up(inc_s, off, 64);
+        if (lane >= off) { inc_l += ol; inc_s += os; }
       }
-      if (e < E) s_base[e] = carry + inc - nt;
-      carry += __shfl(inc, 63, 64);
+      if (e < E) { s_long[e] = carry_l + inc_l - nl; s_short[e] = carry_s + inc_s - ns; }
+      carry_l += __shfl(inc_l, 63, 64);
+      carry_s += __shfl(inc_s, 63, 64);
     }
-    if (lane == 0) s_base[E] = carry;
+    if (lane == 0) { s_long[E] = carry_l; s_short[E] = carry_s; }
   }
-  __syncthreads();
-  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn.  Logical
-  // tile ids are cut into eight equal contiguous runs, one per XCD (one L2), so
-  // hardware id b works on logical id (b % 8) * per_xcd + b / 8.
-  int n_m = s_base[E] < max_tiles ? s_base[E] : max_tiles;
-  const long long total = static_cast<long long>(n_m) * n_tiles_n;
-  const long long per_xcd = (total + 7) / 8;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   int4v *entry = reinterpret_cast<int4v *>(plan);
-  for (long long b = threadIdx.x; b < wgs; b += blockDim.x) {
-    const long long slot = b >> 3;
-    const long long logical = (b & 7) * per_xcd + slot;
-    if (slot >= per_xcd || logical >= total) entry[b] = int4v{-1, 0, 0, 0};
-  }
+  for (long long b = threadIdx.x; b < wgs; b += blockDim.x) entry[b] = int4v{-1, 0, 0, 0};
+  __syncthreads();
+  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn, so XCD x
+  // runs ids x, x+8, ... in order.  Each class is cut into eight equal
+  // contiguous runs of logical tile ids, one per XCD (one L2): slot j of XCD x
+  // is long tile x*per_long + j for j < per_long, else short tile
+  // x*per_short + (j - per_long).
+  const long long total_long = static_cast<long long>(s_long[E]) * n_tiles_n;
+  const long long total_short = static_cast<long long>(s_short[E]) * n_tiles_n;
+  const long long per_long = (total_long + 7) / 8;
+  const long long per_short = (total_short + 7) / 8;
   // one wavefront per expert
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
   for (int e = wave; e < E; e += nwave) {
     const int lo = s_off[e];
     int cnt = s_off[e + 1] - lo;
     cnt = cnt > 0 ? cnt : 0;
-    int nt = s_base[e + 1] - s_base[e];
-    if (s_base[e] + nt > max_tiles) nt = max_tiles - s_base[e];
-    // Launch order inside an expert: runs of up to kOrderGroupM M tiles, and
-    // inside a run the M tile varies fastest.  The ~32 workgroups an XCD runs at
-    // a time (consecutive logical ids) then form a patch of a M tiles x 32/a N
-    // tiles of ONE expert: a weight tile is pulled from HBM once for a M tiles,
-    // a token tile once for 32/a N tiles, and HBM traffic per patch, which goes
-    // as 1/a + a/32, is near its minimum for a = 4..8.
-    const long long first = static_cast<long long>(s_base[e]) * n_tiles_n;
-    for (int l = lane; l < nt * n_tiles_n; l += 64) {
+    const int nl = s_long[e + 1] - s_long[e];
+    const int ns = s_short[e + 1] - s_short[e];
+    // Launch order of an expert's long tiles: runs of up to kOrderGroupM M
+    // tiles, and inside a run the M tile varies fastest.  The ~32 workgroups an
+    // XCD runs at a time (consecutive logical ids) then form a patch of a M
+    // tiles x 32/a N tiles of ONE expert: a weight tile is pulled from HBM once
+    // for a M tiles, a token tile once for 32/a N tiles, and HBM traffic per
+    // patch, which goes as 1/a + a/32, is near its minimum for a = 4..8.
+    const long long first = static_cast<long long>(s_long[e]) * n_tiles_n;
+    for (int l = lane; l < nl * n_tiles_n; l += 64) {
       const int run = l / (kOrderGroupM * n_tiles_n);            // which run of M tiles
       const int run_first = run * kOrderGroupM;
-      const int run_size = (nt - run_first) < kOrderGroupM ? (nt - run_first) : kOrderGroupM;
+      const int run_size = (nl - run_first) < kOrderGroupM ? (nl - run_first) : kOrderGroupM;
       const int in_run = l - run * kOrderGroupM * n_tiles_n;
       const int i = run_first + in_run % run_size;               // M tile within the expert
       const int tn = in_run / run_size;
       const long long logical = first + l;
-      const long long b = (logical % per_xcd) * 8 + logical / per_xcd;   // hardware id
+      const long long b = (logical % per_long) * 8 + logical / per_long;   // hardware id
       const int rows = (cnt - i * BM) < BM ? (cnt - i * BM) : BM;
-      entry[b] = int4v{e, lo + i * BM, rows, tn};
+      if (b < wgs) entry[b] = int4v{e, lo + i * BM, rows, tn};
+    }
+    if (ns) {
+      const int i = nl;                                          // the expert's last M tile
+      const long long first_s = static_cast<long long>(s_short[e]) * n_tiles_n;
+      for (int tn = lane; tn < n_tiles_n; tn += 64) {
+        const long long logical = first_s + tn;
+        const long long b = (per_long + logical % per_short) * 8 + logical / per_short;
+        if (b < wgs) entry[b] = int4v{e, lo + i * BM, cnt - i * BM, tn};
+      }
     }
   }
 }
@@ -169,6 +188,49 @@ grouped_gemm_kernel(GroupedArgs p) {
     b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r) * 8;
   }
 
+  const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
+  if constexpr (Cfg::SCHED == 4 || Cfg::SCHED == 5) {
+    using R = std::conditional_t<Cfg::SCHED == 4, Ring16Mainloop<Cfg>, Roll16Mainloop<Cfg>>;
+    float4v acc[R::TM][R::TN];
+#pragma unroll
+    for (int tm = 0; tm < R::TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < R::TN; ++tn) acc[tm][tn] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+    R::run(acc, a_src, b_src, p.K, rows);
+    // Epilogue: bias (+ GELU) (+ row scale), fp16, 8-byte stores through the row index.
+    float bias_v[R::TN][4];
+    int col[R::TN];
+#pragma unroll
+    for (int tn = 0; tn < R::TN; ++tn) {
+      col[tn] = n0 + acc16_col4<Cfg>(tn);
+      half4 bv = {0, 0, 0, 0};
+      if (col[tn] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn]);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) bias_v[tn][c] = static_cast<float>(bv[c]);
+    }
+#pragma unroll
+    for (int tm = 0; tm < R::TM; ++tm) {
+      const int lr = acc16_row<Cfg>(tm);
+      if (lr < rows) {
+        const int j = row0 + lr;
+        const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
+        const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
+        half_t *dst = p.C + crow * p.N;
+#pragma unroll
+        for (int tn = 0; tn < R::TN; ++tn) {
+          half4 o;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            float v = acc[tm][tn][c] + bias_v[tn][c];
+            if (kGelu) v = gelu_erf(v);
+            o[c] = static_cast<half_t>(v * sc);
+          }
+          if (col[tn] < p.N) *reinterpret_cast<half4 *>(dst + col[tn]) = o;
+        }
+      }
+    }
+    return;
+  } else {
   typename ML::acc_t acc[Cfg::TM][Cfg::TN];
 #pragma unroll
   for (int tm = 0; tm < Cfg::TM; ++tm)
@@ -186,7 +248,6 @@ grouped_gemm_kernel(GroupedArgs p) {
   }
 
   // Epilogue: bias (+ GELU) (+ row scale), fp16, 8-byte stores through the row index.
-  const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
   float bias_v[Cfg::TN][4][4];
   int col[Cfg::TN][4];
 #pragma unroll
@@ -222,6 +283,7 @@ grouped_gemm_kernel(GroupedArgs p) {
         }
     }
   }
+  }
 }
 
 // ---- variants -------------------------------------------------------------------
@@ -234,6 +296,8 @@ using Cfg1 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 3>;   // 4 wavefronts of 128x1
 using Cfg2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 0>;   // 8 wavefronts, two whole-tile stages
 using Cfg3 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 1>;   // 8 wavefronts, BK=32 x 4 stages, ping-pong
 using Cfg4 = GemmCfg<256, 128, 32, 2, 2, 3, 2, 2, 0>;   // 4 wavefronts, 72 KB LDS: two workgroups per CU
+using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 4>;   // 4 wavefronts of 128x128, 16x16x32 MFMA, mid-tile barrier
+using Cfg6 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 8, 5>;   // 8 wavefronts of 128x64, 16x16x32 MFMA, rolling token fragments
 
 int g_variant = 0;
 
@@ -245,7 +309,7 @@ struct Launch {
 
 #define CCF_VARIANT(C) {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>}
 const Launch kVariants[] = {CCF_VARIANT(Cfg0), CCF_VARIANT(Cfg1), CCF_VARIANT(Cfg2), CCF_VARIANT(Cfg3),
-                            CCF_VARIANT(Cfg4)};
+                            CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5), CCF_VARIANT(Cfg6)};
 #undef CCF_VARIANT
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kMinBM = 128;
