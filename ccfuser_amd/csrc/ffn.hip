@@ -189,8 +189,8 @@ grouped_gemm_kernel(GroupedArgs p) {
   }
 
   const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
-  if constexpr (Cfg::SCHED == 4 || Cfg::SCHED == 5) {
-    using R = std::conditional_t<Cfg::SCHED == 4, Ring16Mainloop<Cfg>, Roll16Mainloop<Cfg>>;
+  if constexpr (Cfg::SCHED == 4) {
+    using R = Ring16Mainloop<Cfg>;
     float4v acc[R::TM][R::TN];
 #pragma unroll
     for (int tm = 0; tm < R::TM; ++tm)
@@ -297,9 +297,9 @@ using Cfg2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 0>;   // 8 wavefronts, two who
 using Cfg3 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 1>;   // 8 wavefronts, BK=32 x 4 stages, ping-pong
 using Cfg4 = GemmCfg<256, 128, 32, 2, 2, 3, 2, 2, 0>;   // 4 wavefronts, 72 KB LDS: two workgroups per CU
 using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 4>;   // 4 wavefronts of 128x128, 16x16x32 MFMA, mid-tile barrier
-using Cfg6 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 8, 5>;   // 8 wavefronts of 128x64, 16x16x32 MFMA, rolling token fragments
 
-int g_variant = 0;
+constexpr int kDefaultVariant = 5;
+int g_variant = kDefaultVariant;
 
 struct Launch {
   int bm, bn, threads;
@@ -309,7 +309,7 @@ struct Launch {
 
 #define CCF_VARIANT(C) {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>}
 const Launch kVariants[] = {CCF_VARIANT(Cfg0), CCF_VARIANT(Cfg1), CCF_VARIANT(Cfg2), CCF_VARIANT(Cfg3),
-                            CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5), CCF_VARIANT(Cfg6)};
+                            CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5)};
 #undef CCF_VARIANT
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kMinBM = 128;
@@ -366,9 +366,9 @@ extern "C" int ccf_set_option(const char *name, int value) {
   using namespace ccf;
   CCF_REQUIRE(name, CCF_ERR_ARG, "set_option: null name");
   if (!strcmp(name, "gemm_variant")) {
-    CCF_REQUIRE(value >= 0 && value < kNumVariants, CCF_ERR_ARG, "set_option: gemm_variant %d outside 0..%d",
+    CCF_REQUIRE(value >= -1 && value < kNumVariants, CCF_ERR_ARG, "set_option: gemm_variant %d outside -1..%d",
                 value, kNumVariants - 1);
-    g_variant = value;
+    g_variant = value < 0 ? kDefaultVariant : value;     // -1: back to the default
     return CCF_OK;
   }
   return fail(CCF_ERR_ARG, "set_option: unknown option %s", name);

@@ -655,17 +655,28 @@ struct Ring16Mainloop {
                                                  const half_t *const (&src)[NLOAD], int k_elem,
                                                  const int (&a_off)[2], const int (&b_off)[2], int wave,
                                                  int live_m) {
-    static_for<0, PER_SUB>([&](auto II) {
+    // what goes out behind MFMA i
+    auto behind = [&](auto II) {
       constexpr int i = II.value;
-      constexpr int tm = i / TN, tn = i % TN;
-      if (FULL || tm < live_m)
-        acc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[SUB][tn], a[SUB][tm], acc[tm][tn], 0, 0, 0);
       if constexpr (i < FRAGS) read_frag<RA, RB, RSUB, i>(a[SUB ^ 1], b[SUB ^ 1], a_off, b_off);
       if constexpr (i % Cfg::DMA_EVERY == 0 && i / Cfg::DMA_EVERY < NLOAD) {
         constexpr int l = i / Cfg::DMA_EVERY;
         lds_dma16(src[l] + k_elem, slot<WS>() + (l * Cfg::NW + wave) * 1024);
       }
       __builtin_amdgcn_sched_barrier(0);
+    };
+    static_for<0, TM>([&](auto T) {
+      constexpr int tm = T.value;
+      // one (wavefront-uniform) branch per row block, not per MFMA
+      if (FULL || tm < live_m) {
+        static_for<0, TN>([&](auto J) {
+          constexpr int tn = J.value;
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[SUB][tn], a[SUB][tm], acc[tm][tn], 0, 0, 0);
+          behind(std::integral_constant<int, tm * TN + tn>{});
+        });
+      } else {
+        static_for<0, TN>([&](auto J) { behind(std::integral_constant<int, tm * TN + J.value>{}); });
+      }
     });
   }
 
@@ -691,192 +702,6 @@ struct Ring16Mainloop {
       frags_ready(a[1], b[1]);
       __builtin_amdgcn_sched_barrier(0);
       substep<1, NA, NB, 0, SA, Cfg::B_DMA, FULL>(acc, a, b, b_src, k2, a_off, b_off, wave, live_m);
-    }
-  };
-
-  // rows: real rows of this M tile (1..BM).
-  static __device__ __forceinline__ void run(acc_t (&acc)[TM][TN], const half_t *const (&a_src)[Cfg::A_DMA],
-                                             const half_t *const (&b_src)[Cfg::B_DMA], int K, int rows) {
-    const int wave = threadIdx.x >> 6;
-    const int lane = threadIdx.x & 63;
-    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-    const int KT = K / Cfg::BK;
-    int live_m = (rows - wm * Cfg::WTM + 15) / 16;       // 16-row blocks of this wavefront with real rows
-    live_m = live_m < 0 ? 0 : (live_m > TM ? TM : live_m);
-    live_m = __builtin_amdgcn_readfirstlane(live_m);
-    // lane l of a 16x16x32 operand: row l%16, K elements 8*(l/16) .. +7 of the substep's 32
-    int a_off[2], b_off[2];
-    {
-      const int ra = wm * Cfg::WTM + (lane & 15);
-      const int rb = wn * Cfg::WTN + (lane & 15);
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
-        const int c = sub * 4 + (lane >> 4);
-        a_off[sub] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
-        b_off[sub] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
-      }
-    }
-    // Prologue: A(0) -> slot 0, B(0) -> slot 1, A(1) -> slot 2, B(1) -> slot 3.
-    const int k1 = (KT > 1 ? 1 : 0) * Cfg::BK;
-    issue_all<0>(a_src, 0, wave);
-    issue_all<1>(b_src, 0, wave);
-    issue_all<2>(a_src, k1, wave);
-    issue_all<3>(b_src, k1, wave);
-    wait_vmcnt<Cfg::A_DMA + Cfg::B_DMA>();
-    block_barrier();
-    half8 a[2][TM], b[2][TN];
-    static_for<0, FRAGS>([&](auto I) { read_frag<0, 1, 0, I.value>(a[0], b[0], a_off, b_off); });
-    if (live_m == TM) {
-      for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
-        static_for<0, NSLOT>([&](auto U) {
-          Step<U.value, true>::run(acc, a, b, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave, live_m);
-        });
-      }
-    } else {
-      for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
-        static_for<0, NSLOT>([&](auto U) {
-          Step<U.value, false>::run(acc, a, b, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave, live_m);
-        });
-      }
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    wait_vmcnt<0>();
-  }
-};
-
-// ---- 16x16x32, two wavefronts per SIMD, rolling token fragments -------------------
-// One wavefront cannot issue 16x16x32 MFMAs back to back at the full rate
-// (measured: one every 18 cycles, not 16, before any other instruction), and
-// every LDS read or tile load it issues in between costs MFMA slots.  With two
-// wavefronts per SIMD the other one fills those gaps, but each has only 256
-// registers: 128 accumulators (a 128x64 tile), so the fragments cannot all be
-// double buffered.  The four weight fragments of a substep are (b[2][TN]);
-// the eight token fragments are not: a[tm] is read by the four MFMAs of row
-// block tm only, so the read of its successor goes out right behind the last
-// of them and has the other 28 MFMAs of the substep to return.
-//
-// Order of the 12 fragment reads of a substep: b0 a0 b1 b2 b3 a1 .. a7.  Before
-// the first MFMA of row block tm the wavefront waits until at most 7 (tm = 0)
-// or 11 (tm > 0) reads are in flight: those are the reads issued after a[tm]'s.
-// The workgroup barrier sits behind the first row block of substep 1: by then
-// the last read of tile k (issued behind the last MFMA of substep 0) has had
-// four MFMAs to return, and everything behind the barrier (the prefetch of
-// tile k+1's fragments, the loads of B(k+2) into A(k)'s slot) follows the same
-// rules as in Ring16Mainloop.
-template <class Cfg>
-struct Roll16Mainloop {
-  using acc_t = float4v;
-  static_assert(Cfg::BK == 64, "two K=32 substeps per K tile");
-  static_assert(Cfg::A_BYTES == Cfg::B_BYTES, "ring slots are one size");
-  static constexpr int NSLOT = 5;
-  static constexpr int TM = Cfg::WTM / 16, TN = Cfg::WTN / 16;   // 16x16 blocks per wavefront
-  static constexpr int PER_SUB = TM * TN;
-  static_assert(TN == 4 && TM >= 2, "read schedule written for four weight fragments");
-  static_assert(TM + TN <= 15, "LDS reads in flight are counted in four bits");
-  static_assert((Cfg::A_DMA - 1) * Cfg::DMA_EVERY + 1 < PER_SUB - TN &&
-                    (Cfg::B_DMA - 1) * Cfg::DMA_EVERY + 1 < PER_SUB - TN,
-                "not enough MFMA slots for the tile loads");
-
-  // One LDS object; slot S is bytes [S*A_BYTES, (S+1)*A_BYTES).
-  template <int S>
-  static __device__ __forceinline__ lds_char *slot() {
-    return stage_buf<300, NSLOT * Cfg::A_BYTES>() + S * Cfg::A_BYTES;
-  }
-  // LDS byte address of (slot S) + off, added where it is used: left to itself
-  // the compiler keeps all 20 slot x fragment-offset sums in registers across
-  // the loop, which the 256-register budget cannot afford.
-  template <int S>
-  static __device__ __forceinline__ uint32_t in_slot(uint32_t off) {
-    const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(slot<S>()));
-    uint32_t r;
-    asm volatile("v_add_u32 %0, %1, %2" : "=v"(r) : "s"(base), "v"(off));
-    return r;
-  }
-
-  template <int SLOT, int N>
-  static __device__ __forceinline__ void issue_all(const half_t *const (&src)[N], int k_elem, int wave) {
-    static_for<0, N>([&](auto I) {
-      lds_dma16(src[I.value] + k_elem, slot<SLOT>() + (I.value * Cfg::NW + wave) * 1024);
-    });
-  }
-
-  static __device__ __forceinline__ void tie(half8 &x) { asm volatile("" : "+v"(x)); }
-  template <int N>
-  static __device__ __forceinline__ void wait_reads() {
-    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N));
-  }
-
-  // Reads behind MFMA I of a substep that fetches the fragments of (slots RA/RB,
-  // K half RSUB) into a[] and bn[].  FIRST is the MFMA index of the first read.
-  // ra / rb: LDS address of this lane's chunk of row block 0 in the slots read from.
-  template <int FIRST, int I>
-  static __device__ __forceinline__ void reads_behind(half8 (&a)[TM], half8 (&bn)[TN], uint32_t ra, uint32_t rb) {
-    constexpr int tm = I / TN, tn = I % TN;
-    if constexpr (I >= FIRST && I < FIRST + TN)
-      bn[I - FIRST] = lds_read_b128<(I - FIRST) * 16 * Cfg::CPR * 16>(rb);
-    // a[0] is free once row block 0 is done, but no read may go out before FIRST
-    if constexpr (FIRST > TN - 1 && I == FIRST) a[0] = lds_read_b128<0>(ra);
-    if constexpr (tn == TN - 1 && (tm > 0 || FIRST <= TN - 1)) a[tm] = lds_read_b128<tm * 16 * Cfg::CPR * 16>(ra);
-  }
-
-  template <int U, bool FULL>
-  struct Step {
-    static __device__ __forceinline__ void run(acc_t (&acc)[TM][TN], half8 (&a)[TM], half8 (&b)[2][TN],
-                                               const half_t *const (&a_src)[Cfg::A_DMA],
-                                               const half_t *const (&b_src)[Cfg::B_DMA],
-                                               const int (&a_off)[2], const int (&b_off)[2], int kt, int KT,
-                                               int wave, int live_m) {
-      constexpr int SA = (2 * U) % NSLOT, SB = (2 * U + 1) % NSLOT;       // tile kt
-      constexpr int NA = (2 * U + 2) % NSLOT, NB = (2 * U + 3) % NSLOT;   // tile kt+1
-      constexpr int WA = (2 * U + 4) % NSLOT;                             // A(kt+2); B(kt+2) goes to SA
-      constexpr int BAR = TN;                                             // barrier sits before MFMA BAR of substep 1
-      if (kt >= KT) return;                                               // uniform
-      // past the end the last K tile is fetched again into slots nobody reads
-      const int k2 = ((kt + 2 < KT) ? kt + 2 : KT - 1) * Cfg::BK;
-      // substep 0: fragments of K half 0 in a[], b[0]; fetch K half 1 into a[], b[1]
-      const uint32_t ra1 = in_slot<SA>(a_off[1]), rb1 = in_slot<SB>(b_off[1]);
-      static_for<0, PER_SUB>([&](auto II) {
-        constexpr int i = II.value;
-        constexpr int tm = i / TN, tn = i % TN;
-        if constexpr (tn == 0) {
-          wait_reads<tm == 0 ? TM - 1 : TM + TN - 1>();
-          tie(a[tm]);
-          if constexpr (tm == 0) static_for<0, TN>([&](auto J) { tie(b[0][J.value]); });
-        }
-        if (FULL || tm < live_m)
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[0][tn], a[tm], acc[tm][tn], 0, 0, 0);
-        reads_behind<0, i>(a, b[1], ra1, rb1);
-        if constexpr (i % Cfg::DMA_EVERY == 1 && i / Cfg::DMA_EVERY < Cfg::A_DMA) {
-          constexpr int l = i / Cfg::DMA_EVERY;
-          lds_dma16(a_src[l] + k2, slot<WA>() + (l * Cfg::NW + wave) * 1024);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      });
-      // substep 1: K half 1; behind the barrier fetch tile kt+1's K half 0 into a[], b[0]
-      const uint32_t ra0 = in_slot<NA>(a_off[0]), rb0 = in_slot<NB>(b_off[0]);
-      static_for<0, PER_SUB>([&](auto II) {
-        constexpr int i = II.value;
-        constexpr int tm = i / TN, tn = i % TN;
-        if constexpr (i == 0) {
-          wait_reads<TM - 1>();
-          tie(a[0]);
-          static_for<0, TN>([&](auto J) { tie(b[1][J.value]); });
-        }
-        if constexpr (i == BAR) {
-          // B(kt+1) and everything older have landed; A(kt+2) may stay in flight
-          wait_vmcnt<Cfg::A_DMA>();
-          block_barrier();                                                // waits for every LDS read, too
-          static_for<1, TM>([&](auto T) { tie(a[T.value]); });
-        }
-        if (FULL || tm < live_m)
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[1][tn], a[tm], acc[tm][tn], 0, 0, 0);
-        reads_behind<BAR, i>(a, b[0], ra0, rb0);
-        if constexpr (i >= BAR && (i - BAR) % Cfg::DMA_EVERY == 1 && (i - BAR) / Cfg::DMA_EVERY < Cfg::B_DMA) {
-          constexpr int l = (i - BAR) / Cfg::DMA_EVERY;
-          lds_dma16(b_src[l] + k2, slot<SA>() + (l * Cfg::NW + wave) * 1024);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      });
     }
   };
 
@@ -910,12 +735,8 @@ struct Roll16Mainloop {
     issue_all<3>(b_src, k1, wave);
     wait_vmcnt<Cfg::A_DMA + Cfg::B_DMA>();
     block_barrier();
-    half8 a[TM], b[2][TN];
-    // same order as the reads of a substep: b0 a0 b1 b2 b3 a1 .. a7
-    {
-      const uint32_t ra0 = in_slot<0>(a_off[0]), rb0 = in_slot<1>(b_off[0]);
-      static_for<0, PER_SUB>([&](auto II) { reads_behind<TN, II.value>(a, b[0], ra0, rb0); });
-    }
+    half8 a[2][TM], b[2][TN];
+    static_for<0, FRAGS>([&](auto I) { read_frag<0, 1, 0, I.value>(a[0], b[0], a_off, b_off); });
     if (live_m == TM) {
       for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
         static_for<0, NSLOT>([&](auto U) {

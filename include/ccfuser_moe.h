@@ -54,8 +54,8 @@ const char *ccf_last_error(void);
 
 /*
  * Tuning knobs (no counterpart in the reference).  "gemm_variant" selects the
- * grouped-GEMM tile configuration used by the FFN entry points; 0 is the
- * default.  Process-wide; not meant to be changed while work is in flight.
+ * grouped-GEMM main-loop variant used by the FFN entry points; -1 restores
+ * the default.  Process-wide; not meant to be changed while work is in flight.
  */
 int ccf_set_option(const char *name, int value);
 
