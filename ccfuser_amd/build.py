@@ -28,6 +28,8 @@ COMMON = [
 PER_FILE = {
     # the gate's fp32 accumulation order must survive the optimiser
     "gate.hip": ["-ffp-contract=off"],
+    # the 16x16x32 main loop names its accumulation registers itself: nothing of the compiler's may live there
+    "ffn.hip": ["-mllvm", "-amdgpu-spill-vgpr-to-agpr=0"],
 }
 
 

@@ -82,9 +82,10 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
   __syncthreads();
   // Hardware hands consecutive workgroup ids to the 8 XCDs in turn, so XCD x
   // runs ids x, x+8, ... in order.  Each class is cut into eight equal
-  // contiguous runs of logical tile ids, one per XCD (one L2): slot j of XCD x
-  // is long tile x*per_long + j for j < per_long, else short tile
-  // x*per_short + (j - per_long).
+  // contiguous runs of logical tile ids, one per XCD (one L2): with nl long
+  // tiles on XCD x, its slot j is long tile x*per_long + j for j < nl, else
+  // short tile x*per_short + (j - nl).  The used slots of an XCD are a prefix:
+  // the first idle entry ends its list.
   const long long total_long = static_cast<long long>(s_long[E]) * n_tiles_n;
   const long long total_short = static_cast<long long>(s_short[E]) * n_tiles_n;
   const long long per_long = (total_long + 7) / 8;
@@ -121,7 +122,10 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
       const long long first_s = static_cast<long long>(s_short[e]) * n_tiles_n;
       for (int tn = lane; tn < n_tiles_n; tn += 64) {
         const long long logical = first_s + tn;
-        const long long b = (per_long + logical % per_short) * 8 + logical / per_short;
+        const long long x = logical / per_short;
+        long long nl_x = total_long - x * per_long;              // long tiles on this XCD
+        nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
+        const long long b = (nl_x + logical % per_short) * 8 + x;
         if (b < wgs) entry[b] = int4v{e, lo + i * BM, cnt - i * BM, tn};
       }
     }
@@ -159,6 +163,81 @@ __device__ __forceinline__ float gelu_erf(float v) {
   return 0.5f * fmaf(fabsf(v), erf_abs, v);
 }
 
+// Global source of every tile load of this lane for the tile of plan entry
+// `ent`: K element 0 of the (clamped) A row and B row, at this lane's K chunk.
+// Padded A rows re-read the tile's last real row, B rows past N the last row.
+template <class Cfg>
+__device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v ent,
+                                             const half_t *(&a_src)[Cfg::A_DMA],
+                                             const half_t *(&b_src)[Cfg::B_DMA]) {
+  using ML = GemmMainloop<Cfg>;
+  const int row0 = ent[1], rows = ent[2], n0 = ent[3] * Cfg::BN;
+  const half_t *Be = p.B + static_cast<size_t>(ent[0]) * p.N * p.K;
+#pragma unroll
+  for (int i = 0; i < Cfg::A_DMA; ++i) {
+    const int r = ML::dma_row(i);
+    const int rc = r < rows ? r : rows - 1;
+    const int g = p.a_rows ? p.a_rows[row0 + rc] : row0 + rc;
+    a_src[i] = p.A + static_cast<size_t>(g) * p.K + ML::dma_chunk(r) * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < Cfg::B_DMA; ++i) {
+    const int r = ML::dma_row(i);
+    const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
+    b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r) * 8;
+  }
+}
+
+// Epilogue of the 16x16x32 accumulator layout: bias (+ GELU) (+ row scale),
+// fp16, 8-byte stores through the row index.
+template <class Cfg, bool kGelu>
+__device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0, int rows, int n0) {
+  using R = Ring16Mainloop<Cfg>;
+  constexpr int TM = R::TM, TN = R::TN;
+  const int tid = fresh_tid();
+  const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
+  float bias_v[TN][4];
+  int col[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) {
+    col[tn] = n0 + acc16_col4<Cfg>(tn, tid);
+    half4 bv = {0, 0, 0, 0};
+    if (col[tn] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn]);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) bias_v[tn][c] = static_cast<float>(bv[c]);
+  }
+  static_for<0, TM>([&](auto T) {
+    constexpr int tm = T.value;
+    const int lr = acc16_row<Cfg>(tm, tid);
+    // the accumulator reads are unconditional (they are asm the compiler must not skip per lane)
+    float v[TN][4];
+    static_for<0, TN>([&](auto J) {
+      constexpr int tn = J.value;
+      v[tn][0] = R::template acc_get<tm, tn, 0>();
+      v[tn][1] = R::template acc_get<tm, tn, 1>();
+      v[tn][2] = R::template acc_get<tm, tn, 2>();
+      v[tn][3] = R::template acc_get<tm, tn, 3>();
+    });
+    if (lr < rows) {
+      const int j = row0 + lr;
+      const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
+      const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
+      half_t *dst = p.C + crow * p.N;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        half4 o;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          float x = v[tn][c] + bias_v[tn][c];
+          if (kGelu) x = gelu_erf(x);
+          o[c] = static_cast<half_t>(x * sc);
+        }
+        if (col[tn] < p.N) *reinterpret_cast<half4 *>(dst + col[tn]) = o;
+      }
+    }
+  });
+}
+
 template <class Cfg, bool kGelu>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_kernel(GroupedArgs p) {
@@ -170,65 +249,15 @@ grouped_gemm_kernel(GroupedArgs p) {
   const int rows = ent[2];
   const int tile_n = ent[3];
   const int n0 = tile_n * Cfg::BN;
-  const half_t *Be = p.B + static_cast<size_t>(e) * p.N * p.K;
 
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[Cfg::B_DMA];
-#pragma unroll
-  for (int i = 0; i < Cfg::A_DMA; ++i) {
-    const int r = ML::dma_row(i);
-    const int rc = r < rows ? r : rows - 1;          // padded rows re-read a valid row
-    const int g = p.a_rows ? p.a_rows[row0 + rc] : row0 + rc;
-    a_src[i] = p.A + static_cast<size_t>(g) * p.K + ML::dma_chunk(r) * 8;
-  }
-#pragma unroll
-  for (int i = 0; i < Cfg::B_DMA; ++i) {
-    const int r = ML::dma_row(i);
-    const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-    b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r) * 8;
-  }
+  tile_sources<Cfg>(p, ent, a_src, b_src);
 
   const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
   if constexpr (Cfg::SCHED == 4) {
-    using R = Ring16Mainloop<Cfg>;
-    float4v acc[R::TM][R::TN];
-#pragma unroll
-    for (int tm = 0; tm < R::TM; ++tm)
-#pragma unroll
-      for (int tn = 0; tn < R::TN; ++tn) acc[tm][tn] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
-    R::run(acc, a_src, b_src, p.K, rows);
-    // Epilogue: bias (+ GELU) (+ row scale), fp16, 8-byte stores through the row index.
-    float bias_v[R::TN][4];
-    int col[R::TN];
-#pragma unroll
-    for (int tn = 0; tn < R::TN; ++tn) {
-      col[tn] = n0 + acc16_col4<Cfg>(tn);
-      half4 bv = {0, 0, 0, 0};
-      if (col[tn] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn]);
-#pragma unroll
-      for (int c = 0; c < 4; ++c) bias_v[tn][c] = static_cast<float>(bv[c]);
-    }
-#pragma unroll
-    for (int tm = 0; tm < R::TM; ++tm) {
-      const int lr = acc16_row<Cfg>(tm);
-      if (lr < rows) {
-        const int j = row0 + lr;
-        const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
-        const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
-        half_t *dst = p.C + crow * p.N;
-#pragma unroll
-        for (int tn = 0; tn < R::TN; ++tn) {
-          half4 o;
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            float v = acc[tm][tn][c] + bias_v[tn][c];
-            if (kGelu) v = gelu_erf(v);
-            o[c] = static_cast<half_t>(v * sc);
-          }
-          if (col[tn] < p.N) *reinterpret_cast<half4 *>(dst + col[tn]) = o;
-        }
-      }
-    }
+    Ring16Mainloop<Cfg>::run(a_src, b_src, p.K, rows);
+    epilogue16<Cfg, kGelu>(p, e, row0, rows, n0);
     return;
   } else {
   typename ML::acc_t acc[Cfg::TM][Cfg::TN];
@@ -286,6 +315,123 @@ grouped_gemm_kernel(GroupedArgs p) {
   }
 }
 
+// ---- persistent form -------------------------------------------------------------
+// One workgroup per CU walks the plan entries of its XCD (entry b belongs to XCD
+// b % 8; the workgroup with blockIdx b takes slots b/8, b/8 + gridDim/8, ...).
+// What it buys over one workgroup per tile: the first two K tiles of the NEXT
+// tile are loaded by the last two K-tile steps of the current one (where the
+// plain kernel re-fetches its last K tile into slots nobody reads), so they
+// arrive under the epilogue, and the next main loop starts with operands in
+// LDS and its first fragments in registers; no workgroup launch, no pipeline
+// fill, no drain between tiles.  The ring phase (which slot holds what) simply
+// carries on across tiles.
+//
+// Per tile (K has at least four K tiles): the row indices of the next tile's A
+// rows are requested before the first step (plain loads in inline asm, so that
+// no compiler-placed wait drains the tile loads in flight; the vmcnt wait of
+// the first barrier covers them); steps 0 .. KT-3 run with this tile's sources;
+// then the sources of the next tile are computed and the last two steps load
+// its K tiles 0 and 1.
+template <class Cfg, bool kGelu>
+__global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
+grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
+  using ML = GemmMainloop<Cfg>;
+  using R = Ring16Mainloop<Cfg>;
+  constexpr int TM = R::TM, TN = R::TN;
+  const int4v *plan = reinterpret_cast<const int4v *>(p.plan);
+  const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
+  int slot_j = blockIdx.x >> 3;
+  if (slot_j >= slots_per_xcd) return;
+  int4v ent = plan[slot_j * 8 + xcd];
+  if (ent[0] < 0) return;                             // the used slots of an XCD are a prefix
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int KT = p.K / Cfg::BK;
+
+  const half_t *a_src[Cfg::A_DMA];
+  const half_t *b_src[Cfg::B_DMA];
+  tile_sources<Cfg>(p, ent, a_src, b_src);
+  int a_off[2], b_off[2];
+  R::frag_offsets(a_off, b_off);
+  half8 fa[2][TM], fb[2][TN];
+  R::prologue(fa, fb, a_src, b_src, KT, a_off, b_off, wave);
+  R::reserve();
+  int phase = 0;
+
+  for (;;) {
+    // the entry after this one; without one, the tail steps re-fetch this tile's first K tiles
+    const int nj = slot_j + stride;
+    int4v nent = ent;
+    bool has_next = false;
+    if (nj < slots_per_xcd) {
+      const int4v t = plan[nj * 8 + xcd];
+      if (t[0] >= 0) {
+        nent = t;
+        has_next = true;
+      }
+    }
+    const int n_row0 = nent[1], n_rows = nent[2];
+
+    R::zero_acc();
+
+    int next_row[Cfg::A_DMA];                         // A row of the next tile per tile load
+    const int tid0 = fresh_tid();
+#pragma unroll
+    for (int i = 0; i < Cfg::A_DMA; ++i) {
+      const int r = ML::dma_row(i, tid0);
+      const int rc = r < n_rows ? r : n_rows - 1;
+      if (p.a_rows) {
+        const int32_t *src = p.a_rows + n_row0 + rc;
+        asm volatile("global_load_dword %0, %1, off" : "=v"(next_row[i]) : "v"(src) : "memory");
+      } else {
+        next_row[i] = n_row0 + rc;
+      }
+    }
+
+    const int live_m = R::live_blocks(ent[2]);
+    R::acc_settle();
+    if (live_m == TM) {
+      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, p.K, phase, wave, live_m);
+    } else {
+      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, p.K, phase, wave, live_m);
+    }
+    {
+      // sources of the next tile (tile_sources() with the row indices already at hand); the
+      // empty asm keeps the compiler from computing them before the loop above and holding
+      // 16 more registers across it
+      int n_e = nent[0], n_tn = nent[3];
+      asm volatile("" : "+s"(n_e), "+s"(n_tn));
+      const half_t *Be = p.B + static_cast<size_t>(n_e) * p.N * p.K;
+      const int n0 = n_tn * Cfg::BN;
+      const int tid1 = fresh_tid();
+#pragma unroll
+      for (int i = 0; i < Cfg::A_DMA; ++i) {
+        asm volatile("" : "+v"(next_row[i]));         // requested before step 0, complete at its barrier
+        const int r = ML::dma_row(i, tid1);
+        a_src[i] = p.A + static_cast<size_t>(next_row[i]) * p.K + ML::dma_chunk(r, tid1) * 8;
+      }
+#pragma unroll
+      for (int i = 0; i < Cfg::B_DMA; ++i) {
+        const int r = ML::dma_row(i, tid1);
+        const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
+        b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r, tid1) * 8;
+      }
+    }
+    if (live_m == TM) {
+      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, p.K, phase, wave, live_m);
+    } else {
+      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, p.K, phase, wave, live_m);
+    }
+    R::acc_settle();
+    epilogue16<Cfg, kGelu>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
+    R::acc_settle();
+    if (!has_next) break;
+    ent = nent;
+    slot_j = nj;
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  wait_vmcnt<0>();
+}
+
 // ---- variants -------------------------------------------------------------------
 // 256x256x64 tiles throughout (the most flop per byte pulled from L2 that the
 // register file allows).  What differs is how the tile loads are pipelined and
@@ -297,20 +443,43 @@ using Cfg2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 0>;   // 8 wavefronts, two who
 using Cfg3 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 1>;   // 8 wavefronts, BK=32 x 4 stages, ping-pong
 using Cfg4 = GemmCfg<256, 128, 32, 2, 2, 3, 2, 2, 0>;   // 4 wavefronts, 72 KB LDS: two workgroups per CU
 using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 4>;   // 4 wavefronts of 128x128, 16x16x32 MFMA, mid-tile barrier
+// variant 6: Cfg5 again, persistent workgroups
 
-constexpr int kDefaultVariant = 5;
+constexpr int kDefaultVariant = 6;
 int g_variant = kDefaultVariant;
 
 struct Launch {
   int bm, bn, threads;
   void (*plain)(GroupedArgs);
   void (*gelu)(GroupedArgs);
+  // persistent form (one workgroup per CU), or null; used when K has at least kPersistentMinKT K tiles
+  void (*persistent_plain)(GroupedArgs, int);
+  void (*persistent_gelu)(GroupedArgs, int);
 };
+constexpr int kPersistentMinKT = 4;
 
-#define CCF_VARIANT(C) {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>}
+#define CCF_VARIANT(C) {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>, nullptr, nullptr}
+#define CCF_VARIANT_P(C)                                                                          \
+  {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>,          \
+   grouped_gemm_persistent_kernel<C, false>, grouped_gemm_persistent_kernel<C, true>}
 const Launch kVariants[] = {CCF_VARIANT(Cfg0), CCF_VARIANT(Cfg1), CCF_VARIANT(Cfg2), CCF_VARIANT(Cfg3),
-                            CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5)};
+                            CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5), CCF_VARIANT_P(Cfg5)};
 #undef CCF_VARIANT
+#undef CCF_VARIANT_P
+
+// Compute units of the current device, rounded down to whole XCD rounds of 8.
+int persistent_grid() {
+  static thread_local int cached_dev = -1, cached = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev != cached_dev) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cached = cus / 8 * 8;
+    cached_dev = dev;
+  }
+  return cached;
+}
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kMinBM = 128;
 
@@ -354,8 +523,15 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.K = K;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
-  hipLaunchKernelGGL(gelu ? v.gelu : v.plain, dim3(static_cast<unsigned>(wgs)), dim3(v.threads), 0,
-                     stream, p);
+  const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
+  if (grid >= 8) {
+    const long long g = grid < wgs ? grid : wgs;                // wgs is a multiple of 8
+    hipLaunchKernelGGL(gelu ? v.persistent_gelu : v.persistent_plain, dim3(static_cast<unsigned>(g)),
+                       dim3(v.threads), 0, stream, p, static_cast<int>(wgs / 8));
+  } else {
+    hipLaunchKernelGGL(gelu ? v.gelu : v.plain, dim3(static_cast<unsigned>(wgs)), dim3(v.threads), 0,
+                       stream, p);
+  }
   return check_launch(what);
 }
 

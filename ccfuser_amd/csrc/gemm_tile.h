@@ -117,6 +117,15 @@ __device__ __forceinline__ void lds_dma16(const void *gptr, lds_char *lds_wave_b
                                    (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
 }
 
+// threadIdx.x as a value the compiler cannot trace back: what is derived from it
+// is computed where it is used, not once at kernel start and then held in
+// registers across the main loop (the persistent kernel has none to spare).
+__device__ __forceinline__ int fresh_tid() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WGS_PER_CU_ = 1,
           int DMA_EVERY_ = 2, int SCHED_ = 0>
 struct GemmCfg {
@@ -426,14 +435,18 @@ struct GemmMainloop {
   }
 
   // Tile row this lane fetches with its i-th A (or B) load, and the K-chunk.
-  static __device__ __forceinline__ int dma_row(int i) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // tid: threadIdx.x, or fresh_tid() where the values derived from it must not
+  // be computed early and kept in registers.
+  static __device__ __forceinline__ int dma_row(int i, int tid) {
+    const int wave = tid >> 6, lane = tid & 63;
     return (i * Cfg::NW + wave) * Cfg::ROWS_PER_DMA + lane / Cfg::CPR;
   }
-  static __device__ __forceinline__ int dma_chunk(int row) {
-    const int lane = threadIdx.x & 63;
+  static __device__ __forceinline__ int dma_chunk(int row, int tid) {
+    const int lane = tid & 63;
     return (lane % Cfg::CPR) ^ swz<Cfg::CPR>(row);
   }
+  static __device__ __forceinline__ int dma_row(int i) { return dma_row(i, threadIdx.x); }
+  static __device__ __forceinline__ int dma_chunk(int row) { return dma_chunk(row, threadIdx.x); }
 };
 
 // ---- five-slot ring ------------------------------------------------------------
@@ -599,12 +612,18 @@ struct RingMainloop {
 // * A(k+2) is loaded during substep 0 into the fifth slot, B(k+2) during
 //   substep 1 into the slot A(k) just left; at the barrier only A(k+2) may
 //   still be in flight.
+//
+// The ring phase (which slot holds what) is a run-time value: one step body
+// serves every phase, the slot addresses are a few scalar adds per K tile, and a
+// caller that runs tile after tile (the persistent kernel) simply carries the
+// phase on.
 template <class Cfg>
 struct Ring16Mainloop {
   using acc_t = float4v;
   static_assert(Cfg::BK == 64, "two K=32 substeps per K tile");
   static_assert(Cfg::A_BYTES == Cfg::B_BYTES, "ring slots are one size");
   static constexpr int NSLOT = 5;
+  static constexpr int SLOT_BYTES = Cfg::A_BYTES;
   static constexpr int TM = Cfg::WTM / 16, TN = Cfg::WTN / 16;   // 16x16 blocks per wavefront
   static constexpr int FRAGS = TM + TN;
   static constexpr int PER_SUB = TM * TN;                        // MFMAs per substep
@@ -612,28 +631,44 @@ struct Ring16Mainloop {
   static_assert(PER_SUB / Cfg::DMA_EVERY >= Cfg::A_DMA && PER_SUB / Cfg::DMA_EVERY >= Cfg::B_DMA,
                 "not enough MFMA slots for the tile loads");
 
-  template <int S>
-  static __device__ __forceinline__ lds_char *slot() {
-    return stage_buf<200 + S, Cfg::A_BYTES>();
+  // One LDS object; slot s is bytes [s * SLOT_BYTES, (s + 1) * SLOT_BYTES).
+  static __device__ __forceinline__ lds_char *lds() { return stage_buf<200, NSLOT * SLOT_BYTES>(); }
+  static __device__ __forceinline__ uint32_t lds_addr() {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds()));
+  }
+  // (x mod 5) for 0 <= x < 10
+  static __device__ __forceinline__ int mod5(int x) { return x >= NSLOT ? x - NSLOT : x; }
+
+  // Slots of ring phase ph (0..4): K tile kt in a/b, kt+1 in na/nb, A(kt+2) goes to wa, B(kt+2) to a.
+  struct Slots {
+    int a, b, na, nb, wa;   // byte offsets into lds()
+  };
+  static __device__ __forceinline__ Slots slots_of(int ph) {
+    Slots s;
+    const int x = mod5(2 * ph);                      // 2*ph mod 5
+    s.a = x * SLOT_BYTES;
+    s.b = mod5(x + 1) * SLOT_BYTES;
+    s.na = mod5(x + 2) * SLOT_BYTES;
+    s.nb = mod5(x + 3) * SLOT_BYTES;
+    s.wa = mod5(x + 4) * SLOT_BYTES;
+    return s;
   }
 
-  template <int SLOT, int N>
-  static __device__ __forceinline__ void issue_all(const half_t *const (&src)[N], int k_elem, int wave) {
+  template <int N>
+  static __device__ __forceinline__ void issue_all(const half_t *const (&src)[N], int k_elem, int slot_off, int wave) {
     static_for<0, N>([&](auto I) {
-      lds_dma16(src[I.value] + k_elem, slot<SLOT>() + (I.value * Cfg::NW + wave) * 1024);
+      lds_dma16(src[I.value] + k_elem, lds() + slot_off + (I.value * Cfg::NW + wave) * 1024);
     });
   }
 
-  // Fragment I of substep SUB: the weight fragments first, then the token fragments.
-  template <int SA, int SB, int SUB, int I>
-  static __device__ __forceinline__ void read_frag(half8 (&a)[TM], half8 (&b)[TN], const int (&a_off)[2],
-                                                   const int (&b_off)[2]) {
-    const uint32_t base_a = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(slot<SA>()));
-    const uint32_t base_b = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(slot<SB>()));
+  // Fragment I of a substep: the weight fragments first, then the token fragments.
+  // ra / rb: LDS address of this lane's chunk of row block 0 in the slots read from.
+  template <int I>
+  static __device__ __forceinline__ void read_frag(half8 (&a)[TM], half8 (&b)[TN], uint32_t ra, uint32_t rb) {
     if constexpr (I < TN) {
-      b[I] = lds_read_b128<I * 16 * Cfg::CPR * 16>(base_b + b_off[SUB]);
+      b[I] = lds_read_b128<I * 16 * Cfg::CPR * 16>(rb);
     } else {
-      a[I - TN] = lds_read_b128<(I - TN) * 16 * Cfg::CPR * 16>(base_a + a_off[SUB]);
+      a[I - TN] = lds_read_b128<(I - TN) * 16 * Cfg::CPR * 16>(ra);
     }
   }
 
@@ -647,21 +682,54 @@ struct Ring16Mainloop {
     for (int i = 0; i < TN; ++i) asm volatile("" : "+v"(b[i]));
   }
 
+  // The accumulators are not C++ objects: block (tm, tn) lives in the accumulation
+  // registers a[4*(tm*TN+tn) .. +3], named literally in inline asm.  With 256
+  // of them next to 128 fragment registers the register allocator otherwise
+  // splits them between the two register files and copies them around inside
+  // the loop (or spills) as soon as the control flow is more than one loop.
+  // The file is compiled with VGPR-to-AGPR spilling off, so nothing else ever
+  // lives there; reserve() makes the kernel own all 256.  Being opaque, the
+  // MFMAs get no hazard padding from the compiler: callers keep the required
+  // distance to any other instruction that touches an accumulator (settle()).
+  static_assert(TM * TN * 4 <= 256, "accumulation registers");
+  static __device__ __forceinline__ void reserve() { asm volatile("" ::: "a255"); }
+  // acc(tm, tn) += w (16 weight rows) x t (16 token rows), K = 32
+  template <int BLK>
+  static __device__ __forceinline__ void mfma16(const half8 &w, const half8 &t) {
+    asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]"
+                 :
+                 : "v"(w), "v"(t), "n"(4 * BLK), "n"(4 * BLK + 3));
+  }
+  static __device__ __forceinline__ void zero_acc() {
+    static_for<0, TM * TN * 4>([&](auto R_) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(R_.value)); });
+  }
+  // element c (0..3) of block (tm, tn)
+  template <int TM_, int TN_, int C>
+  static __device__ __forceinline__ float acc_get() {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v) : "n"((TM_ * TN + TN_) * 4 + C));
+    return v;
+  }
+  // Distance between an MFMA and the first other reader or writer of an
+  // accumulator, or the other way round (a 4-pass MFMA needs at most 11 wait
+  // states; this is 32).
+  static __device__ __forceinline__ void acc_settle() { asm volatile("s_nop 15\n s_nop 15" ::: "memory"); }
+
   // One substep: PER_SUB MFMAs on fragment buffer SUB; behind the first FRAGS of
-  // them the reads of the NEXT substep's fragments (slots RA, RB, K half RSUB)
-  // into the other buffer; behind every DMA_EVERY-th one a tile load into slot WS.
-  template <int SUB, int RA, int RB, int RSUB, int WS, int NLOAD, bool FULL>
-  static __device__ __forceinline__ void substep(acc_t (&acc)[TM][TN], half8 (&a)[2][TM], half8 (&b)[2][TN],
-                                                 const half_t *const (&src)[NLOAD], int k_elem,
-                                                 const int (&a_off)[2], const int (&b_off)[2], int wave,
-                                                 int live_m) {
+  // them the reads of the NEXT substep's fragments (LDS addresses ra, rb) into
+  // the other buffer; behind every DMA_EVERY-th one a tile load into the slot
+  // at byte offset ws.
+  template <int SUB, int NLOAD, bool FULL>
+  static __device__ __forceinline__ void substep(half8 (&a)[2][TM], half8 (&b)[2][TN],
+                                                 const half_t *const (&src)[NLOAD], int k_elem, uint32_t ra,
+                                                 uint32_t rb, int ws, int wave, int live_m) {
     // what goes out behind MFMA i
     auto behind = [&](auto II) {
       constexpr int i = II.value;
-      if constexpr (i < FRAGS) read_frag<RA, RB, RSUB, i>(a[SUB ^ 1], b[SUB ^ 1], a_off, b_off);
+      if constexpr (i < FRAGS) read_frag<i>(a[SUB ^ 1], b[SUB ^ 1], ra, rb);
       if constexpr (i % Cfg::DMA_EVERY == 0 && i / Cfg::DMA_EVERY < NLOAD) {
         constexpr int l = i / Cfg::DMA_EVERY;
-        lds_dma16(src[l] + k_elem, slot<WS>() + (l * Cfg::NW + wave) * 1024);
+        lds_dma16(src[l] + k_elem, lds() + ws + (l * Cfg::NW + wave) * 1024);
       }
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -671,7 +739,7 @@ struct Ring16Mainloop {
       if (FULL || tm < live_m) {
         static_for<0, TN>([&](auto J) {
           constexpr int tn = J.value;
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[SUB][tn], a[SUB][tm], acc[tm][tn], 0, 0, 0);
+          mfma16<tm * TN + tn>(b[SUB][tn], a[SUB][tm]);
           behind(std::integral_constant<int, tm * TN + tn>{});
         });
       } else {
@@ -680,78 +748,110 @@ struct Ring16Mainloop {
     });
   }
 
-  template <int U, bool FULL>
-  struct Step {
-    static __device__ __forceinline__ void run(acc_t (&acc)[TM][TN], half8 (&a)[2][TM], half8 (&b)[2][TN],
-                                               const half_t *const (&a_src)[Cfg::A_DMA],
-                                               const half_t *const (&b_src)[Cfg::B_DMA],
-                                               const int (&a_off)[2], const int (&b_off)[2], int kt, int KT,
-                                               int wave, int live_m) {
-      constexpr int SA = (2 * U) % NSLOT, SB = (2 * U + 1) % NSLOT;       // tile kt
-      constexpr int NA = (2 * U + 2) % NSLOT, NB = (2 * U + 3) % NSLOT;   // tile kt+1
-      constexpr int WA = (2 * U + 4) % NSLOT;                             // A(kt+2); B(kt+2) goes to SA
-      if (kt >= KT) return;                                               // uniform
-      // past the end the last K tile is fetched again into slots nobody reads
-      const int k2 = ((kt + 2 < KT) ? kt + 2 : KT - 1) * Cfg::BK;
-      frags_ready(a[0], b[0]);
-      __builtin_amdgcn_sched_barrier(0);
-      substep<0, SA, SB, 1, WA, Cfg::A_DMA, FULL>(acc, a, b, a_src, k2, a_off, b_off, wave, live_m);
-      // B(kt+1) and everything older have landed; A(kt+2) may stay in flight
-      wait_vmcnt<Cfg::A_DMA>();
-      block_barrier();
-      frags_ready(a[1], b[1]);
-      __builtin_amdgcn_sched_barrier(0);
-      substep<1, NA, NB, 0, SA, Cfg::B_DMA, FULL>(acc, a, b, b_src, k2, a_off, b_off, wave, live_m);
-    }
-  };
+  // K tile kt in ring phase ph; k2: K element offset of the K tile that the loads
+  // of this step fetch (A into the fifth slot, B into the slot A(kt) leaves).
+  template <bool FULL>
+  static __device__ __forceinline__ void step(half8 (&a)[2][TM], half8 (&b)[2][TN],
+                                              const half_t *const (&a_src)[Cfg::A_DMA],
+                                              const half_t *const (&b_src)[Cfg::B_DMA], const int (&a_off)[2],
+                                              const int (&b_off)[2], int k2, int ph, int wave, int live_m) {
+    const Slots s = slots_of(ph);
+    const uint32_t base = lds_addr();
+    frags_ready(a[0], b[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    // K half 0; fetch the fragments of K half 1 of this tile; load A(kt+2)
+    substep<0, Cfg::A_DMA, FULL>(a, b, a_src, k2, base + s.a + a_off[1], base + s.b + b_off[1], s.wa, wave,
+                                 live_m);
+    // B(kt+1) and everything older have landed; A(kt+2) may stay in flight
+    wait_vmcnt<Cfg::A_DMA>();
+    block_barrier();
+    frags_ready(a[1], b[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    // K half 1; fetch the fragments of K half 0 of tile kt+1; load B(kt+2) into A(kt)'s slot
+    substep<1, Cfg::B_DMA, FULL>(a, b, b_src, k2, base + s.na + a_off[0], base + s.nb + b_off[0], s.a, wave,
+                                 live_m);
+  }
 
-  // rows: real rows of this M tile (1..BM).
-  static __device__ __forceinline__ void run(acc_t (&acc)[TM][TN], const half_t *const (&a_src)[Cfg::A_DMA],
-                                             const half_t *const (&b_src)[Cfg::B_DMA], int K, int rows) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-    const int KT = K / Cfg::BK;
-    int live_m = (rows - wm * Cfg::WTM + 15) / 16;       // 16-row blocks of this wavefront with real rows
-    live_m = live_m < 0 ? 0 : (live_m > TM ? TM : live_m);
-    live_m = __builtin_amdgcn_readfirstlane(live_m);
-    // lane l of a 16x16x32 operand: row l%16, K elements 8*(l/16) .. +7 of the substep's 32
-    int a_off[2], b_off[2];
-    {
-      const int ra = wm * Cfg::WTM + (lane & 15);
-      const int rb = wn * Cfg::WTN + (lane & 15);
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
-        const int c = sub * 4 + (lane >> 4);
-        a_off[sub] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
-        b_off[sub] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
-      }
+  // `steps` consecutive K-tile steps starting in ring phase `phase` (updated).
+  // Step i loads the K tile at element offset min(k2_first + i*BK, k2_max).
+  template <bool FULL>
+  static __device__ __forceinline__ void k_range(half8 (&a)[2][TM], half8 (&b)[2][TN],
+                                                 const half_t *const (&a_src)[Cfg::A_DMA],
+                                                 const half_t *const (&b_src)[Cfg::B_DMA], const int (&a_off)[2],
+                                                 const int (&b_off)[2], int steps, int k2_first, int k2_max,
+                                                 int &phase, int wave, int live_m) {
+    int ph = phase;
+    int k2 = k2_first;
+    for (int i = 0; i < steps; ++i) {
+      step<FULL>(a, b, a_src, b_src, a_off, b_off, k2 < k2_max ? k2 : k2_max, ph, wave, live_m);
+      k2 += Cfg::BK;
+      ph = ph == NSLOT - 1 ? 0 : ph + 1;
     }
-    // Prologue: A(0) -> slot 0, B(0) -> slot 1, A(1) -> slot 2, B(1) -> slot 3.
+    phase = ph;
+  }
+
+  // Byte offsets in a slot of this lane's operand chunk of row block 0, per K half:
+  // lane l of a 16x16x32 operand holds row l%16, K elements 8*(l/16) .. +7 of the 32.
+  static __device__ __forceinline__ void frag_offsets(int (&a_off)[2], int (&b_off)[2]) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int ra = (wave / Cfg::WN) * Cfg::WTM + (lane & 15);
+    const int rb = (wave % Cfg::WN) * Cfg::WTN + (lane & 15);
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      const int c = sub * 4 + (lane >> 4);
+      a_off[sub] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
+      b_off[sub] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
+    }
+  }
+
+  // 16-row blocks of this wavefront that hold real rows of an M tile with `rows` rows.
+  static __device__ __forceinline__ int live_blocks(int rows) {
+    const int wm = (threadIdx.x >> 6) / Cfg::WN;
+    int live_m = (rows - wm * Cfg::WTM + 15) / 16;
+    live_m = live_m < 0 ? 0 : (live_m > TM ? TM : live_m);
+    return __builtin_amdgcn_readfirstlane(live_m);
+  }
+
+  // Phase 0: A(0) -> slot 0, B(0) -> slot 1, A(1) -> slot 2, B(1) -> slot 3, then
+  // the fragments of K half 0 of tile 0 into a[0], b[0].
+  static __device__ __forceinline__ void prologue(half8 (&a)[2][TM], half8 (&b)[2][TN],
+                                                  const half_t *const (&a_src)[Cfg::A_DMA],
+                                                  const half_t *const (&b_src)[Cfg::B_DMA], int KT,
+                                                  const int (&a_off)[2], const int (&b_off)[2], int wave) {
     const int k1 = (KT > 1 ? 1 : 0) * Cfg::BK;
-    issue_all<0>(a_src, 0, wave);
-    issue_all<1>(b_src, 0, wave);
-    issue_all<2>(a_src, k1, wave);
-    issue_all<3>(b_src, k1, wave);
+    issue_all(a_src, 0, 0 * SLOT_BYTES, wave);
+    issue_all(b_src, 0, 1 * SLOT_BYTES, wave);
+    issue_all(a_src, k1, 2 * SLOT_BYTES, wave);
+    issue_all(b_src, k1, 3 * SLOT_BYTES, wave);
     wait_vmcnt<Cfg::A_DMA + Cfg::B_DMA>();
     block_barrier();
+    const uint32_t ra = lds_addr() + a_off[0], rb = lds_addr() + SLOT_BYTES + b_off[0];
+    static_for<0, FRAGS>([&](auto I) { read_frag<I.value>(a[0], b[0], ra, rb); });
+  }
+
+  // rows: real rows of this M tile (1..BM).
+  static __device__ __forceinline__ void run(const half_t *const (&a_src)[Cfg::A_DMA],
+                                             const half_t *const (&b_src)[Cfg::B_DMA], int K, int rows) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int KT = K / Cfg::BK;
+    const int live_m = live_blocks(rows);
+    int a_off[2], b_off[2];
+    frag_offsets(a_off, b_off);
     half8 a[2][TM], b[2][TN];
-    static_for<0, FRAGS>([&](auto I) { read_frag<0, 1, 0, I.value>(a[0], b[0], a_off, b_off); });
+    prologue(a, b, a_src, b_src, KT, a_off, b_off, wave);
+    int phase = 0;
+    reserve();
+    zero_acc();
+    acc_settle();
+    // past the end of K the last K tile is fetched again into slots nobody reads
     if (live_m == TM) {
-      for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
-        static_for<0, NSLOT>([&](auto U) {
-          Step<U.value, true>::run(acc, a, b, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave, live_m);
-        });
-      }
+      k_range<true>(a, b, a_src, b_src, a_off, b_off, KT, 2 * Cfg::BK, (KT - 1) * Cfg::BK, phase, wave, live_m);
     } else {
-      for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
-        static_for<0, NSLOT>([&](auto U) {
-          Step<U.value, false>::run(acc, a, b, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave, live_m);
-        });
-      }
+      k_range<false>(a, b, a_src, b_src, a_off, b_off, KT, 2 * Cfg::BK, (KT - 1) * Cfg::BK, phase, wave, live_m);
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     wait_vmcnt<0>();
+    acc_settle();
   }
 };
 
@@ -760,13 +860,13 @@ struct Ring16Mainloop {
 //   row = wm*WTM + tm*16 + lane%16
 //   col = wn*WTN + tn*16 + 4*(lane/16) + r
 template <class Cfg>
-__device__ __forceinline__ int acc16_row(int tm) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+__device__ __forceinline__ int acc16_row(int tm, int tid) {
+  const int wave = tid >> 6, lane = tid & 63;
   return (wave / Cfg::WN) * Cfg::WTM + tm * 16 + (lane & 15);
 }
 template <class Cfg>
-__device__ __forceinline__ int acc16_col4(int tn) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+__device__ __forceinline__ int acc16_col4(int tn, int tid) {
+  const int wave = tid >> 6, lane = tid & 63;
   return (wave % Cfg::WN) * Cfg::WTN + tn * 16 + 4 * (lane >> 4);
 }
 

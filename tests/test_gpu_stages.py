@@ -162,7 +162,7 @@ def _ffn_case(R, d, f, E, seed, skew=False):
     return x, w1, b1, w2, b2, e_of_row
 
 
-@pytest.mark.parametrize("variant", list(range(6)))
+@pytest.mark.parametrize("variant", list(range(7)))
 @pytest.mark.parametrize("R,d,f,E,skew,seed", [
     (512, 256, 1024, 4, False, 0),
     (700, 768, 3072, 32, True, 1),
