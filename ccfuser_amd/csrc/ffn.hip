@@ -145,22 +145,29 @@ struct GroupedArgs {
   int N, K;
 };
 
-// erf-form GELU, 0.5*v*(1+erf(v/sqrt2)), with erf from Abramowitz-Stegun 7.1.26
-// (|error| <= 1.5e-7, far below one fp16 ulp of the result):
-//   erf(z) = 1 - (a1 t + .. + a5 t^5) exp(-z^2),  t = 1/(1 + p z),  z >= 0
-// and 0.5*v*(1 + sign(v) erf(|z|)) = 0.5*(v + |v| erf(|z|)).  About 14
-// instructions instead of the library erff's ~40.
+// erf-form GELU, 0.5*v*(1+erf(v/sqrt2)) = 0.5*(v + |v| erf(|z|)), z = v/sqrt2.
+// erf(|z|) is an odd minimax polynomial z*Q(z^2) (degree 8 in z^2, fitted on
+// [0, 3]; beyond 3, where 1 - erf < 2.3e-5, z is clamped and the result capped
+// at 1).  Measured in fp32 against the exact function over [-8, 8]: erf within
+// 2.8e-5, GELU within 5.7e-5 absolute, an eighth of the fp16 rounding step of
+// a result of magnitude 1.  15 full-rate instructions and no transcendental
+// (the library erff is ~40, the exp-based form 15 plus rcp and exp at quarter
+// rate); the FFN1 epilogue applies it to 256 values per lane and tile.
 __device__ __forceinline__ float gelu_erf(float v) {
-  const float az = fabsf(v) * 0.70710678118654752440f;
-  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, az, 1.0f));
-  float poly = fmaf(1.061405429f, t, -1.453152027f);
-  poly = fmaf(poly, t, 1.421413741f);
-  poly = fmaf(poly, t, -0.284496736f);
-  poly = fmaf(poly, t, 0.254829592f);
-  poly *= t;
-  const float ex = __builtin_amdgcn_exp2f(-1.4426950408889634f * az * az);
-  const float erf_abs = fmaf(-poly, ex, 1.0f);
-  return 0.5f * fmaf(fabsf(v), erf_abs, v);
+  const float az = fminf(fabsf(v) * 0.70710678118654752440f, 3.0f);
+  const float t = az * az;
+  float q = 4.0742129669979477e-08f;
+  q = fmaf(q, t, -1.944823679878027e-06f);
+  q = fmaf(q, t, 4.106053529540077e-05f);
+  q = fmaf(q, t, -0.000511036952957511f);
+  q = fmaf(q, t, 0.00423542782664299f);
+  q = fmaf(q, t, -0.02510286308825016f);
+  q = fmaf(q, t, 0.11107933521270752f);
+  q = fmaf(q, t, -0.375314861536026f);
+  q = fmaf(q, t, 1.1282684803009033f);
+  const float erf_abs = fminf(q * az, 1.0f);
+  const float hv = 0.5f * v;
+  return fmaf(fabsf(hv), erf_abs, hv);
 }
 
 // Global source of every tile load of this lane for the tile of plan entry

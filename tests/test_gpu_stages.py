@@ -220,6 +220,16 @@ def test_ffn_special_cases():
     y = torch.zeros(R, d, dtype=torch.float16, device="cuda")
     ops.ffn2(h, None, off, R, dev(w2), dev(b2), y)
     assert torch.equal(y.cpu(), b2.expand(R, d))
+    # the GELU itself over [-8, 8] (zero weights: h = gelu(b1)); every fp16 value of the
+    # sweep within one fp16 rounding step of the exact erf form
+    f2 = 4096
+    sweep = torch.linspace(-8.0, 8.0, f2).half().reshape(1, f2)
+    h2 = ops.ffn1(dev(x), None, off, R, dev(torch.zeros(1, f2, d).half()), dev(sweep), gelu=True)
+    exact = O.gelu_exact(sweep.float()).reshape(-1)
+    got = h2[0].cpu().float()
+    step = torch.maximum(exact.abs() * 2.0 ** -10, torch.tensor(6.2e-5))
+    assert bool(((got - exact).abs() <= step).all()), float(((got - exact).abs() / step).max())
+    assert torch.equal(h2[0], h2[R - 1])
     # pre-activation output
     w1 = (torch.randn(1, f, d, generator=g) * 0.05).half()
     pre = ops.ffn1(dev(x), None, off, R, dev(w1), dev(b1), gelu=False)
