@@ -140,7 +140,7 @@ struct GroupedArgs {
   const half_t *bias;       // [E, N]
   half_t *C;                // [*, N]
   const int32_t *c_rows;    // row of C for sorted row j, or NULL (identity)
-  const half_t *row_scale;  // [rows] or NULL
+  const half_t *row_scale;  // [rows] or NULL; NULL with the GELU epilogue
   const int32_t *plan;
   int N, K;
 };
@@ -149,25 +149,27 @@ struct GroupedArgs {
 // erf(|z|) is an odd minimax polynomial z*Q(z^2) (degree 8 in z^2, fitted on
 // [0, 3]; beyond 3, where 1 - erf < 2.3e-5, z is clamped and the result capped
 // at 1).  Measured in fp32 against the exact function over [-8, 8]: erf within
-// 2.8e-5, GELU within 5.7e-5 absolute, an eighth of the fp16 rounding step of
-// a result of magnitude 1.  15 full-rate instructions and no transcendental
+// 2.8e-5, GELU within 6.2e-5 absolute, an eighth of the fp16 rounding step of
+// a result of magnitude 1.  14 full-rate instructions and no transcendental
 // (the library erff is ~40, the exp-based form 15 plus rcp and exp at quarter
 // rate); the FFN1 epilogue applies it to 256 values per lane and tile.
 __device__ __forceinline__ float gelu_erf(float v) {
-  const float az = fminf(fabsf(v) * 0.70710678118654752440f, 3.0f);
-  const float t = az * az;
-  float q = 4.0742129669979477e-08f;
-  q = fmaf(q, t, -1.944823679878027e-06f);
-  q = fmaf(q, t, 4.106053529540077e-05f);
-  q = fmaf(q, t, -0.000511036952957511f);
-  q = fmaf(q, t, 0.00423542782664299f);
-  q = fmaf(q, t, -0.02510286308825016f);
-  q = fmaf(q, t, 0.11107933521270752f);
-  q = fmaf(q, t, -0.375314861536026f);
-  q = fmaf(q, t, 1.1282684803009033f);
-  const float erf_abs = fminf(q * az, 1.0f);
-  const float hv = 0.5f * v;
-  return fmaf(fabsf(hv), erf_abs, hv);
+  // u = |v| clamped at 3*sqrt2; the 1/sqrt2 of z = u/sqrt2 is folded into the coefficients:
+  // erf(z) = u * Q'(u^2) with c'_k = c_k / sqrt2^(2k+1)
+  const float u = fminf(fabsf(v), 4.2426406871192851464f);
+  const float t = u * u;
+  float q = 1.1253530e-10f * 0.5f;                 // 0.5 * c'_8 .. the 0.5 of GELU is folded in too
+  q = fmaf(q, t, -1.0743734e-08f * 0.5f);
+  q = fmaf(q, t, 4.5365911e-07f * 0.5f);
+  q = fmaf(q, t, -1.1292428e-05f * 0.5f);
+  q = fmaf(q, t, 1.8718123e-04f * 0.5f);
+  q = fmaf(q, t, -2.2188006e-03f * 0.5f);
+  q = fmaf(q, t, 1.9636238e-02f * 0.5f);
+  q = fmaf(q, t, -1.3269384e-01f * 0.5f);
+  q = fmaf(q, t, 7.9780629e-01f * 0.5f);
+  const float half_erf = fminf(q * u, 0.5f);       // 0.5 * erf(|z|)
+  // 0.5*v + |v| * 0.5*erf(|z|)
+  return fmaf(fabsf(v), half_erf, 0.5f * v);
 }
 
 // Global source of every tile load of this lane for the tile of plan entry
@@ -236,8 +238,9 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           float x = v[tn][c] + bias_v[tn][c];
-          if (kGelu) x = gelu_erf(x);
-          o[c] = static_cast<half_t>(x * sc);
+          if (kGelu) x = gelu_erf(x);                 // FFN1: no row scale
+          else x *= sc;
+          o[c] = static_cast<half_t>(x);
         }
         if (col[tn] < p.N) *reinterpret_cast<half4 *>(dst + col[tn]) = o;
       }
@@ -405,7 +408,7 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       // sources of the next tile (tile_sources() with the row indices already at hand); the
       // empty asm keeps the compiler from computing them before the loop above and holding
       // 16 more registers across it
-      int n_e = nent[0], n_tn = nent[3];
+      int n_e = __builtin_amdgcn_readfirstlane(nent[0]), n_tn = __builtin_amdgcn_readfirstlane(nent[3]);
       asm volatile("" : "+s"(n_e), "+s"(n_tn));
       const half_t *Be = p.B + static_cast<size_t>(n_e) * p.N * p.K;
       const int n0 = n_tn * Cfg::BN;
@@ -510,6 +513,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   CCF_REQUIRE(N % 8 == 0, CCF_ERR_SHAPE, "%s: N=%d is not a multiple of 8", what, N);
   CCF_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C) && aligned16(bias), CCF_ERR_ARG,
               "%s: operands must be 16-byte aligned", what);
+  CCF_REQUIRE(!(gelu && row_scale), CCF_ERR_ARG, "%s: the GELU epilogue takes no row scale", what);
   if (max_rows == 0) return CCF_OK;
   const Launch &v = kVariants[g_variant];
   const int max_tiles = max_tiles_for(max_rows, E, v.bm);
