@@ -39,6 +39,9 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 
+// tuning knobs set through ccf_set_option()
+extern int g_gate_waves;   // gate.hip
+
 }  // namespace ccf
 
 #define CCF_REQUIRE(cond, code, ...)                 \

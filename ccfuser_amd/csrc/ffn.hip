@@ -558,6 +558,11 @@ extern "C" int ccf_set_option(const char *name, int value) {
     g_variant = value < 0 ? kDefaultVariant : value;     // -1: back to the default
     return CCF_OK;
   }
+  if (!strcmp(name, "gate_waves")) {
+    CCF_REQUIRE(value == 4 || value == 16, CCF_ERR_ARG, "set_option: gate_waves %d is neither 4 nor 16", value);
+    g_gate_waves = value;
+    return CCF_OK;
+  }
   return fail(CCF_ERR_ARG, "set_option: unknown option %s", name);
 }
 

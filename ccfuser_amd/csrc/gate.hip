@@ -19,6 +19,7 @@
 #include <limits.h>
 
 namespace ccf {
+int g_gate_waves = 16;   // wavefronts per gate workgroup when the weights sit in LDS; 4 forces the small one
 namespace {
 
 constexpr int kMaxTopK = 8;
@@ -107,20 +108,20 @@ __device__ inline void fold_lanes(float (&v)[N], int lane) {
 // d_model <= 4096).  Logits of all experts are parked in LDS until the last
 // expert group is done, then each wavefront picks the top-k of its tokens.
 // None of this changes the order of the additions.
-template <typename T, int TT, bool kWLds>
-__global__ void __launch_bounds__(256)
+template <typename T, int TT, bool kWLds, int GW>
+__global__ void __launch_bounds__(GW * 64)
 gate_kernel(const T *__restrict__ x, const T *__restrict__ wg, const T *__restrict__ bg,
             int tokens, int d, int E, int k, int groups_per_block, int64_t *__restrict__ idx_out,
             T *__restrict__ score_out, T *__restrict__ logits_out) {
 #pragma clang fp contract(off)
   constexpr int kBatch = 8 / TT;                   // x chunks requested together per lane
-  extern __shared__ float s_logit[];               // [groups_per_block][4 waves][TT][E], then weights
+  extern __shared__ float s_logit[];               // [groups_per_block][GW wavefronts][TT][E], then weights
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   const int nchunk = d >> 3;
   const int niter = (nchunk + kWave - 1) / kWave;
-  const int n_groups = (tokens + 4 * TT - 1) / (4 * TT);
-  T *w_lds = reinterpret_cast<T *>(s_logit + static_cast<size_t>(groups_per_block) * 4 * TT * E);
+  const int n_groups = (tokens + GW * TT - 1) / (GW * TT);
+  T *w_lds = reinterpret_cast<T *>(s_logit + static_cast<size_t>(groups_per_block) * GW * TT * E);
 
   for (int e0 = 0; e0 < E; e0 += kGateEG) {
     const int ng = (E - e0) < kGateEG ? (E - e0) : kGateEG;
@@ -131,11 +132,11 @@ gate_kernel(const T *__restrict__ x, const T *__restrict__ wg, const T *__restri
       const int per_row = static_cast<int>(static_cast<size_t>(d) * sizeof(T) / 16);
       const int total = kGateEG * per_row;
       int4v *dst = reinterpret_cast<int4v *>(w_lds);
-      for (int i0 = threadIdx.x; i0 < total; i0 += 256 * 8) {
+      for (int i0 = threadIdx.x; i0 < total; i0 += GW * 64 * 8) {
         int4v tmp[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-          const int i = i0 + u * 256;
+          const int i = i0 + u * GW * 64;
           if (i < total) {
             int row = e0 + i / per_row;
             row = row < E ? row : E - 1;
@@ -144,7 +145,7 @@ gate_kernel(const T *__restrict__ x, const T *__restrict__ wg, const T *__restri
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u)
-          if (i0 + u * 256 < total) dst[i0 + u * 256] = tmp[u];
+          if (i0 + u * GW * 64 < total) dst[i0 + u * GW * 64] = tmp[u];
       }
       __syncthreads();
     }
@@ -153,8 +154,8 @@ gate_kernel(const T *__restrict__ x, const T *__restrict__ wg, const T *__restri
     for (int gi = 0; gi < groups_per_block; ++gi) {
       const int grp = blockIdx.x + gi * gridDim.x;
       if (grp >= n_groups) break;                  // uniform per workgroup
-      const int t0 = (grp * 4 + wave) * TT;
-      float *mine = s_logit + (static_cast<size_t>(gi) * 4 + wave) * TT * E;
+      const int t0 = (grp * GW + wave) * TT;
+      float *mine = s_logit + (static_cast<size_t>(gi) * GW + wave) * TT * E;
       const T *xrow[TT];
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) {
@@ -227,8 +228,8 @@ gate_kernel(const T *__restrict__ x, const T *__restrict__ wg, const T *__restri
   for (int gi = 0; gi < groups_per_block; ++gi) {
     const int grp = blockIdx.x + gi * gridDim.x;
     if (grp >= n_groups) break;
-    const int t0 = (grp * 4 + wave) * TT;
-    const float *mine = s_logit + (static_cast<size_t>(gi) * 4 + wave) * TT * E;
+    const int t0 = (grp * GW + wave) * TT;
+    const float *mine = s_logit + (static_cast<size_t>(gi) * GW + wave) * TT * E;
 #pragma unroll 1
     for (int tt = 0; tt < TT; ++tt) {
       const int t = t0 + tt;
@@ -317,17 +318,26 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
   const size_t esz = dtype == CCF_F16 ? 2 : 4;
   const size_t w_bytes = static_cast<size_t>(group) * d_model * esz;
   const bool w_lds = w_bytes <= 65536;             // one expert group of weights fits next to the logits
-  const int n_groups = (tokens + 4 * tt - 1) / (4 * tt);
-  const int max_blocks = 512;                      // two persistent workgroups per CU
-  const int blocks = n_groups < max_blocks ? n_groups : max_blocks;
-  const int groups_per_block = (n_groups + blocks - 1) / blocks;
-  dim3 grid(blocks), block(256);
-  const size_t lds = sizeof(float) * 4 * tt * static_cast<size_t>(tot_expert) * groups_per_block +
-                     (w_lds ? w_bytes : 0);
+  // Wavefronts per workgroup: 16 (one workgroup per CU stages the weights once for 16
+  // wavefronts) when the weights sit in LDS, else 4 (two workgroups per CU).
+  const int gw = (w_lds && g_gate_waves != 4) ? 16 : 4;
+  const int n_groups = (tokens + gw * tt - 1) / (gw * tt);
+  const int max_blocks = gw == 16 ? 256 : 512;     // persistent workgroups
+  int blocks = n_groups < max_blocks ? n_groups : max_blocks;
+  int groups_per_block = (n_groups + blocks - 1) / blocks;
+  // the logits of a workgroup's tokens wait in LDS: more workgroups when they would not fit
+  const size_t per_group = sizeof(float) * gw * tt * static_cast<size_t>(tot_expert);
+  const size_t lds_budget = 160 * 1024 - (w_lds ? w_bytes : 0);
+  if (per_group * groups_per_block > lds_budget && per_group <= lds_budget) {
+    groups_per_block = static_cast<int>(lds_budget / per_group);
+    blocks = (n_groups + groups_per_block - 1) / groups_per_block;
+  }
+  dim3 grid(blocks), block(gw * 64);
+  const size_t lds = per_group * groups_per_block + (w_lds ? w_bytes : 0);
   CCF_REQUIRE(lds <= 160 * 1024, CCF_ERR_SHAPE, "gate: %zu bytes of LDS needed", lds);
-#define CCF_GATE_LAUNCH(TYPE, TT, WL)                                                              \
+#define CCF_GATE_LAUNCH(TYPE, TT, WL, GWV)                                                            \
   do {                                                                                             \
-    auto kern = gate_kernel<TYPE, TT, WL>;                                                         \
+    auto kern = gate_kernel<TYPE, TT, WL, GWV>;                                                    \
     if (lds > 65536) {                                                                             \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                     \
                                          hipFuncAttributeMaxDynamicSharedMemorySize,               \
@@ -340,17 +350,20 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
                        static_cast<TYPE *>(score_out),                                             \
                        static_cast<TYPE *>(logits_out));                                           \
   } while (0)
-#define CCF_GATE_TT(TYPE, WL)                    \
-  do {                                           \
-    if (tt == 4) CCF_GATE_LAUNCH(TYPE, 4, WL);   \
-    else if (tt == 2) CCF_GATE_LAUNCH(TYPE, 2, WL); \
-    else CCF_GATE_LAUNCH(TYPE, 1, WL);           \
+#define CCF_GATE_TT(TYPE, WL, GWV)                    \
+  do {                                                \
+    if (tt == 4) CCF_GATE_LAUNCH(TYPE, 4, WL, GWV);   \
+    else if (tt == 2) CCF_GATE_LAUNCH(TYPE, 2, WL, GWV); \
+    else CCF_GATE_LAUNCH(TYPE, 1, WL, GWV);           \
   } while (0)
-  if (dtype == CCF_F16) {
-    if (w_lds) CCF_GATE_TT(half_t, true); else CCF_GATE_TT(half_t, false);
-  } else {
-    if (w_lds) CCF_GATE_TT(float, true); else CCF_GATE_TT(float, false);
-  }
+#define CCF_GATE_W(TYPE)                                              \
+  do {                                                                \
+    if (!w_lds) CCF_GATE_TT(TYPE, false, 4);                          \
+    else if (gw == 16) CCF_GATE_TT(TYPE, true, 16);                   \
+    else CCF_GATE_TT(TYPE, true, 4);                                  \
+  } while (0)
+  if (dtype == CCF_F16) CCF_GATE_W(half_t); else CCF_GATE_W(float);
+#undef CCF_GATE_W
 #undef CCF_GATE_TT
 #undef CCF_GATE_LAUNCH
   return check_launch("gate_kernel");

@@ -48,6 +48,29 @@ def test_gate_bit_exact(T, d, E, k, dtype, seed):
     assert torch.allclose(score.float().sum(-1).cpu(), torch.ones(T), atol=2e-3)
 
 
+@pytest.mark.parametrize("waves", [4, 16])
+@pytest.mark.parametrize("T,d,E,k", [(5000, 512, 8, 2), (9000, 256, 32, 1), (40000, 128, 16, 2)])
+def test_gate_workgroup_sizes(waves, T, d, E, k):
+    """Both workgroup shapes of the gate, with several token groups per workgroup
+    and (T >= 8192, 32768) two and four tokens per wavefront."""
+    from ccfuser_amd import ops
+    _say(f"gate waves={waves} T={T} d={d} E={E} k={k}")
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, d, generator=g).half()
+    wg = (torch.randn(E, d, generator=g) * 0.05).half()
+    bg = (torch.randn(E, generator=g) * 0.05).half()
+    idx_ref, score_ref, logits_ref = O.naive_gate(x, wg, bg, k)
+    ops.set_option("gate_waves", waves)
+    try:
+        idx, score, logits = ops.gate_topk_softmax(dev(x), dev(wg), dev(bg), k, return_logits=True)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_option("gate_waves", 16)
+    assert torch.equal(logits.cpu(), logits_ref), "logits differ bitwise"
+    assert torch.equal(idx.cpu(), idx_ref), "expert choice differs"
+    assert (score.cpu().float() - score_ref.float()).abs().max() <= 1e-3
+
+
 def test_gate_ties_go_to_lower_expert():
     from ccfuser_amd import ops
     x = torch.ones(8, 64, dtype=torch.float16)
