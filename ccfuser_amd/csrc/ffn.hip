@@ -452,7 +452,7 @@ using Cfg1 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 3>;   // 4 wavefronts of 128x1
 using Cfg2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 0>;   // 8 wavefronts, two whole-tile stages
 using Cfg3 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 1>;   // 8 wavefronts, BK=32 x 4 stages, ping-pong
 using Cfg4 = GemmCfg<256, 128, 32, 2, 2, 3, 2, 2, 0>;   // 4 wavefronts, 72 KB LDS: two workgroups per CU
-using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 4>;   // 4 wavefronts of 128x128, 16x16x32 MFMA, mid-tile barrier
+using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 8, 4>;   // 4 wavefronts of 128x128, 16x16x32 MFMA, mid-tile barrier
 // variant 6: Cfg5 again, persistent workgroups
 
 constexpr int kDefaultVariant = 6;
