@@ -155,6 +155,9 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
               "moe_forward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   if (tokens == 0) return CCF_OK;
   MoeWs w = carve_moe(workspace, tokens, d_model, d_ffn, num_expert, top_k);
+  // counts and offsets are written straight into the caller's arrays when given
+  if (counts_out) w.counts = counts_out;
+  if (offsets_out) w.offsets = offsets_out;
   const int n = tokens * top_k;
   hipStream_t st = as_stream(stream);
   int rc;
@@ -186,11 +189,6 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
     e = hipMemcpyAsync(score_out, w.score, sizeof(half_t) * n, hipMemcpyDeviceToDevice, st);
   if (pos_out && e == hipSuccess)
     e = hipMemcpyAsync(pos_out, w.pos, sizeof(int64_t) * n, hipMemcpyDeviceToDevice, st);
-  if (counts_out && e == hipSuccess)
-    e = hipMemcpyAsync(counts_out, w.counts, sizeof(int32_t) * num_expert, hipMemcpyDeviceToDevice, st);
-  if (offsets_out && e == hipSuccess)
-    e = hipMemcpyAsync(offsets_out, w.offsets, sizeof(int32_t) * (num_expert + 1),
-                       hipMemcpyDeviceToDevice, st);
   if (e != hipSuccess) return fail(CCF_ERR_HIP, "moe_forward: copy failed: %s", hipGetErrorString(e));
   return CCF_OK;
 }
