@@ -6,10 +6,12 @@ been built, or a call fails, the caller gets an exception.
 from __future__ import annotations
 
 import ctypes as C
+import os
 from pathlib import Path
 from typing import Optional
 
-LIB_PATH = Path(__file__).resolve().parent / "libccfuser_moe.so"
+# CCFUSER_MOE_LIB overrides the path (to compare two builds in one process launch each)
+LIB_PATH = Path(os.environ.get("CCFUSER_MOE_LIB") or Path(__file__).resolve().parent / "libccfuser_moe.so")
 
 _lib: Optional[C.CDLL] = None
 
