@@ -35,9 +35,28 @@ __host__ __device__ inline long long launched_wgs(int max_tiles, int n_tiles_n) 
 
 constexpr int kOrderGroupM = 8;
 
-// Tiles come in two classes.  A "long" M tile holds more than BM/2 rows and
-// takes a full tile's time; a "short" one (an expert's last tile with at most
-// BM/2 rows) skips most of its MFMAs and ends early.  Workgroups that share an
+// Rows of M tile i of an expert with cnt rows in nt = ceil(cnt / BM) tiles.  When
+// the last tile would hold at most BM/2 rows, it and the one before it share
+// their rows evenly instead: a nearly empty tile still streams a whole weight
+// panel, on its own and from HBM (its siblings have long passed), which costs
+// about as much as a full tile; two half-full tiles run in step with their
+// siblings, share the panel in L2, and skip half of their MFMAs.
+__device__ inline void tile_rows(int cnt, int nt, int i, int BM, int &first_row, int &rows) {
+  const int last = cnt - (nt - 1) * BM;
+  if (nt >= 2 && last <= BM / 2 && i >= nt - 2) {
+    const int both = BM + last;
+    const int h = (both + 1) / 2;
+    first_row = (nt - 2) * BM + (i == nt - 2 ? 0 : h);
+    rows = i == nt - 2 ? h : both - h;
+  } else {
+    first_row = i * BM;
+    rows = (cnt - i * BM) < BM ? (cnt - i * BM) : BM;
+  }
+}
+
+// Tiles come in two classes.  A "long" M tile holds more than BM/2 rows; a
+// "short" one is the only tile of an expert with at most BM/2 rows, skips most
+// of its MFMAs and ends early.  Workgroups that share an
 // XCD share weight and token tiles through its L2 only while they walk K in
 // step, and a workgroup that ends early puts every later one on its CU out of
 // step, so all long tiles are launched first and the short ones after them,
@@ -61,7 +80,7 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
       int cnt = e < E ? s_off[e + 1] - s_off[e] : 0;
       cnt = cnt > 0 ? cnt : 0;
       const int nt = (cnt + BM - 1) / BM;
-      const int ns = (nt > 0 && cnt - (nt - 1) * BM <= BM / 2) ? 1 : 0;
+      const int ns = (nt == 1 && cnt <= BM / 2) ? 1 : 0;        // a short tile only when it is the expert's only one
       const int nl = nt - ns;
       int inc_l = nl, inc_s = ns;
 #pragma unroll
@@ -114,8 +133,9 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
       const int tn = in_run / run_size;
       const long long logical = first + l;
       const long long b = (logical % per_long) * 8 + logical / per_long;   // hardware id
-      const int rows = (cnt - i * BM) < BM ? (cnt - i * BM) : BM;
-      if (b < wgs) entry[b] = int4v{e, lo + i * BM, rows, tn};
+      int first_row, rows;
+      tile_rows(cnt, nl, i, BM, first_row, rows);
+      if (b < wgs) entry[b] = int4v{e, lo + first_row, rows, tn};
     }
     if (ns) {
       const int i = nl;                                          // the expert's last M tile
@@ -172,6 +192,19 @@ __device__ __forceinline__ float gelu_erf(float v) {
   return fmaf(fabsf(v), half_erf, 0.5f * v);
 }
 
+// Row of the tile's row range [0, rows) that tile row r (0 .. BM-1) holds; padded
+// tile rows repeat a real one.  The 16x16x32 kernels give the upper and the
+// lower half of the tile (one row of wavefronts each) half of the rows each,
+// so that a partly filled tile skips MFMAs in both; the others fill from the top.
+template <class Cfg>
+__device__ __forceinline__ int tile_row_to_local(int r, int rows) {
+  if constexpr (Cfg::SCHED == 4) {
+    return Ring16Mainloop<Cfg>::local_row(r, rows);
+  } else {
+    return r < rows ? r : rows - 1;
+  }
+}
+
 // Global source of every tile load of this lane for the tile of plan entry
 // `ent`: K element 0 of the (clamped) A row and B row, at this lane's K chunk.
 // Padded A rows re-read the tile's last real row, B rows past N the last row.
@@ -185,7 +218,7 @@ __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v e
 #pragma unroll
   for (int i = 0; i < Cfg::A_DMA; ++i) {
     const int r = ML::dma_row(i);
-    const int rc = r < rows ? r : rows - 1;
+    const int rc = tile_row_to_local<Cfg>(r, rows);
     const int g = p.a_rows ? p.a_rows[row0 + rc] : row0 + rc;
     a_src[i] = p.A + static_cast<size_t>(g) * p.K + ML::dma_chunk(r) * 8;
   }
@@ -217,7 +250,9 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
   }
   static_for<0, TM>([&](auto T) {
     constexpr int tm = T.value;
-    const int lr = acc16_row<Cfg>(tm, tid);
+    const int tr = acc16_row<Cfg>(tm, tid);               // tile row
+    const bool real = R::row_is_real(tr, rows);
+    const int lr = R::local_row(tr, rows);
     // the accumulator reads are unconditional (they are asm the compiler must not skip per lane)
     float v[TN][4];
     static_for<0, TN>([&](auto J) {
@@ -227,7 +262,7 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
       v[tn][2] = R::template acc_get<tm, tn, 2>();
       v[tn][3] = R::template acc_get<tm, tn, 3>();
     });
-    if (lr < rows) {
+    if (real) {
       const int j = row0 + lr;
       const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
       const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
@@ -388,7 +423,7 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
 #pragma unroll
     for (int i = 0; i < Cfg::A_DMA; ++i) {
       const int r = ML::dma_row(i, tid0);
-      const int rc = r < n_rows ? r : n_rows - 1;
+      const int rc = R::local_row(r, n_rows);
       if (p.a_rows) {
         const int32_t *src = p.a_rows + n_row0 + rc;
         asm volatile("global_load_dword %0, %1, off" : "=v"(next_row[i]) : "v"(src) : "memory");

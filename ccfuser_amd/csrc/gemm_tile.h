@@ -808,11 +808,26 @@ struct Ring16Mainloop {
     }
   }
 
+  // The tile's rows [0, rows) are split between the two rows of wavefronts: the
+  // first (rows+1)/2 sit in tile rows 0 .., the rest in tile rows WTM .., so a
+  // partly filled tile has padding, and skips MFMAs, in both halves.
+  static_assert(Cfg::WM == 2, "row split written for two rows of wavefronts");
+  static __device__ __forceinline__ int local_row(int r, int rows) {
+    const int h0 = (rows + 1) >> 1, h1 = rows - h0;
+    const int q = r - Cfg::WTM;
+    return r < Cfg::WTM ? (r < h0 ? r : h0 - 1) : (q < h1 ? h0 + q : rows - 1);
+  }
+  static __device__ __forceinline__ bool row_is_real(int r, int rows) {
+    const int h0 = (rows + 1) >> 1, h1 = rows - h0;
+    return r < Cfg::WTM ? r < h0 : r - Cfg::WTM < h1;
+  }
   // 16-row blocks of this wavefront that hold real rows of an M tile with `rows` rows.
   static __device__ __forceinline__ int live_blocks(int rows) {
     const int wm = (threadIdx.x >> 6) / Cfg::WN;
-    int live_m = (rows - wm * Cfg::WTM + 15) / 16;
-    live_m = live_m < 0 ? 0 : (live_m > TM ? TM : live_m);
+    const int h0 = (rows + 1) >> 1;
+    const int mine = wm == 0 ? h0 : rows - h0;
+    int live_m = (mine + 15) / 16;
+    live_m = live_m > TM ? TM : live_m;
     return __builtin_amdgcn_readfirstlane(live_m);
   }
 
