@@ -279,6 +279,90 @@ int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capaci
   return check_launch("pos_kernel");
 }
 
+// Block plan in the reference's wire format (AsyncExpertAssignment.divide_into_block,
+// mix_moe/mix_moe/transformer.py:150-250, at world_size 1 with the identity expert
+// plan): per expert the full block_size-row blocks form the "local" list and a
+// shorter tail the "remote" list, both in expert order; the lists are interleaved
+// l0, r0, l1, r1, ... (transformer.py:199).  Closed form of the interleave: local
+// item i sits at 2i while i < nR, else at nR + i; remote item i at 2i + 1 while
+// i < nL, else at nL + i.  expert_block_ids / expert_block_id_idxs are the CSR from
+// expert to its blocks in plan order (transformer.py:213-219).
+// One workgroup; one thread per expert for the scans, then one per block.
+__global__ void __launch_bounds__(1024)
+blocks_kernel(const int32_t *__restrict__ counts, int E, int bs, int rank, int max_blocks,
+              int32_t *__restrict__ expert_ids, int32_t *__restrict__ ranks,
+              int32_t *__restrict__ lens, int32_t *__restrict__ start_addrs,
+              int32_t *__restrict__ expert_block_ids, int32_t *__restrict__ expert_block_id_idxs,
+              int32_t *__restrict__ block_nums) {
+  __shared__ int s_start[kMaxExpert + 1], s_full[kMaxExpert + 1], s_tail[kMaxExpert + 1];
+  const int t = threadIdx.x;
+  const int c = t < E ? counts[t] : 0;
+  // inclusive scans of rows, full blocks and tails, shifted by one entry
+  if (t == 0) s_start[0] = s_full[0] = s_tail[0] = 0;
+  s_start[t + 1] = c;
+  s_full[t + 1] = c / bs;
+  s_tail[t + 1] = (c % bs) != 0;
+  __syncthreads();
+  for (int d = 1; d < kMaxExpert; d <<= 1) {
+    int a = 0, b = 0, g = 0;
+    if (t + 1 > d) {
+      a = s_start[t + 1 - d];
+      b = s_full[t + 1 - d];
+      g = s_tail[t + 1 - d];
+    }
+    __syncthreads();
+    s_start[t + 1] += a;
+    s_full[t + 1] += b;
+    s_tail[t + 1] += g;
+    __syncthreads();
+  }
+  const int nL = s_full[E], nR = s_tail[E];
+  auto pos_local = [&](int i) { return i < nR ? 2 * i : nR + i; };
+  auto pos_remote = [&](int i) { return i < nL ? 2 * i + 1 : nL + i; };
+  if (t == 0) {
+    block_nums[0] = nL + nR;
+    block_nums[1] = nR;
+    expert_block_id_idxs[E] = nL + nR;
+  }
+  if (t < E) expert_block_id_idxs[t] = s_full[t] + s_tail[t];
+  // full blocks
+  for (int i = t; i < nL; i += 1024) {
+    int lo = 0, hi = E;                     // expert e with s_full[e] <= i < s_full[e + 1]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_full[mid] <= i) lo = mid; else hi = mid;
+    }
+    const int e = lo, b = i - s_full[e], p = pos_local(i);
+    const bool has_tail = s_tail[e + 1] != s_tail[e];
+    const int before = (has_tail && pos_remote(s_tail[e]) < p) ? 1 : 0;
+    if (p < max_blocks) {
+      expert_ids[p] = e;
+      ranks[p] = rank;
+      lens[p] = bs;
+      start_addrs[p] = s_start[e] + b * bs;
+    }
+    const int slot = s_full[e] + s_tail[e] + b + before;
+    if (slot < max_blocks) expert_block_ids[slot] = p;
+  }
+  // tails
+  if (t < E && (c % bs) != 0) {
+    const int e = t, p = pos_remote(s_tail[e]), nfull = c / bs;
+    int lo = 0, hi = nfull;                 // full blocks of e planned before the tail
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (pos_local(s_full[e] + mid) < p) lo = mid + 1; else hi = mid;
+    }
+    if (p < max_blocks) {
+      expert_ids[p] = e;
+      ranks[p] = rank;
+      lens[p] = c % bs;
+      start_addrs[p] = s_start[e] + nfull * bs;
+    }
+    const int slot = s_full[e] + s_tail[e] + lo;
+    if (slot < max_blocks) expert_block_ids[slot] = p;
+  }
+}
+
 }  // namespace
 }  // namespace ccf
 
@@ -343,4 +427,23 @@ extern "C" int ccf_segments_to_rows(const int32_t *seg_start, const int32_t *seg
   hipLaunchKernelGGL(segments_kernel, dim3(1), dim3(1024), 0, as_stream(stream), seg_start, seg_len,
                      seg_expert, n_seg, num_expert, total_rows, counts, offsets, rows);
   return check_launch("segments_kernel");
+}
+
+extern "C" int ccf_plan_blocks(const int32_t *counts, int num_expert, int block_size, int rank,
+                               int max_blocks, int32_t *expert_ids, int32_t *ranks, int32_t *lens,
+                               int32_t *start_addrs, int32_t *expert_block_ids,
+                               int32_t *expert_block_id_idxs, int32_t *block_nums,
+                               ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(counts && expert_ids && ranks && lens && start_addrs && expert_block_ids &&
+                  expert_block_id_idxs && block_nums,
+              CCF_ERR_ARG, "plan_blocks: null pointer");
+  CCF_REQUIRE(num_expert > 0 && block_size > 0 && max_blocks >= 0, CCF_ERR_ARG,
+              "plan_blocks: bad size");
+  CCF_REQUIRE(num_expert <= kMaxExpert, CCF_ERR_SHAPE, "plan_blocks: num_expert=%d exceeds %d",
+              num_expert, kMaxExpert);
+  hipLaunchKernelGGL(blocks_kernel, dim3(1), dim3(1024), 0, as_stream(stream), counts, num_expert,
+                     block_size, rank, max_blocks, expert_ids, ranks, lens, start_addrs,
+                     expert_block_ids, expert_block_id_idxs, block_nums);
+  return check_launch("blocks_kernel");
 }

@@ -51,16 +51,20 @@ class BlockInfos(dict):
     ``inv_pos`` [tokens*top_k] and the ints ``max_rows`` / ``n_flat`` drive the
     grouped GEMMs, whose tile list is derived from ``offsets`` on the device.
     The reference's nine keys (transformer.py:242-250) are produced on first
-    access from the counts; that access synchronises the host once.
+    access by one small kernel from the counts; the arrays are then trimmed to
+    ``total_block_num`` entries, which reads two ints back (the reference's
+    ``total_block_num`` / ``remote_block_num`` are Python ints).
     """
 
     def __missing__(self, key):
         if key not in _COMPAT_KEYS:
             raise KeyError(key)
-        plan = plan_blocks(self["counts"].cpu().numpy())
-        dev = self["counts"].device
+        plan = ops.plan_blocks(self["counts"], self["n_flat"])
+        total, remote = plan.pop("block_nums").tolist()
         for k, v in plan.items():
-            self[k] = v if isinstance(v, int) else torch.tensor(v, dtype=torch.int32, device=dev)
+            self[k] = v if k == "expert_block_id_idxs" else v[:total]
+        self["local_expert_id_indexs"] = self["expert_ids"]
+        self["total_block_num"], self["remote_block_num"] = total, remote
         return dict.__getitem__(self, key)
 
 

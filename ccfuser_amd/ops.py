@@ -127,6 +127,29 @@ def route(gate_idx: torch.Tensor, num_expert: int, top_k: int, capacity: int = -
     return out
 
 
+def plan_blocks(counts: torch.Tensor, max_rows: int, block_size: int = 64, rank: int = 0) -> Dict[str, torch.Tensor]:
+    """The reference's block arrays (transformer.py:242-250) from per-expert counts,
+    on the device and without a host synchronisation.
+
+    Arrays have ``max_rows // block_size + E`` entries (an upper bound for any
+    counts summing to at most ``max_rows``); ``block_nums`` holds
+    ``{total_block_num, remote_block_num}`` and says how many are valid.
+    """
+    _check(counts, "counts", dtype=torch.int32, ndim=1)
+    E = counts.numel()
+    dev = counts.device
+    cap = int(max_rows) // int(block_size) + E
+    names = ("expert_ids", "ranks", "lens", "start_addrs", "expert_block_ids")
+    out = {k: torch.zeros(cap, dtype=torch.int32, device=dev) for k in names}
+    out["expert_block_id_idxs"] = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    out["block_nums"] = torch.empty(2, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("ccf_plan_blocks", _ptr(counts), E, int(block_size), int(rank), cap,
+                  *[_ptr(out[k]) for k in names], _ptr(out["expert_block_id_idxs"]),
+                  _ptr(out["block_nums"]), _stream(counts))
+    return out
+
+
 def segments_to_rows(seg_start, seg_len, seg_expert, num_expert: int, total_rows: int):
     for t, nm in ((seg_start, "seg_start"), (seg_len, "seg_len"), (seg_expert, "seg_expert")):
         _check(t, nm, dtype=torch.int32, ndim=1)

@@ -129,6 +129,29 @@ int ccf_route(const int64_t *gate_idx, int n_flat, int num_expert, int top_k,
               ccf_stream_t stream);
 
 /*
+ * Block plan in the reference's wire format, built on the device from the
+ * per-expert counts: what AsyncExpertAssignment.divide_into_block computes in
+ * Python loops and ships with seven blocking copies
+ * (mix_moe/mix_moe/transformer.py:150-250) at world_size 1 with the identity
+ * expert plan.  Per expert the full block_size-row blocks and a shorter tail;
+ * full blocks and tails interleaved l0, r0, l1, r1, ... (transformer.py:199).
+ * Unlike the reference an expert with fewer than block_size rows keeps its
+ * tail block (transformer.py:184-193 plans a tail only next to a full block).
+ *   counts int32 [num_expert]
+ *   expert_ids, ranks, lens, start_addrs, expert_block_ids int32 [max_blocks];
+ *     max_blocks >= sum(counts) / block_size + num_expert holds every plan,
+ *     blocks beyond max_blocks are not written; ranks[] = rank
+ *   expert_block_id_idxs int32 [num_expert + 1]  CSR expert -> expert_block_ids
+ *   block_nums int32 [2]  {total_block_num, remote_block_num (= tails)}
+ * local_expert_id_indexs of the reference equals expert_ids on one GPU.
+ */
+int ccf_plan_blocks(const int32_t *counts, int num_expert, int block_size, int rank,
+                    int max_blocks, int32_t *expert_ids, int32_t *ranks, int32_t *lens,
+                    int32_t *start_addrs, int32_t *expert_block_ids,
+                    int32_t *expert_block_id_idxs, int32_t *block_nums,
+                    ccf_stream_t stream);
+
+/*
  * Rows addressed by (start, len, expert) triples -> per-expert counts,
  * offsets and a row list grouped by expert (segment order, then row order).
  * The triple is what the reference plans per block

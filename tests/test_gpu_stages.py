@@ -133,6 +133,42 @@ def test_expert_count_and_assign_pos_mirror_the_reference_calls():
     assert torch.equal(lec_cum.cpu(), off_ref[:-1])      # cum_count ends at the segment starts
 
 
+def _count_cases():
+    import os
+    import numpy as np
+    g = torch.Generator().manual_seed(5)
+    table = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_all_expert_count.npy"))
+    cases = [row.tolist() for row in table]                       # the reference's skewed 4x64 table
+    cases += [[0, 0, 0], [63], [64], [65], [1, 64, 0, 128, 130, 5], [64] * 7, [3] * 9,
+              [700, 0, 1, 0, 64, 63, 1000],                       # more full blocks than tails
+              [1] * 40 + [128],                                   # more tails than full blocks
+              torch.randint(0, 300, (1000,), generator=g).tolist(),
+              torch.randint(0, 3, (1024,), generator=g).tolist()]
+    return cases
+
+
+@pytest.mark.parametrize("case", range(15))
+def test_plan_blocks_matches_divide_into_block(case):
+    """Device block planner against the oracle's divide_into_block, every array bit-exact."""
+    from ccfuser_amd import ops
+    counts = _count_cases()[case]
+    _say(f"plan_blocks case={case} E={len(counts)} rows={sum(counts)}")
+    ref = O.divide_into_block(counts, 64)
+    got = ops.plan_blocks(torch.tensor(counts, dtype=torch.int32, device="cuda"), sum(counts), 64)
+    total, remote = got["block_nums"].tolist()
+    assert (total, remote) == (ref["total_block_num"], ref["remote_block_num"])
+    for k in ("expert_ids", "ranks", "lens", "start_addrs", "expert_block_ids"):
+        assert got[k][:total].tolist() == ref[k], k
+        assert got[k].numel() >= total
+    assert got["expert_block_id_idxs"].tolist() == ref["expert_block_id_idxs"]
+    got32 = ops.plan_blocks(torch.tensor(counts, dtype=torch.int32, device="cuda"), sum(counts), 32, rank=3)
+    ref32 = O.divide_into_block(counts, 32)
+    t32 = int(got32["block_nums"][0])
+    assert t32 == ref32["total_block_num"]
+    assert got32["start_addrs"][:t32].tolist() == ref32["start_addrs"]
+    assert got32["ranks"][:t32].tolist() == [3] * t32
+
+
 # ------------------------------------------------- row moves and combine
 def test_local_scatter_gather_with_reference_pos_vector():
     """The reference's own scatter check: index_select(input, 0, pos) with its
