@@ -1,7 +1,8 @@
-"""CPU oracle for the per-GPU MoE layer forward.  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for the per-GPU MoE layer forward and backward.  TEST INFRASTRUCTURE ONLY.
 
 This module restates, on the CPU with numpy and torch's CPU kernels, the
-arithmetic of the reference's MoE layer forward:
+arithmetic of the reference's MoE layer forward, and the gradients of it that
+the reference's backward pair computes:
 
     gate (linear -> top-k -> softmax)      mix_moe/mix_moe/gates/naive_gate.py:26-45
     expert count, cumulative sum, pos      mix_moe/mix_moe/functions.py:83-105
@@ -13,6 +14,8 @@ arithmetic of the reference's MoE layer forward:
     un-permute to flat token*k order       mix_moe/csrc/mix_moe.h:431-433
     gate-weighted combine                  mix_moe/mix_moe/layers.py:550-559
     64-row block planner (one GPU)         mix_moe/mix_moe/transformer.py:150-250
+    backward of the two expert GEMMs       mix_moe/csrc/mix_moe.h:300-388, 439-505
+                                           mix_moe/mix_moe/linear.py:91-113, 148-173
 
 Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
 ``bench.py`` may import it.  The product (``ccfuser_amd``) never does; its
@@ -38,6 +41,10 @@ something other than its own formula: torch library routines (``F.linear``,
 ``index_select``, ``F.gelu``, ``bmm``), brute-force Python loops on tiny
 inputs, closed forms (k=1, single expert, zero weights), and the two input
 vectors the reference ships (csrc/pos.pt, mix_moe/all_expert_count.pt).  The
+backward functions are closed-form chain rules and use no autograd; they are
+pinned against torch's autograd through library operations (``F.linear``,
+``topk``, ``softmax``, ``index_select``, ``F.gelu``, ``index_copy``, ``bmm``)
+and against central finite differences in float64 on tiny inputs.  The
 reference holds no expected-output vectors for this path and its Python cannot
 be imported without its CUDA extension, so the third-party arithmetic it
 delegates to torch (README pins torch 2.0.1) is pinned by the textbook
@@ -296,6 +303,129 @@ def ffn_segments(x, seg_start, seg_len, seg_expert, w1, b1, w2, b2, *,
         out[s:s + n] = expert_ffn(x[s:s + n], off, w1[e:e + 1], b1[e:e + 1], w2[e:e + 1],
                                   b2[e:e + 1], round_intermediate=round_intermediate)
     return out
+
+
+# --------------------------------------------------------------------------
+# backward of the same path (closed-form chain rule, fp32, no autograd)
+# --------------------------------------------------------------------------
+def combine_backward(grad_out: torch.Tensor, y_flat: torch.Tensor, score: torch.Tensor,
+                     top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Backward of ``combine`` (the bmm at layers.py:556): ``grad_y_flat[t*k+s] =
+    score[t,s] * grad_out[t]`` and ``grad_score[t,s] = <grad_out[t], y_flat[t*k+s]>``."""
+    g = grad_out.to(torch.float32)
+    sc = score.to(torch.float32).reshape(-1, top_k)
+    gy = (sc[:, :, None] * g[:, None, :]).reshape(-1, g.shape[1])
+    gs = (y_flat.to(torch.float32).view(-1, top_k, g.shape[1]) * g[:, None, :]).sum(-1)
+    return gy, gs
+
+
+def gelu_backward(grad_act: torch.Tensor, h_pre: torch.Tensor) -> torch.Tensor:
+    """d/dh of the erf GELU: ``Phi(h) + h * phi(h)`` times the incoming gradient."""
+    h = h_pre.to(torch.float32)
+    cdf = 0.5 * (1.0 + torch.erf(h * (1.0 / math.sqrt(2.0))))
+    pdf = torch.exp(-0.5 * h * h) * (1.0 / math.sqrt(2.0 * math.pi))
+    return grad_act.to(torch.float32) * (cdf + h * pdf)
+
+
+def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, pos: torch.Tensor,
+                  offsets: torch.Tensor, w2: torch.Tensor):
+    """``second_gemm_backward`` (mix_moe.h:439-505): the gradient rows are brought into
+    expert order (``local_scatter`` at 453-454, the inverse of the index_copy_ at 433),
+    ``grad_act = gy @ w2[e]`` (first_mix_gemm at 470-483 with the stored [E, d, f]
+    weight as [E, K, N]), ``grad_w2[e] = gy^T @ act`` (launch_compute_weight_grad,
+    497-503).  The reference returns ``grad_bias`` uninitialised (489); here it is the
+    column sum of ``gy`` over the expert's rows, which is what the forward's
+    ``+ b2[e]`` differentiates to.  Returns (grad_act [R, f], grad_w2, grad_b2)."""
+    off = offsets.tolist()
+    gy = grad_y_flat.to(torch.float32)[pos]
+    a32 = act.to(torch.float32)
+    E, d, f = w2.shape
+    g_act = torch.zeros(gy.shape[0], f)
+    g_w = torch.zeros(E, d, f)
+    g_b = torch.zeros(E, d)
+    for e in range(E):
+        lo, hi = off[e], off[e + 1]
+        if hi == lo:
+            continue
+        g_act[lo:hi] = torch.mm(gy[lo:hi], w2[e].to(torch.float32))
+        g_w[e] = torch.mm(gy[lo:hi].t(), a32[lo:hi])
+        g_b[e] = gy[lo:hi].sum(0)
+    return g_act, g_w, g_b
+
+
+def ffn1_backward(grad_h: torch.Tensor, x: torch.Tensor, pos: torch.Tensor, top_k: int,
+                  offsets: torch.Tensor, w1: torch.Tensor):
+    """``first_gemm_backward`` (mix_moe.h:300-388): ``grad_buf = grad_h @ w1[e]``
+    (second_mix_gemm at 322-335 with the stored [E, f, d] weight as [E, K, N]),
+    ``grad_w1[e] = grad_h^T @ buf`` (347-353), and the rows added back onto their
+    tokens, ``grad_in.index_add_(0, pos // k, grad_buf)`` (359-365).  ``grad_bias``
+    as in ``ffn2_backward``.  Returns (grad_in [T, d], grad_w1, grad_b1)."""
+    off = offsets.tolist()
+    gh = grad_h.to(torch.float32)
+    src = torch.div(pos, top_k, rounding_mode="floor")
+    buf = x.to(torch.float32)[src]
+    E, f, d = w1.shape
+    g_buf = torch.zeros(gh.shape[0], d)
+    g_w = torch.zeros(E, f, d)
+    g_b = torch.zeros(E, f)
+    for e in range(E):
+        lo, hi = off[e], off[e + 1]
+        if hi == lo:
+            continue
+        g_buf[lo:hi] = torch.mm(gh[lo:hi], w1[e].to(torch.float32))
+        g_w[e] = torch.mm(gh[lo:hi].t(), buf[lo:hi])
+        g_b[e] = gh[lo:hi].sum(0)
+    g_in = torch.zeros(x.shape[0], d)
+    g_in.index_add_(0, src, g_buf)
+    return g_in, g_w, g_b
+
+
+def gate_backward(grad_score: torch.Tensor, score: torch.Tensor, idx: torch.Tensor,
+                  x: torch.Tensor, wg: torch.Tensor):
+    """Backward of ``NaiveGate.forward`` (naive_gate.py:31-38) for the gradient of the
+    scores: softmax over the k selected logits, the selection as a scatter into
+    [T, E], then the linear layer.  Returns (grad_x [T, d], grad_wg, grad_bg)."""
+    T, k = idx.shape
+    s = score.to(torch.float32).reshape(T, k)
+    g = grad_score.to(torch.float32).reshape(T, k)
+    g_val = s * (g - (s * g).sum(-1, keepdim=True))
+    g_logits = torch.zeros(T, wg.shape[0])
+    g_logits.scatter_add_(1, idx, g_val)
+    return (torch.mm(g_logits, wg.to(torch.float32)), torch.mm(g_logits.t(), x.to(torch.float32)),
+            g_logits.sum(0))
+
+
+def moe_layer_backward(x, wg, bg, w1, b1, w2, b2, top_k: int, grad_out: torch.Tensor, *,
+                       capacity: int = -1) -> Dict[str, torch.Tensor]:
+    """Gradients of ``moe_layer_forward``'s ``out`` with respect to ``x`` and every
+    parameter, for the incoming ``grad_out`` [T, d]: the forward is recomputed in fp32
+    and the stages above are chained in reverse.  The routing is piecewise constant."""
+    T = x.shape[0]
+    E = w1.shape[0]
+    idx, score, _ = naive_gate(x, wg, bg, top_k)
+    idx_kept = limit_by_capacity(idx, E, capacity)
+    pos, offsets = assign_pos(idx_kept, E)
+    off = offsets.tolist()
+    buf = local_scatter(x, pos, top_k).to(torch.float32)
+    h_pre = torch.zeros(buf.shape[0], w1.shape[1])
+    y_sorted = torch.zeros(buf.shape[0], w2.shape[1])
+    for e in range(E):
+        lo, hi = off[e], off[e + 1]
+        if hi > lo:
+            h_pre[lo:hi] = torch.mm(buf[lo:hi], w1[e].to(torch.float32).t()) + b1[e].to(torch.float32)
+            y_sorted[lo:hi] = torch.mm(gelu_exact(h_pre[lo:hi]), w2[e].to(torch.float32).t()) \
+                + b2[e].to(torch.float32)
+    act = gelu_exact(h_pre)
+    y_flat = unpermute(y_sorted, pos, T * top_k)
+    g_y_flat, g_score = combine_backward(grad_out, y_flat, score, top_k)
+    g_act, g_w2, g_b2 = ffn2_backward(g_y_flat, act, pos, offsets, w2)
+    g_h = gelu_backward(g_act, h_pre)
+    g_x, g_w1, g_b1 = ffn1_backward(g_h, x, pos, top_k, offsets, w1)
+    gx_gate, g_wg, g_bg = gate_backward(g_score, score, idx, x, wg)
+    return {"x": g_x + gx_gate, "x_experts": g_x, "x_gate": gx_gate, "wg": g_wg, "bg": g_bg,
+            "w1": g_w1, "b1": g_b1, "w2": g_w2, "b2": g_b2, "score": g_score, "act": g_act,
+            "h": g_h, "y_flat": g_y_flat, "h_pre": h_pre, "act_fwd": act, "y_flat_fwd": y_flat,
+            "pos": pos, "offsets": offsets, "idx": idx, "score_fwd": score}
 
 
 # --------------------------------------------------------------------------
