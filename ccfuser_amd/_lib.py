@@ -37,6 +37,10 @@ SIGNATURES = {
     "ccf_ffn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "ccf_ffn1_forward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p, _p, _sz, _p]),
     "ccf_ffn2_forward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
+    "ccf_combine_backward": (_i, [_p, _p, _p, _p, _i, _i, _i, _p, _p, _p]),
+    "ccf_ffn_backward_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "ccf_ffn2_backward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
+    "ccf_ffn1_backward": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
     "ccf_moe_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "ccf_moe_forward": (_i, [_p] * 7 + [_i] * 6 + [_p] * 6 + [_p, _sz, _p]),
     "ccf_moe_forward_set_events": (_i, [C.POINTER(_p), _i]),

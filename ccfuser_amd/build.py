@@ -16,7 +16,7 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIB = HERE / "libccfuser_moe.so"
-SOURCES = ["api.hip", "gate.hip", "route.hip", "rows.hip", "ffn.hip"]
+SOURCES = ["api.hip", "gate.hip", "route.hip", "rows.hip", "bwd.hip", "ffn.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = [

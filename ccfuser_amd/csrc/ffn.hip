@@ -163,6 +163,12 @@ struct GroupedArgs {
   const half_t *row_scale;  // [rows] or NULL; NULL with the GELU epilogue
   const int32_t *plan;
   int N, K;
+  // K-segment form (weight gradients): the contraction runs over a per-expert
+  // range of columns of A and B, which are then [rows, lda] and [N, ldb] matrices
+  // shared by all experts; expert e owns columns k_seg[e] .. k_seg[e+1] (multiples
+  // of BK, at least four K tiles) and rows e*seg_rows .. of C.  NULL otherwise.
+  const int32_t *k_seg;
+  int lda, ldb, seg_rows;
 };
 
 // erf-form GELU, 0.5*v*(1+erf(v/sqrt2)) = 0.5*(v + |v| erf(|z|)), z = v/sqrt2.
@@ -208,25 +214,45 @@ __device__ __forceinline__ int tile_row_to_local(int r, int rows) {
 // Global source of every tile load of this lane for the tile of plan entry
 // `ent`: K element 0 of the (clamped) A row and B row, at this lane's K chunk.
 // Padded A rows re-read the tile's last real row, B rows past N the last row.
-template <class Cfg>
+template <class Cfg, bool kSeg = false>
 __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v ent,
                                              const half_t *(&a_src)[Cfg::A_DMA],
                                              const half_t *(&b_src)[Cfg::B_DMA]) {
   using ML = GemmMainloop<Cfg>;
   const int row0 = ent[1], rows = ent[2], n0 = ent[3] * Cfg::BN;
-  const half_t *Be = p.B + static_cast<size_t>(ent[0]) * p.N * p.K;
+  const int lda = kSeg ? p.lda : p.K, ldb = kSeg ? p.ldb : p.K;
+  const half_t *Ae = p.A, *Be;
+  if constexpr (kSeg) {
+    const int koff = p.k_seg[ent[0]];
+    Ae = p.A + koff;
+    Be = p.B + koff;
+  } else {
+    Be = p.B + static_cast<size_t>(ent[0]) * p.N * p.K;
+  }
 #pragma unroll
   for (int i = 0; i < Cfg::A_DMA; ++i) {
     const int r = ML::dma_row(i);
     const int rc = tile_row_to_local<Cfg>(r, rows);
-    const int g = p.a_rows ? p.a_rows[row0 + rc] : row0 + rc;
-    a_src[i] = p.A + static_cast<size_t>(g) * p.K + ML::dma_chunk(r) * 8;
+    int g = row0 + rc;
+    if constexpr (kSeg) g -= ent[0] * p.seg_rows;      // sorted row j of expert e is row j - e*seg_rows of A
+    else if (p.a_rows) g = p.a_rows[g];
+    a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(g)) * static_cast<uint32_t>(lda) + ML::dma_chunk(r) * 8;
   }
 #pragma unroll
   for (int i = 0; i < Cfg::B_DMA; ++i) {
     const int r = ML::dma_row(i);
     const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-    b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r) * 8;
+    b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r) * 8;
+  }
+}
+
+// K tiles of expert e's contraction.
+template <class Cfg, bool kSeg>
+__device__ __forceinline__ int k_tiles_of(const GroupedArgs &p, int e) {
+  if constexpr (kSeg) {
+    return __builtin_amdgcn_readfirstlane((p.k_seg[e + 1] - p.k_seg[e]) / Cfg::BK);
+  } else {
+    return p.K / Cfg::BK;
   }
 }
 
@@ -244,7 +270,7 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
   for (int tn = 0; tn < TN; ++tn) {
     col[tn] = n0 + acc16_col4<Cfg>(tn, tid);
     half4 bv = {0, 0, 0, 0};
-    if (col[tn] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn]);
+    if (p.bias && col[tn] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn]);
 #pragma unroll
     for (int c = 0; c < 4; ++c) bias_v[tn][c] = static_cast<float>(bv[c]);
   }
@@ -283,7 +309,7 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
   });
 }
 
-template <class Cfg, bool kGelu>
+template <class Cfg, bool kGelu, bool kSeg = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_kernel(GroupedArgs p) {
   using ML = GemmMainloop<Cfg>;
@@ -297,11 +323,11 @@ grouped_gemm_kernel(GroupedArgs p) {
 
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[Cfg::B_DMA];
-  tile_sources<Cfg>(p, ent, a_src, b_src);
+  tile_sources<Cfg, kSeg>(p, ent, a_src, b_src);
 
   const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
   if constexpr (Cfg::SCHED == 4) {
-    Ring16Mainloop<Cfg>::run(a_src, b_src, p.K, rows);
+    Ring16Mainloop<Cfg>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, rows);
     epilogue16<Cfg, kGelu>(p, e, row0, rows, n0);
     return;
   } else {
@@ -330,7 +356,7 @@ grouped_gemm_kernel(GroupedArgs p) {
     for (int q = 0; q < 4; ++q) {
       col[tn][q] = n0 + acc_col4<Cfg>(tn, q);
       half4 bv = {0, 0, 0, 0};
-      if (col[tn][q] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn][q]);
+      if (p.bias && col[tn][q] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn][q]);
 #pragma unroll
       for (int c = 0; c < 4; ++c) bias_v[tn][q][c] = static_cast<float>(bv[c]);
     }
@@ -377,7 +403,7 @@ grouped_gemm_kernel(GroupedArgs p) {
 // the first barrier covers them); steps 0 .. KT-3 run with this tile's sources;
 // then the sources of the next tile are computed and the last two steps load
 // its K tiles 0 and 1.
-template <class Cfg, bool kGelu>
+template <class Cfg, bool kGelu, bool kSeg = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   using ML = GemmMainloop<Cfg>;
@@ -390,15 +416,14 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   int4v ent = plan[slot_j * 8 + xcd];
   if (ent[0] < 0) return;                             // the used slots of an XCD are a prefix
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int KT = p.K / Cfg::BK;
 
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[Cfg::B_DMA];
-  tile_sources<Cfg>(p, ent, a_src, b_src);
+  tile_sources<Cfg, kSeg>(p, ent, a_src, b_src);
   int a_off[2], b_off[2];
   R::frag_offsets(a_off, b_off);
   half8 fa[2][TM], fb[2][TN];
-  R::prologue(fa, fb, a_src, b_src, KT, a_off, b_off, wave);
+  R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg>(p, ent[0]), a_off, b_off, wave);
   R::reserve();
   int phase = 0;
 
@@ -415,29 +440,33 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       }
     }
     const int n_row0 = nent[1], n_rows = nent[2];
+    const int KT = k_tiles_of<Cfg, kSeg>(p, ent[0]);
+    const int k_end = KT * Cfg::BK;
 
     R::zero_acc();
 
     int next_row[Cfg::A_DMA];                         // A row of the next tile per tile load
-    const int tid0 = fresh_tid();
+    if constexpr (!kSeg) {
+      const int tid0 = fresh_tid();
 #pragma unroll
-    for (int i = 0; i < Cfg::A_DMA; ++i) {
-      const int r = ML::dma_row(i, tid0);
-      const int rc = R::local_row(r, n_rows);
-      if (p.a_rows) {
-        const int32_t *src = p.a_rows + n_row0 + rc;
-        asm volatile("global_load_dword %0, %1, off" : "=v"(next_row[i]) : "v"(src) : "memory");
-      } else {
-        next_row[i] = n_row0 + rc;
+      for (int i = 0; i < Cfg::A_DMA; ++i) {
+        const int r = ML::dma_row(i, tid0);
+        const int rc = R::local_row(r, n_rows);
+        if (p.a_rows) {
+          const int32_t *src = p.a_rows + n_row0 + rc;
+          asm volatile("global_load_dword %0, %1, off" : "=v"(next_row[i]) : "v"(src) : "memory");
+        } else {
+          next_row[i] = n_row0 + rc;
+        }
       }
     }
 
     const int live_m = R::live_blocks(ent[2]);
     R::acc_settle();
     if (live_m == TM) {
-      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, p.K, phase, wave, live_m);
+      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m);
     } else {
-      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, p.K, phase, wave, live_m);
+      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m);
     }
     {
       // sources of the next tile (tile_sources() with the row indices already at hand); the
@@ -445,26 +474,42 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       // 16 more registers across it
       int n_e = __builtin_amdgcn_readfirstlane(nent[0]), n_tn = __builtin_amdgcn_readfirstlane(nent[3]);
       asm volatile("" : "+s"(n_e), "+s"(n_tn));
-      const half_t *Be = p.B + static_cast<size_t>(n_e) * p.N * p.K;
+      const int lda = kSeg ? p.lda : p.K, ldb = kSeg ? p.ldb : p.K;
+      const half_t *Ae = p.A, *Be;
+      if constexpr (kSeg) {
+        const int koff = p.k_seg[n_e];
+        Ae = p.A + koff;
+        Be = p.B + koff;
+      } else {
+        Be = p.B + static_cast<size_t>(n_e) * p.N * p.K;
+      }
       const int n0 = n_tn * Cfg::BN;
       const int tid1 = fresh_tid();
 #pragma unroll
       for (int i = 0; i < Cfg::A_DMA; ++i) {
-        asm volatile("" : "+v"(next_row[i]));         // requested before step 0, complete at its barrier
         const int r = ML::dma_row(i, tid1);
-        a_src[i] = p.A + static_cast<size_t>(next_row[i]) * p.K + ML::dma_chunk(r, tid1) * 8;
+        if constexpr (kSeg) {
+          // sorted row j of expert e is row j - e*seg_rows of A; nothing to look up, so it is computed here
+          int nr0 = __builtin_amdgcn_readfirstlane(nent[1]), nrows = __builtin_amdgcn_readfirstlane(nent[2]);
+          asm volatile("" : "+s"(nr0), "+s"(nrows));
+          next_row[i] = nr0 - n_e * p.seg_rows + R::local_row(r, nrows);
+        } else {
+          asm volatile("" : "+v"(next_row[i]));       // requested before step 0, complete at its barrier
+        }
+        a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(next_row[i])) * static_cast<uint32_t>(lda) +
+                   ML::dma_chunk(r, tid1) * 8;
       }
 #pragma unroll
       for (int i = 0; i < Cfg::B_DMA; ++i) {
         const int r = ML::dma_row(i, tid1);
         const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-        b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r, tid1) * 8;
+        b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r, tid1) * 8;
       }
     }
     if (live_m == TM) {
-      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, p.K, phase, wave, live_m);
+      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m);
     } else {
-      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, p.K, phase, wave, live_m);
+      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m);
     }
     R::acc_settle();
     epilogue16<Cfg, kGelu>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
@@ -541,12 +586,12 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
                  int N, int K, const half_t *B, const half_t *bias, bool gelu, half_t *C,
                  const int32_t *c_rows, const half_t *row_scale, int32_t *plan, hipStream_t stream,
                  const char *what) {
-  CCF_REQUIRE(A && offsets && B && bias && C && plan, CCF_ERR_ARG, "%s: null pointer", what);
+  CCF_REQUIRE(A && offsets && B && C && plan, CCF_ERR_ARG, "%s: null pointer", what);
   CCF_REQUIRE(max_rows >= 0 && E > 0 && N > 0 && K > 0, CCF_ERR_ARG, "%s: bad size", what);
   CCF_REQUIRE(E <= 1024, CCF_ERR_SHAPE, "%s: num_expert=%d exceeds 1024", what, E);
   CCF_REQUIRE(K % 64 == 0, CCF_ERR_SHAPE, "%s: K=%d is not a multiple of 64", what, K);
   CCF_REQUIRE(N % 8 == 0, CCF_ERR_SHAPE, "%s: N=%d is not a multiple of 8", what, N);
-  CCF_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C) && aligned16(bias), CCF_ERR_ARG,
+  CCF_REQUIRE(aligned16(A) && aligned16(B) && aligned16(C) && (!bias || aligned16(bias)), CCF_ERR_ARG,
               "%s: operands must be 16-byte aligned", what);
   CCF_REQUIRE(!(gelu && row_scale), CCF_ERR_ARG, "%s: the GELU epilogue takes no row scale", what);
   if (max_rows == 0) return CCF_OK;
@@ -567,6 +612,9 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.plan = plan;
   p.N = N;
   p.K = K;
+  p.k_seg = nullptr;
+  p.lda = p.ldb = K;
+  p.seg_rows = 0;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
@@ -579,6 +627,128 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
                        stream, p);
   }
   return check_launch(what);
+}
+
+// C[e*M + m, n] = sum over k in [k_seg[e], k_seg[e+1]) of A[m, k] * B[n, k]: the weight
+// gradient of expert e from the two transposed activation matrices.  row_off[e] = e*M.
+int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const int32_t *k_seg,
+                      const int32_t *row_off, int E, int M, int N, half_t *C, int32_t *plan,
+                      hipStream_t stream, const char *what) {
+  CCF_REQUIRE(A && B && k_seg && row_off && C && plan, CCF_ERR_ARG, "%s: null pointer", what);
+  CCF_REQUIRE(lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0, CCF_ERR_SHAPE, "%s: strides and N must be multiples of 8", what);
+  CCF_REQUIRE(static_cast<long long>(E) * M < (1ll << 31), CCF_ERR_SHAPE, "%s: output too tall", what);
+  const int max_rows = E * M;
+  const int max_tiles = max_tiles_for(max_rows, E, Cfg5::BM);
+  const int n_tiles_n = (N + Cfg5::BN - 1) / Cfg5::BN;
+  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, row_off, E, Cfg5::BM, max_tiles,
+                     max_rows, n_tiles_n, plan);
+  if (int rc = check_launch("plan_kernel")) return rc;
+  GroupedArgs p;
+  p.A = A;
+  p.a_rows = nullptr;
+  p.B = B;
+  p.bias = nullptr;
+  p.C = C;
+  p.c_rows = nullptr;
+  p.row_scale = nullptr;
+  p.plan = plan;
+  p.N = N;
+  p.K = 0;
+  p.k_seg = k_seg;
+  p.lda = lda;
+  p.ldb = ldb;
+  p.seg_rows = M;
+  const long long wgs = launched_wgs(max_tiles, n_tiles_n);
+  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
+  const int grid = persistent_grid();
+  if (grid >= 8) {
+    const long long g = grid < wgs ? grid : wgs;
+    hipLaunchKernelGGL((grouped_gemm_persistent_kernel<Cfg5, false, true>), dim3(static_cast<unsigned>(g)),
+                       dim3(Cfg5::THREADS), 0, stream, p, static_cast<int>(wgs / 8));
+  } else {
+    hipLaunchKernelGGL((grouped_gemm_kernel<Cfg5, false, true>), dim3(static_cast<unsigned>(wgs)),
+                       dim3(Cfg5::THREADS), 0, stream, p);
+  }
+  return check_launch(what);
+}
+
+// Workspace of the backward entry points, carved in this order.
+struct BackwardWs {
+  int32_t *plan_rows;      // tile plan of the input-gradient GEMM
+  int32_t *plan_w;         // tile plan of the weight-gradient GEMM
+  int32_t *k_seg, *row_off, *blk_row0, *blk_cnt;
+  half_t *w_t;             // [E, in, out] transposed weight
+  half_t *a_t, *b_t;       // [out, ld_t], [in, ld_t] transposed activations
+  float *partial;          // [ld_t / 64, out] bias partial sums
+  int ld_t, n_blk;
+  size_t bytes;
+};
+
+BackwardWs carve_backward(void *base, int max_rows, int E, int d, int f) {
+  BackwardWs w;
+  const int big = d > f ? d : f;
+  w.ld_t = padded_rows(max_rows, E);
+  w.n_blk = w.ld_t / 64;
+  char *p = static_cast<char *>(base);
+  auto take = [&](size_t bytes) {
+    char *r = p;
+    p += round_up(bytes, 256);
+    return r;
+  };
+  w.plan_rows = reinterpret_cast<int32_t *>(take(plan_bytes(max_rows, E, big)));
+  w.plan_w = reinterpret_cast<int32_t *>(take(plan_bytes(E * big, E, big)));
+  w.k_seg = reinterpret_cast<int32_t *>(take(sizeof(int32_t) * (E + 1)));
+  w.row_off = reinterpret_cast<int32_t *>(take(sizeof(int32_t) * (E + 1)));
+  w.blk_row0 = reinterpret_cast<int32_t *>(take(sizeof(int32_t) * w.n_blk));
+  w.blk_cnt = reinterpret_cast<int32_t *>(take(sizeof(int32_t) * w.n_blk));
+  w.w_t = reinterpret_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(E) * d * f));
+  w.a_t = reinterpret_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(big) * w.ld_t));
+  w.b_t = reinterpret_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(big) * w.ld_t));
+  w.partial = reinterpret_cast<float *>(take(sizeof(float) * static_cast<size_t>(w.n_blk) * big));
+  w.bytes = static_cast<size_t>(p - static_cast<char *>(base));
+  return w;
+}
+
+// One expert linear layer's backward.  Forward was out[c_row(j)] = in[a_row(j)] * w[e]^T + b[e]
+// with w [E, n_out, n_in].  Given grad_out rows (through g_rows) and the forward's input rows
+// (through in_rows):
+//   grad_in[gi_rows(j)] = grad_out[g_rows(j)] * w[e]            (grouped GEMM on w^T)
+//   grad_w[e] = grad_out_e^T * in_e,  grad_b[e] = column sums of grad_out_e
+int linear_backward(const half_t *grad_out, const int32_t *g_rows, const half_t *in,
+                    const int32_t *in_rows, const int32_t *offsets, int max_rows, int E, int n_in,
+                    int n_out, const half_t *w, half_t *grad_in, const int32_t *gi_rows,
+                    half_t *grad_w, half_t *grad_b, void *workspace, size_t workspace_bytes,
+                    int d, int f, hipStream_t stream, const char *what) {
+  CCF_REQUIRE(grad_out && in && offsets && w && grad_in && grad_w && grad_b, CCF_ERR_ARG,
+              "%s: null pointer", what);
+  CCF_REQUIRE(max_rows >= 0 && E > 0 && E <= 1024 && d > 0 && f > 0, CCF_ERR_ARG, "%s: bad size", what);
+  CCF_REQUIRE(d % 64 == 0 && f % 64 == 0, CCF_ERR_SHAPE,
+              "%s: d_model=%d and d_ffn=%d must be multiples of 64", what, d, f);
+  CCF_REQUIRE(aligned16(grad_out) && aligned16(in) && aligned16(w) && aligned16(grad_in) &&
+                  aligned16(grad_w) && aligned16(grad_b) && aligned16(workspace),
+              CCF_ERR_ARG, "%s: operands must be 16-byte aligned", what);
+  const size_t need = ccf_ffn_backward_workspace_bytes(max_rows, E, d, f);
+  CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
+              "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);
+  const BackwardWs ws = carve_backward(workspace, max_rows, E, d, f);
+  // input gradient
+  if (int rc = launch_transpose_weights(w, ws.w_t, E, n_out, n_in, stream)) return rc;
+  if (int rc = grouped_gemm(grad_out, g_rows, offsets, max_rows, E, n_in, n_out, ws.w_t, nullptr, false,
+                            grad_in, gi_rows, nullptr, ws.plan_rows, stream, what))
+    return rc;
+  // weight and bias gradients
+  if (int rc = launch_kseg(offsets, E, max_rows, n_out, ws.n_blk, ws.k_seg, ws.row_off, ws.blk_row0,
+                           ws.blk_cnt, stream))
+    return rc;
+  if (int rc = launch_transpose_rows(grad_out, g_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_out, ws.ld_t,
+                                     ws.a_t, ws.partial, stream))
+    return rc;
+  if (int rc = launch_transpose_rows(in, in_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_in, ws.ld_t,
+                                     ws.b_t, nullptr, stream))
+    return rc;
+  if (int rc = launch_bias_reduce(ws.partial, ws.k_seg, E, n_out, grad_b, stream)) return rc;
+  return grouped_gemm_kseg(ws.a_t, ws.ld_t, ws.b_t, ws.ld_t, ws.k_seg, ws.row_off, E, n_out, n_in,
+                           grad_w, ws.plan_w, stream, what);
 }
 
 }  // namespace
@@ -633,4 +803,38 @@ extern "C" int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int
                       d_ffn, static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), false,
                       static_cast<half_t *>(y), dst_row, static_cast<const half_t *>(row_scale),
                       static_cast<int32_t *>(workspace), as_stream(stream), "ffn2");
+}
+
+extern "C" size_t ccf_ffn_backward_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn) {
+  if (max_rows < 0 || num_expert <= 0 || d_model <= 0 || d_ffn <= 0) return 0;
+  return ccf::carve_backward(nullptr, max_rows, num_expert, d_model, d_ffn).bytes;
+}
+
+extern "C" int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const int32_t *dst_row,
+                                 const int32_t *offsets, int max_rows, int num_expert, int d_model,
+                                 int d_ffn, const void *w2, void *grad_act, void *grad_w2,
+                                 void *grad_b2, void *workspace, size_t workspace_bytes,
+                                 ccf_stream_t stream) {
+  using namespace ccf;
+  if (max_rows == 0) return CCF_OK;
+  return linear_backward(static_cast<const half_t *>(grad_y_flat), dst_row,
+                         static_cast<const half_t *>(act), nullptr, offsets, max_rows, num_expert,
+                         d_ffn, d_model, static_cast<const half_t *>(w2),
+                         static_cast<half_t *>(grad_act), nullptr, static_cast<half_t *>(grad_w2),
+                         static_cast<half_t *>(grad_b2), workspace, workspace_bytes, d_model, d_ffn,
+                         as_stream(stream), "ffn2_backward");
+}
+
+extern "C" int ccf_ffn1_backward(const void *grad_h, const void *x, const int32_t *src_row,
+                                 const int32_t *dst_row, const int32_t *offsets, int max_rows,
+                                 int num_expert, int d_model, int d_ffn, const void *w1,
+                                 void *grad_x_flat, void *grad_w1, void *grad_b1, void *workspace,
+                                 size_t workspace_bytes, ccf_stream_t stream) {
+  using namespace ccf;
+  if (max_rows == 0) return CCF_OK;
+  return linear_backward(static_cast<const half_t *>(grad_h), nullptr, static_cast<const half_t *>(x),
+                         src_row, offsets, max_rows, num_expert, d_model, d_ffn,
+                         static_cast<const half_t *>(w1), static_cast<half_t *>(grad_x_flat), dst_row,
+                         static_cast<half_t *>(grad_w1), static_cast<half_t *>(grad_b1), workspace,
+                         workspace_bytes, d_model, d_ffn, as_stream(stream), "ffn1_backward");
 }

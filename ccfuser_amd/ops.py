@@ -279,6 +279,95 @@ def ffn2(h: torch.Tensor, dst_row: Optional[torch.Tensor], offsets: torch.Tensor
     return y
 
 
+# -------------------------------------------------------------- backward
+def combine_backward(grad_out: torch.Tensor, y_flat: torch.Tensor, score: torch.Tensor, top_k: int,
+                     inv_pos: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(grad_y_flat [T*k, d], grad_score [T*k]) of ``combine``; zero for dropped slots."""
+    _check(grad_out, "grad_out", dtype=torch.float16, ndim=2)
+    _check(y_flat, "y_flat", dtype=torch.float16, ndim=2)
+    _check(score, "score", dtype=torch.float16)
+    if inv_pos is not None:
+        _check(inv_pos, "inv_pos", dtype=torch.int32, ndim=1)
+    n, d = y_flat.shape
+    T = grad_out.shape[0]
+    if T * top_k != n or grad_out.shape[1] != d or score.numel() != n or \
+            (inv_pos is not None and inv_pos.numel() != n):
+        raise ValueError("combine_backward: sizes do not match tokens*top_k")
+    g_y = torch.empty_like(y_flat)
+    g_s = torch.empty(n, dtype=torch.float16, device=y_flat.device)
+    with torch.cuda.device(y_flat.device):
+        _lib.call("ccf_combine_backward", _ptr(grad_out), _ptr(y_flat), _ptr(score), _ptr(inv_pos), T,
+                  int(top_k), d, _ptr(g_y), _ptr(g_s), _stream(y_flat))
+    return g_y, g_s
+
+
+def _backward_ws(max_rows: int, E: int, d: int, f: int, like: torch.Tensor) -> torch.Tensor:
+    return _workspace(_lib.lib().ccf_ffn_backward_workspace_bytes(int(max_rows), E, d, f), like)
+
+
+def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optional[torch.Tensor],
+                  offsets: torch.Tensor, max_rows: int, w2: torch.Tensor):
+    """(grad_act [max_rows, f], grad_w2 [E, d, f], grad_b2 [E, d]) of ``ffn2``.
+    Rows of ``grad_act`` past ``offsets[-1]`` are zero."""
+    _check(grad_y_flat, "grad_y_flat", dtype=torch.float16, ndim=2)
+    _check(act, "act", dtype=torch.float16, ndim=2)
+    _check(w2, "ffn2 weight", dtype=torch.float16, ndim=3)
+    _check(offsets, "offsets", dtype=torch.int32, ndim=1)
+    E, d, f = w2.shape
+    if grad_y_flat.shape[1] != d or act.shape[1] != f or offsets.numel() != E + 1 or act.shape[0] < max_rows:
+        raise ValueError("ffn2_backward: shapes do not match the weight")
+    if dst_row is not None:
+        _check(dst_row, "dst_row", dtype=torch.int32, ndim=1)
+        if dst_row.numel() < max_rows:
+            raise ValueError("ffn2_backward: dst_row shorter than max_rows")
+    elif grad_y_flat.shape[0] < max_rows:
+        raise ValueError("ffn2_backward: grad_y_flat has fewer rows than max_rows")
+    dev = act.device
+    g_act = torch.zeros(max_rows, f, dtype=torch.float16, device=dev)
+    g_w = torch.empty_like(w2)
+    g_b = torch.empty(E, d, dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        ws = _backward_ws(max_rows, E, d, f, act)
+        _lib.call("ccf_ffn2_backward", _ptr(grad_y_flat), _ptr(act), _ptr(dst_row), _ptr(offsets),
+                  int(max_rows), E, d, f, _ptr(w2), _ptr(g_act), _ptr(g_w), _ptr(g_b), _ptr(ws),
+                  ws.numel(), _stream(act))
+    return g_act, g_w, g_b
+
+
+def ffn1_backward(grad_h: torch.Tensor, x: torch.Tensor, src_row: Optional[torch.Tensor],
+                  dst_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
+                  w1: torch.Tensor, n_flat: int):
+    """(grad_x_flat [n_flat, d], grad_w1 [E, f, d], grad_b1 [E, f]) of ``ffn1`` without the
+    fused GELU.  ``grad_x_flat[dst_row[j]]`` is the gradient of sorted row j; rows nothing
+    maps to are zero."""
+    _check(grad_h, "grad_h", dtype=torch.float16, ndim=2)
+    _check(x, "x", dtype=torch.float16, ndim=2)
+    _check(w1, "ffn1 weight", dtype=torch.float16, ndim=3)
+    _check(offsets, "offsets", dtype=torch.int32, ndim=1)
+    E, f, d = w1.shape
+    if grad_h.shape[1] != f or x.shape[1] != d or offsets.numel() != E + 1 or grad_h.shape[0] < max_rows:
+        raise ValueError("ffn1_backward: shapes do not match the weight")
+    for t, nm in ((src_row, "src_row"), (dst_row, "dst_row")):
+        if t is not None:
+            _check(t, nm, dtype=torch.int32, ndim=1)
+            if t.numel() < max_rows:
+                raise ValueError(f"ffn1_backward: {nm} shorter than max_rows")
+    if src_row is None and x.shape[0] < max_rows:
+        raise ValueError("ffn1_backward: x has fewer rows than max_rows")
+    if n_flat < max_rows:
+        raise ValueError("ffn1_backward: n_flat smaller than max_rows")
+    dev = x.device
+    g_x = torch.zeros(n_flat, d, dtype=torch.float16, device=dev)
+    g_w = torch.empty_like(w1)
+    g_b = torch.empty(E, f, dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        ws = _backward_ws(max_rows, E, d, f, x)
+        _lib.call("ccf_ffn1_backward", _ptr(grad_h), _ptr(x), _ptr(src_row), _ptr(dst_row), _ptr(offsets),
+                  int(max_rows), E, d, f, _ptr(w1), _ptr(g_x), _ptr(g_w), _ptr(g_b), _ptr(ws),
+                  ws.numel(), _stream(x))
+    return g_x, g_w, g_b
+
+
 # ------------------------------------------------------- the whole layer
 def moe_forward(x, wg, bg, w1, b1, w2, b2, top_k: int, capacity: int = -1,
                 return_routing: bool = False, workspace: Optional[torch.Tensor] = None):

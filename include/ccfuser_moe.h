@@ -282,6 +282,67 @@ int ccf_moe_ffn_segments(const void *x, const int32_t *seg_start,
                          void *workspace, size_t workspace_bytes,
                          ccf_stream_t stream);
 
+/* ------------------------------------------------------------ backward */
+
+/*
+ * Backward of ccf_combine (the bmm at mix_moe/mix_moe/layers.py:556, which the
+ * reference leaves to autograd):
+ *   grad_y_flat[t*k+s, :] = score[t*k+s] * grad_out[t, :]
+ *   grad_score[t*k+s]     = <grad_out[t, :], y_flat[t*k+s, :]>
+ * both zero for dropped slots (inv_pos[i] < 0; inv_pos NULL = none dropped).
+ * All fp16; grad_y_flat [tokens*top_k, hidden], grad_score [tokens*top_k].
+ */
+int ccf_combine_backward(const void *grad_out, const void *y_flat, const void *score,
+                         const int32_t *inv_pos, int tokens, int top_k, int hidden,
+                         void *grad_y_flat, void *grad_score, ccf_stream_t stream);
+
+/* Workspace of ccf_ffn1_backward / ccf_ffn2_backward (transposed weight, transposed
+ * and padded activations, tile plans, bias partial sums). */
+size_t ccf_ffn_backward_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn);
+
+/*
+ * Backward of ccf_ffn2_forward.  Replaces _MixMOE::second_gemm_backward,
+ * mix_moe/csrc/mix_moe.h:439-505 (MixMOELinear2.backward,
+ * mix_moe/mix_moe/linear.py:148-173): the row scatter of grad_out into expert
+ * order (453-454) is the row index of the A loads, the input gradient is the
+ * grouped GEMM on the transposed weight, the weight gradient
+ * (launch_compute_weight_grad, 497-503) is the same grouped GEMM contracting
+ * over each expert's rows; grad_b2 is the column sum of the gradient rows (the
+ * reference returns it uninitialised, 489).
+ *   grad_y_flat fp16 [n_flat, d_model]  gradient of ccf_ffn2_forward's y
+ *   act         fp16 [max_rows, d_ffn]  the forward's input, expert order
+ *   dst_row, offsets                    as in the forward
+ *   w2          fp16 [E, d_model, d_ffn]
+ *   grad_act    fp16 [max_rows, d_ffn]  out; rows >= offsets[E] untouched
+ *   grad_w2     fp16 [E, d_model, d_ffn], grad_b2 fp16 [E, d_model]  out
+ * d_model and d_ffn must be multiples of 64.
+ */
+int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const int32_t *dst_row,
+                      const int32_t *offsets, int max_rows, int num_expert, int d_model,
+                      int d_ffn, const void *w2, void *grad_act, void *grad_w2,
+                      void *grad_b2, void *workspace, size_t workspace_bytes,
+                      ccf_stream_t stream);
+
+/*
+ * Backward of ccf_ffn1_forward without the fused GELU (grad_h is the gradient
+ * of the pre-activation).  Replaces _MixMOE::first_gemm_backward,
+ * mix_moe/csrc/mix_moe.h:300-388 (MixMOELinear1.backward,
+ * mix_moe/mix_moe/linear.py:91-113).
+ *   grad_h      fp16 [max_rows, d_ffn]  expert order
+ *   x           fp16 [tokens, d_model]  the forward's input, read through src_row
+ *   w1          fp16 [E, d_ffn, d_model]
+ *   grad_x_flat fp16 [n_flat, d_model]  out: row dst_row[j] = gradient of sorted
+ *               row j; rows of dropped slots untouched.  The reference's
+ *               index_add_ onto tokens (359-365) is ccf_combine over these rows
+ *               with unit scores.
+ *   grad_w1     fp16 [E, d_ffn, d_model], grad_b1 fp16 [E, d_ffn]  out
+ */
+int ccf_ffn1_backward(const void *grad_h, const void *x, const int32_t *src_row,
+                      const int32_t *dst_row, const int32_t *offsets, int max_rows,
+                      int num_expert, int d_model, int d_ffn, const void *w1,
+                      void *grad_x_flat, void *grad_w1, void *grad_b1, void *workspace,
+                      size_t workspace_bytes, ccf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
