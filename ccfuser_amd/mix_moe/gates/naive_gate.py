@@ -8,6 +8,40 @@ from ... import ops
 from .base_gate import BaseGate
 
 
+class _GateFunction(torch.autograd.Function):
+    """The fused gate kernel with the backward autograd derives for the reference's
+    linear -> topk -> softmax (naive_gate.py:31-38): softmax over the k selected
+    logits, the selection as a scatter into [T, E], then the linear layer.  The two
+    products with the [T, E] gradient are small library GEMMs."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, top_k, return_logits):
+        res = ops.gate_topk_softmax(x, weight.detach().contiguous(),
+                                    None if bias is None else bias.detach(), top_k,
+                                    return_logits=return_logits)
+        ctx.save_for_backward(x, weight, res[0], res[1])
+        ctx.has_bias = bias is not None
+        ctx.mark_non_differentiable(res[0])
+        if return_logits:
+            ctx.mark_non_differentiable(res[2])
+            return res[0], res[1], res[2]
+        return res[0], res[1]
+
+    @staticmethod
+    def backward(ctx, grad_idx, grad_score, grad_logits=None):
+        x, weight, idx, score = ctx.saved_tensors
+        s = score.float()
+        g = grad_score.float()
+        g_val = s * (g - (s * g).sum(-1, keepdim=True))
+        g_logits = torch.zeros(x.shape[0], weight.shape[0], dtype=torch.float32, device=x.device)
+        g_logits.scatter_add_(1, idx, g_val)
+        g16 = g_logits.to(x.dtype)
+        grad_x = torch.mm(g16, weight) if ctx.needs_input_grad[0] else None
+        grad_w = torch.mm(g16.t(), x) if ctx.needs_input_grad[1] else None
+        grad_b = g_logits.sum(0).to(x.dtype) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        return grad_x, grad_w, grad_b, None, None
+
+
 class NaiveGate(BaseGate):
     """``nn.Linear(d_model, tot_expert)`` followed by top-k and a softmax over the
     k selected logits.  The three torch kernels of the reference (linear, topk,
@@ -27,10 +61,7 @@ class NaiveGate(BaseGate):
         x = inp.reshape(-1, inp.shape[-1])
         if not x.is_contiguous():
             x = x.contiguous()
-        with torch.no_grad():
-            res = ops.gate_topk_softmax(x, self.gate.weight.detach().contiguous(),
-                                        None if self.gate.bias is None else self.gate.bias.detach(),
-                                        self.top_k, return_logits=return_all_scores)
+        res = _GateFunction.apply(x, self.gate.weight, self.gate.bias, self.top_k, bool(return_all_scores))
         idx = res[0].view(*lead, self.top_k)
         score = res[1]                                   # [(B*L), top_k], as the reference returns it
         # dummy loss, on the input's device (naive_gate.py:41)

@@ -30,6 +30,25 @@ def _local_gather(inp, pos, out_batch_size, maybe_overlap=True):
     return ops.local_gather(inp.contiguous(), pos.to(torch.int32), out_batch_size)
 
 
+class _Combine(torch.autograd.Function):
+    """Gate-weighted sum over a token's k expert outputs and its backward (the bmm of
+    the reference, layers.py:550-559, and what autograd derives from it)."""
+
+    @staticmethod
+    def forward(ctx, y_flat, score, top_k, inv_pos):
+        flat_score = score.contiguous().view(-1)
+        ctx.save_for_backward(y_flat, flat_score, inv_pos)
+        ctx.top_k = top_k
+        ctx.score_shape = score.shape
+        return ops.combine(y_flat, flat_score, top_k, inv_pos)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        y_flat, flat_score, inv_pos = ctx.saved_tensors
+        g_y, g_s = ops.combine_backward(grad_out.contiguous(), y_flat, flat_score, ctx.top_k, inv_pos)
+        return g_y, g_s.view(ctx.score_shape), None, None
+
+
 class MixMOE(nn.Module):
     """Gate + experts + gate-weighted combine (reference layers.py:34-83, 496-568)."""
 
@@ -77,4 +96,4 @@ class MixMOE(nn.Module):
         once, skipping dropped slots."""
         moe_output = self.moe_forward(moe_inp, pos, moe_inp_block_infos)
         inv_pos = moe_inp_block_infos.get("inv_pos") if hasattr(moe_inp_block_infos, "get") else None
-        return ops.combine(moe_output, gate_score.contiguous().view(-1), self.top_k, inv_pos)
+        return _Combine.apply(moe_output, gate_score, self.top_k, inv_pos)

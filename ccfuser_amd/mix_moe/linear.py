@@ -4,8 +4,8 @@
 ``apply(inp, pos, block_infos, weight, bias)`` (linear.py:60-86, 115-143) but
 hand the stored ``[E, out, in]`` weight straight to the grouped GEMM: the
 per-call ``weight.transpose(-2, -1).contiguous()`` of the reference
-(linear.py:74, 129) is gone.  Only the forward halves exist; calling backward
-raises.
+(linear.py:74, 129) is gone.  The backward halves (linear.py:91-113, 148-173)
+return gradients for the input rows, the weight and the bias.
 """
 import math
 import threading
@@ -49,14 +49,33 @@ class MixMOELinear1(Function):
 
     @staticmethod
     def forward(ctx, input_buf, pos, moe_inp_block_infos, weight, bias=None, fuse_gelu=False):
-        src_row, _, offsets, max_rows, _ = _routing(pos, moe_inp_block_infos)
+        src_row, dst_row, offsets, max_rows, n_flat = _routing(pos, moe_inp_block_infos)
         E = offsets.numel() - 1
+        ctx.save_for_backward(input_buf, weight, src_row, dst_row, offsets,
+                              moe_inp_block_infos.get("inv_pos"))
+        ctx.sizes = (max_rows, n_flat, bool(fuse_gelu))
         return ops.ffn1(input_buf, src_row, offsets, max_rows, weight.detach()[:E],
                         bias.detach()[:E], gelu=bool(fuse_gelu))
 
     @staticmethod
     def backward(ctx, grad_out):
-        raise NotImplementedError("forward-only build: MixMOELinear1.backward is not implemented")
+        """first_gemm_backward (mix_moe/csrc/mix_moe.h:300-388): rows of the input gradient
+        come back in flat token order and are summed per token (the reference's
+        index_add_ at 359-365)."""
+        input_buf, weight, src_row, dst_row, offsets, inv_pos = ctx.saved_tensors
+        max_rows, n_flat, fused = ctx.sizes
+        if fused:
+            raise RuntimeError("MixMOELinear1 ran with the GELU fused into its epilogue, which keeps no "
+                               "pre-activation: run the forward with fuse_gelu=False to differentiate it")
+        E = offsets.numel() - 1
+        grad_w = torch.zeros_like(weight)               # slots past E belong to no expert here
+        grad_b = torch.zeros(weight.shape[0], weight.shape[1], dtype=weight.dtype, device=weight.device)
+        g_flat, _, _ = ops.ffn1_backward(grad_out.contiguous(), input_buf, src_row, dst_row, offsets,
+                                         max_rows, weight.detach()[:E], n_flat, grad_w[:E], grad_b[:E])
+        top_k = n_flat // input_buf.shape[0]
+        ones = torch.ones(n_flat, dtype=g_flat.dtype, device=g_flat.device)
+        grad_in = ops.combine(g_flat, ones, top_k, inv_pos)
+        return grad_in, None, None, grad_w, grad_b, None
 
 
 class MixMOELinear2(Function):
@@ -71,12 +90,23 @@ class MixMOELinear2(Function):
         d = weight.shape[1]
         alloc = torch.zeros if moe_inp_block_infos.get("may_drop", True) else torch.empty
         y = alloc(n_flat, d, dtype=input_buf.dtype, device=input_buf.device)
+        ctx.save_for_backward(input_buf, weight, dst_row, offsets)
+        ctx.sizes = (max_rows,)
         return ops.ffn2(input_buf, dst_row, offsets, max_rows, weight.detach()[:E],
                         bias.detach()[:E], y)
 
     @staticmethod
     def backward(ctx, grad_out):
-        raise NotImplementedError("forward-only build: MixMOELinear2.backward is not implemented")
+        """second_gemm_backward (mix_moe/csrc/mix_moe.h:439-505); the bias gradient, which
+        the reference leaves uninitialised (489), is the column sum of the gradient rows."""
+        input_buf, weight, dst_row, offsets = ctx.saved_tensors
+        (max_rows,) = ctx.sizes
+        E = offsets.numel() - 1
+        grad_w = torch.zeros_like(weight)
+        grad_b = torch.zeros(weight.shape[0], weight.shape[1], dtype=weight.dtype, device=weight.device)
+        g_act, _, _ = ops.ffn2_backward(grad_out.contiguous(), input_buf, dst_row, offsets, max_rows,
+                                        weight.detach()[:E], grad_w[:E], grad_b[:E])
+        return g_act, None, None, grad_w, grad_b
 
 
 class FMoELinear(nn.Module):

@@ -82,7 +82,10 @@ class _Expert(nn.Module):
         return isinstance(self.activation, nn.GELU) and getattr(self.activation, "approximate", "none") == "none"
 
     def forward(self, inp, pos, moe_inp_block_infos):
-        fuse = self._gelu_is_fusable()
+        # fused into the first GEMM's epilogue only when nothing will be differentiated:
+        # the fused form keeps no pre-activation for the GELU's backward
+        wants_grad = torch.is_grad_enabled() and (inp.requires_grad or self.htoh4.weight.requires_grad)
+        fuse = self._gelu_is_fusable() and not wants_grad
         x = MixMOELinear1.apply(inp, pos, moe_inp_block_infos, self.htoh4.weight, self.htoh4.bias, fuse)
         if not fuse:
             x = self.activation(x)
@@ -175,7 +178,9 @@ class MixMOETransformerMLP(MixMOE):
     ``capacity_factor`` (not in the reference) drops overflow beyond
     ``ceil(factor * tokens * top_k / E)`` rows per expert.  ``fused=True`` runs
     the whole forward as one C-ABI call; ``fused=False`` goes stage by stage
-    through ``process_data`` and ``MixMOE.forward`` like the reference.
+    through ``process_data`` and ``MixMOE.forward`` like the reference.  When a
+    gradient is wanted (grad mode on and the input or a parameter requires it)
+    the staged path runs, whose stages carry their backward.
     """
 
     def __init__(self, gate_type, experts, model_dim: int, expert_rank, world_size,
@@ -225,7 +230,9 @@ class MixMOETransformerMLP(MixMOE):
             pos, gate_score, infos = self.async_expert_assign.result
             self.async_ = False
             output = super().forward(inp, pos, gate_score, infos)
-        elif self.fused and self.experts._gelu_is_fusable():
+        elif self.fused and self.experts._gelu_is_fusable() and not (
+                torch.is_grad_enabled() and (inp.requires_grad or
+                                             any(p.requires_grad for p in self.parameters()))):
             ex = self.experts
             with torch.no_grad():
                 output = ops.moe_forward(inp, self.gate.gate.weight.detach(),

@@ -305,8 +305,22 @@ def _backward_ws(max_rows: int, E: int, d: int, f: int, like: torch.Tensor) -> t
     return _workspace(_lib.lib().ccf_ffn_backward_workspace_bytes(int(max_rows), E, d, f), like)
 
 
+def _grad_outputs(w: torch.Tensor, grad_w: Optional[torch.Tensor], grad_b: Optional[torch.Tensor]):
+    E, n_out, _ = w.shape
+    if grad_w is None:
+        grad_w = torch.empty_like(w)
+    if grad_b is None:
+        grad_b = torch.empty(E, n_out, dtype=torch.float16, device=w.device)
+    _check(grad_w, "grad_w", dtype=torch.float16, ndim=3)
+    _check(grad_b, "grad_b", dtype=torch.float16, ndim=2)
+    if grad_w.shape != w.shape or tuple(grad_b.shape) != (E, n_out):
+        raise ValueError("gradient buffers do not match the weight shape")
+    return grad_w, grad_b
+
+
 def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optional[torch.Tensor],
-                  offsets: torch.Tensor, max_rows: int, w2: torch.Tensor):
+                  offsets: torch.Tensor, max_rows: int, w2: torch.Tensor,
+                  grad_w: Optional[torch.Tensor] = None, grad_b: Optional[torch.Tensor] = None):
     """(grad_act [max_rows, f], grad_w2 [E, d, f], grad_b2 [E, d]) of ``ffn2``.
     Rows of ``grad_act`` past ``offsets[-1]`` are zero."""
     _check(grad_y_flat, "grad_y_flat", dtype=torch.float16, ndim=2)
@@ -324,8 +338,7 @@ def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optiona
         raise ValueError("ffn2_backward: grad_y_flat has fewer rows than max_rows")
     dev = act.device
     g_act = torch.zeros(max_rows, f, dtype=torch.float16, device=dev)
-    g_w = torch.empty_like(w2)
-    g_b = torch.empty(E, d, dtype=torch.float16, device=dev)
+    g_w, g_b = _grad_outputs(w2, grad_w, grad_b)
     with torch.cuda.device(dev):
         ws = _backward_ws(max_rows, E, d, f, act)
         _lib.call("ccf_ffn2_backward", _ptr(grad_y_flat), _ptr(act), _ptr(dst_row), _ptr(offsets),
@@ -336,7 +349,8 @@ def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optiona
 
 def ffn1_backward(grad_h: torch.Tensor, x: torch.Tensor, src_row: Optional[torch.Tensor],
                   dst_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
-                  w1: torch.Tensor, n_flat: int):
+                  w1: torch.Tensor, n_flat: int,
+                  grad_w: Optional[torch.Tensor] = None, grad_b: Optional[torch.Tensor] = None):
     """(grad_x_flat [n_flat, d], grad_w1 [E, f, d], grad_b1 [E, f]) of ``ffn1`` without the
     fused GELU.  ``grad_x_flat[dst_row[j]]`` is the gradient of sorted row j; rows nothing
     maps to are zero."""
@@ -358,8 +372,7 @@ def ffn1_backward(grad_h: torch.Tensor, x: torch.Tensor, src_row: Optional[torch
         raise ValueError("ffn1_backward: n_flat smaller than max_rows")
     dev = x.device
     g_x = torch.zeros(n_flat, d, dtype=torch.float16, device=dev)
-    g_w = torch.empty_like(w1)
-    g_b = torch.empty(E, f, dtype=torch.float16, device=dev)
+    g_w, g_b = _grad_outputs(w1, grad_w, grad_b)
     with torch.cuda.device(dev):
         ws = _backward_ws(max_rows, E, d, f, x)
         _lib.call("ccf_ffn1_backward", _ptr(grad_h), _ptr(x), _ptr(src_row), _ptr(dst_row), _ptr(offsets),

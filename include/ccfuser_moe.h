@@ -297,7 +297,9 @@ int ccf_combine_backward(const void *grad_out, const void *y_flat, const void *s
                          void *grad_y_flat, void *grad_score, ccf_stream_t stream);
 
 /* Workspace of ccf_ffn1_backward / ccf_ffn2_backward (transposed weight, transposed
- * and padded activations, tile plans, bias partial sums). */
+ * and padded activations, tile plans, bias partial sums).  No counterpart in the
+ * reference, whose backward allocates its temporaries per call
+ * (mix_moe/csrc/mix_moe.h:316, 340-343, 458-460). */
 size_t ccf_ffn_backward_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn);
 
 /*

@@ -93,3 +93,48 @@ def test_ffn_backward_stages(T, d, f, E, k, cap, skew, seed):
     _close(gin, gin_ref, "grad_in")
     _close(gw1, gw1_ref, "grad_w1")
     _close(gb1, gb1_ref, "grad_b1")
+
+
+@pytest.mark.parametrize("T,d,f,E,k,cf,seed", [
+    (384, 256, 512, 4, 2, None, 10),
+    (512, 256, 512, 8, 2, 1.0, 11),          # capacity factor 1.0 drops slots
+    (200, 512, 256, 4, 1, None, 12),
+])
+def test_module_backward_matches_oracle(T, d, f, E, k, cf, seed):
+    """loss = <out, grad_out> through MixMOETransformerMLP (gate, two expert GEMMs with
+    torch's GELU between them, combine) against the oracle's closed-form gradients."""
+    from ccfuser_amd.mix_moe import MixMOETransformerMLP
+    _say(f"module backward T={T} d={d} f={f} E={E} k={k} cf={cf}")
+    p = _case(T, d, f, E, k, seed)
+    g = torch.Generator().manual_seed(2000 + seed)
+    grad_out = torch.randn(T, d, generator=g).half()
+    mlp = MixMOETransformerMLP("naive", {"num_local_expert": E, "hidden_size": f}, d, 0, 1,
+                               total_batch_size=T, top_k=k, capacity_factor=cf).half().cuda()
+    with torch.no_grad():
+        mlp.gate.gate.weight.copy_(p["wg"]); mlp.gate.gate.bias.copy_(p["bg"])
+        mlp.experts.htoh4.weight[:E].copy_(p["w1"]); mlp.experts.htoh4.bias[:E].copy_(p["b1"])
+        mlp.experts.h4toh.weight[:E].copy_(p["w2"]); mlp.experts.h4toh.bias[:E].copy_(p["b2"])
+    x = p["x"].cuda().requires_grad_(True)
+    out = mlp(x)
+    out.backward(grad_out.cuda())
+    cap = mlp._capacity(T)
+    ref = O.moe_layer_backward(p["x"], p["wg"], p["bg"], p["w1"], p["b1"], p["w2"], p["b2"], k,
+                               grad_out, capacity=cap)
+    fwd = O.moe_layer_forward(p["x"], p["wg"], p["bg"], p["w1"], p["b1"], p["w2"], p["b2"], k, capacity=cap)
+    assert O.max_abs_err(out.detach().cpu(), fwd["out"]) <= MAX_ABS
+    _close(x.grad, ref["x"], "grad_x")
+    _close(mlp.gate.gate.weight.grad, ref["wg"], "grad_wg")
+    _close(mlp.gate.gate.bias.grad, ref["bg"], "grad_bg")
+    _close(mlp.experts.htoh4.weight.grad[:E], ref["w1"], "grad_w1")
+    _close(mlp.experts.htoh4.bias.grad[:E], ref["b1"], "grad_b1")
+    _close(mlp.experts.h4toh.weight.grad[:E], ref["w2"], "grad_w2")
+    _close(mlp.experts.h4toh.bias.grad[:E], ref["b2"], "grad_b2")
+    assert float(mlp.experts.htoh4.weight.grad[E:].abs().max()) == 0.0     # slots of no expert
+    # the path overlapped with a side stream differentiates the same way
+    mlp.zero_grad()
+    x2 = p["x"].cuda().requires_grad_(True)
+    mlp.async_expert_assignment(x2)
+    mlp(x2).backward(grad_out.cuda())
+    _close(x2.grad, ref["x"], "grad_x (async)")
+    _close(mlp.experts.h4toh.weight.grad[:E], ref["w2"], "grad_w2 (async)")
+    mlp.close()
