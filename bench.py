@@ -100,6 +100,89 @@ def cpu_baseline(wl, max_seconds=30.0):
             "ms_per_step": med * 1e3}
 
 
+def bench_backward(a, wl, ops):
+    """One training step of the layer: forward in grad mode (gate, FFN1, torch GELU, FFN2,
+    combine) and the backward of all of it, K times; then the two expert-GEMM backward calls
+    alone, with events around each."""
+    import torch
+    from ccfuser_amd.mix_moe import MixMOETransformerMLP
+    t = wl.tensors
+    T, d, f, E, k = wl.tokens, wl.d_model, wl.d_ffn, wl.num_expert, wl.top_k
+    K, W = a.steps, a.warmup
+    cf = None if wl.capacity < 0 else wl.capacity * E / (T * k)
+    mlp = MixMOETransformerMLP("naive", {"num_local_expert": E, "hidden_size": f}, d, 0, 1,
+                               total_batch_size=T, top_k=k, capacity_factor=cf,
+                               popular_expert_num=0).half().cuda()
+    with torch.no_grad():
+        mlp.gate.gate.weight.copy_(t["wg"]); mlp.gate.gate.bias.copy_(t["bg"])
+        mlp.experts.htoh4.weight.copy_(t["w1"]); mlp.experts.htoh4.bias.copy_(t["b1"])
+        mlp.experts.h4toh.weight.copy_(t["w2"]); mlp.experts.h4toh.bias.copy_(t["b2"])
+    x = t["x"].cuda().requires_grad_(True)
+    gout = torch.randn(T, d, device="cuda", generator=torch.Generator(device="cuda").manual_seed(1)).half()
+
+    def step():
+        mlp.zero_grad(set_to_none=True)
+        x.grad = None
+        mlp(x).backward(gout)
+
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / K * 1e3
+
+    # the expert-GEMM backward calls alone, preallocated outputs
+    with torch.no_grad():
+        idx, _ = mlp.gate(x.detach())
+        rt = ops.route(idx.reshape(-1), E, k, wl.capacity)
+        routed = int(rt["offsets"][-1].item())
+        n = T * k
+        act = torch.randn(n, f, device="cuda").half()
+        gh = torch.randn(n, f, device="cuda").half()
+        gy = torch.randn(n, d, device="cuda").half()
+        w1, w2 = mlp.experts.htoh4.weight.detach(), mlp.experts.h4toh.weight.detach()
+        gw1, gw2 = torch.empty_like(w1), torch.empty_like(w2)
+        gb1 = torch.empty(E, f, dtype=torch.float16, device="cuda")
+        gb2 = torch.empty(E, d, dtype=torch.float16, device="cuda")
+        calls = {"ffn2_backward": lambda: ops.ffn2_backward(gy, act, rt["dst_row"], rt["offsets"], n, w2, gw2, gb2),
+                 "ffn1_backward": lambda: ops.ffn1_backward(gh, x.detach(), rt["src_row"], rt["dst_row"],
+                                                            rt["offsets"], n, w1, n, gw1, gb1)}
+        stage_ms = {}
+        for name, fn in calls.items():
+            for _ in range(max(2, W)):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(K):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            stage_ms[name] = e0.elapsed_time(e1) / K
+    gemm_flop = 4.0 * routed * d * f                    # per backward call: input-gradient + weight-gradient GEMM
+    dom = max(stage_ms, key=stage_ms.get)
+    ach = gemm_flop / (stage_ms[dom] * 1e-3) / 1e12
+    step_flop = 12.0 * routed * d * f
+    line = {
+        "metric": "moe_layer_fwd_bwd_tokens_per_s", "value": T / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"{wl.name}: {wl.description}; forward + backward", "tokens": T, "top_k": k,
+                   "num_expert": E, "d_model": d, "d_ffn": f, "routed_rows": routed,
+                   "capacity": wl.capacity, "seed": wl.seed},
+        "gemm_tflops": step_flop / (ms * 1e-3) / 1e12,
+        "frac_fp16_mfma_peak": step_flop / (ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
+        "stages_ms": stage_ms,
+        "roofline": {"kernel": f"{dom}: input-gradient and weight-gradient grouped GEMMs with their transposes",
+                     "bound": "mfma", "achieved": ach, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": ach / PEAK_FP16_TFLOPS, "traffic": None,
+                     "flop_per_launch": gemm_flop, "avg_launch_ms": stage_ms[dom]},
+    }
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -111,6 +194,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (a known HBM traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--backward", action="store_true",
+                    help="time a training step (forward + backward through the mirrored module) "
+                         "instead of the forward; prints its own metric")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU's share only: this build has no collectives or sharding "
@@ -139,6 +225,9 @@ def main():
     ev = HipEvents()
     K, W = a.steps, a.warmup
     stream = torch.cuda.current_stream().cuda_stream
+
+    if a.backward:
+        return bench_backward(a, wl, ops)
 
     if a.workload == "c4_ep_share":
         names = ("x", "seg_start", "seg_len", "seg_expert", "w1", "b1", "w2", "b2")

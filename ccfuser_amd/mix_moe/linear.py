@@ -34,6 +34,16 @@ class MixMOEInstance(object):
         return MixMOEInstance._instance
 
 
+def _param_grads(weight, E):
+    """Gradient buffers shaped like the parameter; slots past E belong to no expert here."""
+    grad_w = torch.empty_like(weight)
+    grad_b = torch.empty(weight.shape[0], weight.shape[1], dtype=weight.dtype, device=weight.device)
+    if weight.shape[0] > E:
+        grad_w[E:].zero_()
+        grad_b[E:].zero_()
+    return grad_w, grad_b
+
+
 def _routing(pos, block_infos, top_k_hint=None):
     """(src_row, dst_row, offsets, max_rows, n_flat) for the grouped GEMMs."""
     if "offsets" in block_infos:                      # planned by this package: all on device
@@ -53,7 +63,7 @@ class MixMOELinear1(Function):
         E = offsets.numel() - 1
         ctx.save_for_backward(input_buf, weight, src_row, dst_row, offsets,
                               moe_inp_block_infos.get("inv_pos"))
-        ctx.sizes = (max_rows, n_flat, bool(fuse_gelu))
+        ctx.sizes = (max_rows, n_flat, bool(fuse_gelu), bool(moe_inp_block_infos.get("may_drop", True)))
         return ops.ffn1(input_buf, src_row, offsets, max_rows, weight.detach()[:E],
                         bias.detach()[:E], gelu=bool(fuse_gelu))
 
@@ -63,15 +73,15 @@ class MixMOELinear1(Function):
         come back in flat token order and are summed per token (the reference's
         index_add_ at 359-365)."""
         input_buf, weight, src_row, dst_row, offsets, inv_pos = ctx.saved_tensors
-        max_rows, n_flat, fused = ctx.sizes
+        max_rows, n_flat, fused, may_drop = ctx.sizes
         if fused:
             raise RuntimeError("MixMOELinear1 ran with the GELU fused into its epilogue, which keeps no "
                                "pre-activation: run the forward with fuse_gelu=False to differentiate it")
         E = offsets.numel() - 1
-        grad_w = torch.zeros_like(weight)               # slots past E belong to no expert here
-        grad_b = torch.zeros(weight.shape[0], weight.shape[1], dtype=weight.dtype, device=weight.device)
+        grad_w, grad_b = _param_grads(weight, E)
         g_flat, _, _ = ops.ffn1_backward(grad_out.contiguous(), input_buf, src_row, dst_row, offsets,
-                                         max_rows, weight.detach()[:E], n_flat, grad_w[:E], grad_b[:E])
+                                         max_rows, weight.detach()[:E], n_flat, grad_w[:E], grad_b[:E],
+                                         may_drop=may_drop)
         top_k = n_flat // input_buf.shape[0]
         ones = torch.ones(n_flat, dtype=g_flat.dtype, device=g_flat.device)
         grad_in = ops.combine(g_flat, ones, top_k, inv_pos)
@@ -91,7 +101,7 @@ class MixMOELinear2(Function):
         alloc = torch.zeros if moe_inp_block_infos.get("may_drop", True) else torch.empty
         y = alloc(n_flat, d, dtype=input_buf.dtype, device=input_buf.device)
         ctx.save_for_backward(input_buf, weight, dst_row, offsets)
-        ctx.sizes = (max_rows,)
+        ctx.sizes = (max_rows, bool(moe_inp_block_infos.get("may_drop", True)))
         return ops.ffn2(input_buf, dst_row, offsets, max_rows, weight.detach()[:E],
                         bias.detach()[:E], y)
 
@@ -100,12 +110,11 @@ class MixMOELinear2(Function):
         """second_gemm_backward (mix_moe/csrc/mix_moe.h:439-505); the bias gradient, which
         the reference leaves uninitialised (489), is the column sum of the gradient rows."""
         input_buf, weight, dst_row, offsets = ctx.saved_tensors
-        (max_rows,) = ctx.sizes
+        max_rows, may_drop = ctx.sizes
         E = offsets.numel() - 1
-        grad_w = torch.zeros_like(weight)
-        grad_b = torch.zeros(weight.shape[0], weight.shape[1], dtype=weight.dtype, device=weight.device)
+        grad_w, grad_b = _param_grads(weight, E)
         g_act, _, _ = ops.ffn2_backward(grad_out.contiguous(), input_buf, dst_row, offsets, max_rows,
-                                        weight.detach()[:E], grad_w[:E], grad_b[:E])
+                                        weight.detach()[:E], grad_w[:E], grad_b[:E], may_drop=may_drop)
         return g_act, None, None, grad_w, grad_b
 
 

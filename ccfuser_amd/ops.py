@@ -320,9 +320,11 @@ def _grad_outputs(w: torch.Tensor, grad_w: Optional[torch.Tensor], grad_b: Optio
 
 def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optional[torch.Tensor],
                   offsets: torch.Tensor, max_rows: int, w2: torch.Tensor,
-                  grad_w: Optional[torch.Tensor] = None, grad_b: Optional[torch.Tensor] = None):
+                  grad_w: Optional[torch.Tensor] = None, grad_b: Optional[torch.Tensor] = None,
+                  may_drop: bool = True):
     """(grad_act [max_rows, f], grad_w2 [E, d, f], grad_b2 [E, d]) of ``ffn2``.
-    Rows of ``grad_act`` past ``offsets[-1]`` are zero."""
+    Rows of ``grad_act`` past ``offsets[-1]`` are zero (``may_drop=False`` promises there
+    are none and skips the zero fill)."""
     _check(grad_y_flat, "grad_y_flat", dtype=torch.float16, ndim=2)
     _check(act, "act", dtype=torch.float16, ndim=2)
     _check(w2, "ffn2 weight", dtype=torch.float16, ndim=3)
@@ -337,7 +339,7 @@ def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optiona
     elif grad_y_flat.shape[0] < max_rows:
         raise ValueError("ffn2_backward: grad_y_flat has fewer rows than max_rows")
     dev = act.device
-    g_act = torch.zeros(max_rows, f, dtype=torch.float16, device=dev)
+    g_act = (torch.zeros if may_drop else torch.empty)(max_rows, f, dtype=torch.float16, device=dev)
     g_w, g_b = _grad_outputs(w2, grad_w, grad_b)
     with torch.cuda.device(dev):
         ws = _backward_ws(max_rows, E, d, f, act)
@@ -350,10 +352,11 @@ def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optiona
 def ffn1_backward(grad_h: torch.Tensor, x: torch.Tensor, src_row: Optional[torch.Tensor],
                   dst_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
                   w1: torch.Tensor, n_flat: int,
-                  grad_w: Optional[torch.Tensor] = None, grad_b: Optional[torch.Tensor] = None):
+                  grad_w: Optional[torch.Tensor] = None, grad_b: Optional[torch.Tensor] = None,
+                  may_drop: bool = True):
     """(grad_x_flat [n_flat, d], grad_w1 [E, f, d], grad_b1 [E, f]) of ``ffn1`` without the
     fused GELU.  ``grad_x_flat[dst_row[j]]`` is the gradient of sorted row j; rows nothing
-    maps to are zero."""
+    maps to are zero (``may_drop=False`` promises every row is written)."""
     _check(grad_h, "grad_h", dtype=torch.float16, ndim=2)
     _check(x, "x", dtype=torch.float16, ndim=2)
     _check(w1, "ffn1 weight", dtype=torch.float16, ndim=3)
@@ -371,7 +374,7 @@ def ffn1_backward(grad_h: torch.Tensor, x: torch.Tensor, src_row: Optional[torch
     if n_flat < max_rows:
         raise ValueError("ffn1_backward: n_flat smaller than max_rows")
     dev = x.device
-    g_x = torch.zeros(n_flat, d, dtype=torch.float16, device=dev)
+    g_x = (torch.zeros if may_drop else torch.empty)(n_flat, d, dtype=torch.float16, device=dev)
     g_w, g_b = _grad_outputs(w1, grad_w, grad_b)
     with torch.cuda.device(dev):
         ws = _backward_ws(max_rows, E, d, f, x)
