@@ -214,10 +214,10 @@ __device__ __forceinline__ int tile_row_to_local(int r, int rows) {
 // Global source of every tile load of this lane for the tile of plan entry
 // `ent`: K element 0 of the (clamped) A row and B row, at this lane's K chunk.
 // Padded A rows re-read the tile's last real row, B rows past N the last row.
-template <class Cfg, bool kSeg = false>
+template <class Cfg, bool kSeg = false, bool kKN = false>
 __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v ent,
                                              const half_t *(&a_src)[Cfg::A_DMA],
-                                             const half_t *(&b_src)[Cfg::B_DMA]) {
+                                             const half_t *(&b_src)[kKN ? 2 : Cfg::B_DMA]) {
   using ML = GemmMainloop<Cfg>;
   const int row0 = ent[1], rows = ent[2], n0 = ent[3] * Cfg::BN;
   const int lda = kSeg ? p.lda : p.K, ldb = kSeg ? p.ldb : p.K;
@@ -238,11 +238,22 @@ __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v e
     else if (p.a_rows) g = p.a_rows[g];
     a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(g)) * static_cast<uint32_t>(lda) + ML::dma_chunk(r) * 8;
   }
+  if constexpr (kKN) {
+    // B is [E, K, N]: K row r of the tile, the columns LDS unit u of that row holds (N % BN == 0)
+    using R = Ring16Mainloop<Cfg, true>;
+    const int tid = threadIdx.x;
 #pragma unroll
-  for (int i = 0; i < Cfg::B_DMA; ++i) {
-    const int r = ML::dma_row(i);
-    const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-    b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r) * 8;
+    for (int i = 0; i < 2; ++i) {                          // loads 0 and 1; load i >= 2 is 16 rows below load i - 2
+      const int r = R::kn_dma_row(i, tid);
+      b_src[i] = Be + static_cast<size_t>(r) * p.N + n0 + R::kn_col(r, R::kn_dma_unit(tid));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < Cfg::B_DMA; ++i) {
+      const int r = ML::dma_row(i);
+      const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
+      b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r) * 8;
+    }
   }
 }
 
@@ -309,7 +320,7 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
   });
 }
 
-template <class Cfg, bool kGelu, bool kSeg = false>
+template <class Cfg, bool kGelu, bool kSeg = false, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_kernel(GroupedArgs p) {
   using ML = GemmMainloop<Cfg>;
@@ -322,12 +333,12 @@ grouped_gemm_kernel(GroupedArgs p) {
   const int n0 = tile_n * Cfg::BN;
 
   const half_t *a_src[Cfg::A_DMA];
-  const half_t *b_src[Cfg::B_DMA];
-  tile_sources<Cfg, kSeg>(p, ent, a_src, b_src);
+  const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
+  tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
 
   const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
   if constexpr (Cfg::SCHED == 4) {
-    Ring16Mainloop<Cfg>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, rows);
+    Ring16Mainloop<Cfg, kKN>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, rows, p.N);
     epilogue16<Cfg, kGelu>(p, e, row0, rows, n0);
     return;
   } else {
@@ -403,11 +414,12 @@ grouped_gemm_kernel(GroupedArgs p) {
 // the first barrier covers them); steps 0 .. KT-3 run with this tile's sources;
 // then the sources of the next tile are computed and the last two steps load
 // its K tiles 0 and 1.
-template <class Cfg, bool kGelu, bool kSeg = false>
+template <class Cfg, bool kGelu, bool kSeg = false, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   using ML = GemmMainloop<Cfg>;
-  using R = Ring16Mainloop<Cfg>;
+  using R = Ring16Mainloop<Cfg, kKN>;
+  const int bmul = kKN ? p.N : 1;                     // elements between K rows of a [K][N] B
   constexpr int TM = R::TM, TN = R::TN;
   const int4v *plan = reinterpret_cast<const int4v *>(p.plan);
   const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
@@ -418,12 +430,12 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
   const half_t *a_src[Cfg::A_DMA];
-  const half_t *b_src[Cfg::B_DMA];
-  tile_sources<Cfg, kSeg>(p, ent, a_src, b_src);
+  const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
+  tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
   int a_off[2], b_off[2];
   R::frag_offsets(a_off, b_off);
   half8 fa[2][TM], fb[2][TN];
-  R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg>(p, ent[0]), a_off, b_off, wave);
+  R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg>(p, ent[0]), a_off, b_off, wave, bmul);
   R::reserve();
   int phase = 0;
 
@@ -464,9 +476,9 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
     const int live_m = R::live_blocks(ent[2]);
     R::acc_settle();
     if (live_m == TM) {
-      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m);
+      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m, bmul);
     } else {
-      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m);
+      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m, bmul);
     }
     {
       // sources of the next tile (tile_sources() with the row indices already at hand); the
@@ -499,17 +511,25 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
         a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(next_row[i])) * static_cast<uint32_t>(lda) +
                    ML::dma_chunk(r, tid1) * 8;
       }
+      if constexpr (kKN) {
 #pragma unroll
-      for (int i = 0; i < Cfg::B_DMA; ++i) {
-        const int r = ML::dma_row(i, tid1);
-        const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-        b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r, tid1) * 8;
+        for (int i = 0; i < 2; ++i) {
+          const int r = R::kn_dma_row(i, tid1);
+          b_src[i] = Be + static_cast<size_t>(r) * p.N + n0 + R::kn_col(r, R::kn_dma_unit(tid1));
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < Cfg::B_DMA; ++i) {
+          const int r = ML::dma_row(i, tid1);
+          const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
+          b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r, tid1) * 8;
+        }
       }
     }
     if (live_m == TM) {
-      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m);
+      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul);
     } else {
-      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m);
+      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul);
     }
     R::acc_settle();
     epilogue16<Cfg, kGelu>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
@@ -537,6 +557,7 @@ using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 8, 4>;   // 4 wavefronts of 128x1
 
 constexpr int kDefaultVariant = 6;
 int g_variant = kDefaultVariant;
+int g_dgrad_transpose = 0;   // 1: input gradients always on a transposed copy of the weight
 
 struct Launch {
   int bm, bn, threads;
@@ -553,7 +574,11 @@ constexpr int kPersistentMinKT = 4;
   {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>,          \
    grouped_gemm_persistent_kernel<C, false>, grouped_gemm_persistent_kernel<C, true>}
 const Launch kVariants[] = {CCF_VARIANT(Cfg0), CCF_VARIANT(Cfg1), CCF_VARIANT(Cfg2), CCF_VARIANT(Cfg3),
-                            CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5), CCF_VARIANT_P(Cfg5)};
+                            CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5), CCF_VARIANT_P(Cfg5),
+                            // B stored [E, K, N] (input gradients on the stored weight); not selectable
+                            {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, false, false, true>, nullptr,
+                             grouped_gemm_persistent_kernel<Cfg5, false, false, true>, nullptr}};
+constexpr int kKnVariant = 7;
 #undef CCF_VARIANT
 #undef CCF_VARIANT_P
 
@@ -570,7 +595,7 @@ int persistent_grid() {
   }
   return cached;
 }
-constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+constexpr int kNumVariants = kKnVariant;             // what ccf_set_option accepts
 constexpr int kMinBM = 128;
 
 int max_tiles_for(int max_rows, int E, int bm) { return (max_rows + bm - 1) / bm + E; }
@@ -585,8 +610,11 @@ size_t plan_bytes(int max_rows, int E, int n_max) {
 int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets, int max_rows, int E,
                  int N, int K, const half_t *B, const half_t *bias, bool gelu, half_t *C,
                  const int32_t *c_rows, const half_t *row_scale, int32_t *plan, hipStream_t stream,
-                 const char *what) {
+                 const char *what, bool b_kn = false) {
   CCF_REQUIRE(A && offsets && B && C && plan, CCF_ERR_ARG, "%s: null pointer", what);
+  // b_kn: B is [E, K, N] (the stored weight of the layer whose input gradient this is); Cfg5 kernels only
+  CCF_REQUIRE(!b_kn || (N % Cfg5::BN == 0 && !gelu && static_cast<long long>(K) * N < (1ll << 31)), CCF_ERR_SHAPE,
+              "%s: the [K][N] weight form needs N=%d to be a multiple of %d", what, N, Cfg5::BN);
   CCF_REQUIRE(max_rows >= 0 && E > 0 && N > 0 && K > 0, CCF_ERR_ARG, "%s: bad size", what);
   CCF_REQUIRE(E <= 1024, CCF_ERR_SHAPE, "%s: num_expert=%d exceeds 1024", what, E);
   CCF_REQUIRE(K % 64 == 0, CCF_ERR_SHAPE, "%s: K=%d is not a multiple of 64", what, K);
@@ -595,7 +623,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
               "%s: operands must be 16-byte aligned", what);
   CCF_REQUIRE(!(gelu && row_scale), CCF_ERR_ARG, "%s: the GELU epilogue takes no row scale", what);
   if (max_rows == 0) return CCF_OK;
-  const Launch &v = kVariants[g_variant];
+  const Launch &v = kVariants[b_kn ? kKnVariant : g_variant];
   const int max_tiles = max_tiles_for(max_rows, E, v.bm);
   const int n_tiles_n = (N + v.bn - 1) / v.bn;
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, offsets, E, v.bm, max_tiles,
@@ -731,10 +759,13 @@ int linear_backward(const half_t *grad_out, const int32_t *g_rows, const half_t 
   CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
               "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);
   const BackwardWs ws = carve_backward(workspace, max_rows, E, d, f);
-  // input gradient
-  if (int rc = launch_transpose_weights(w, ws.w_t, E, n_out, n_in, stream)) return rc;
-  if (int rc = grouped_gemm(grad_out, g_rows, offsets, max_rows, E, n_in, n_out, ws.w_t, nullptr, false,
-                            grad_in, gi_rows, nullptr, ws.plan_rows, stream, what))
+  // input gradient: on the stored weight read as [K][N] where the shape allows, else on a transposed copy
+  const bool kn = !g_dgrad_transpose && n_in % Cfg5::BN == 0 && static_cast<long long>(n_out) * n_in < (1ll << 31);
+  if (!kn) {
+    if (int rc = launch_transpose_weights(w, ws.w_t, E, n_out, n_in, stream)) return rc;
+  }
+  if (int rc = grouped_gemm(grad_out, g_rows, offsets, max_rows, E, n_in, n_out, kn ? w : ws.w_t, nullptr,
+                            false, grad_in, gi_rows, nullptr, ws.plan_rows, stream, what, kn))
     return rc;
   // weight and bias gradients
   if (int rc = launch_kseg(offsets, E, max_rows, n_out, ws.n_blk, ws.k_seg, ws.row_off, ws.blk_row0,
@@ -761,6 +792,10 @@ extern "C" int ccf_set_option(const char *name, int value) {
     CCF_REQUIRE(value >= -1 && value < kNumVariants, CCF_ERR_ARG, "set_option: gemm_variant %d outside -1..%d",
                 value, kNumVariants - 1);
     g_variant = value < 0 ? kDefaultVariant : value;     // -1: back to the default
+    return CCF_OK;
+  }
+  if (!strcmp(name, "dgrad_transpose")) {
+    g_dgrad_transpose = value != 0;
     return CCF_OK;
   }
   if (!strcmp(name, "gate_waves")) {

@@ -111,6 +111,20 @@ __device__ __forceinline__ half8 lds_read_b128(uint32_t addr) {
   return v;
 }
 
+// 8 bytes per lane from LDS byte address addr + OFF, transposed inside each group
+// of 16 lanes: with source lane j = 4*i + r (i, r in 0..3) holding four 16-bit
+// elements c = 0..3, lane 4*r + c receives element c of source lanes r, 4 + r,
+// 8 + r, 12 + r (measured).  When source lane 4*i + r points at row i, columns
+// 4*r .. 4*r+3 of a row-major matrix, lane l receives rows 0..3 of column l:
+// four consecutive K elements of a [K][N] operand for the MFMA lane of column l.
+template <int OFF>
+__device__ __forceinline__ half4 lds_read_tr_b64(uint32_t addr) {
+  static_assert(OFF >= 0 && OFF < 65536, "ds offset");
+  half4 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+
 __device__ __forceinline__ void lds_dma16(const void *gptr, lds_char *lds_wave_base) {
   // 64 lanes x 16 bytes land at lds_wave_base + lane * 16.
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gptr,
@@ -617,9 +631,26 @@ struct RingMainloop {
 // serves every phase, the slot addresses are a few scalar adds per K tile, and a
 // caller that runs tile after tile (the persistent kernel) simply carries the
 // phase on.
-template <class Cfg>
+//
+// B_KN: the B operand is stored [K][N] (N contiguous) instead of [N][K].  Its
+// half tile then sits in LDS as 64 K rows of BN columns (512 bytes each), and a
+// lane's fragment (eight consecutive K of one column) comes from two transposing
+// 8-byte reads, four rows apart.  The sixteen rows one such read touches
+// (rows 8*g + i for the lane groups g and i = 0..3) would share banks, so the
+// 32-byte chunk a row block occupies inside its 256-byte wavefront span is
+// XORed with f(row) = row%4 + 4*((row/8)%2): two cycles per read, the minimum
+// for 512 bytes.  The XOR sits in address bits 5..7, the column block tn in the
+// same bits, so a fragment's address is the lane's base address XOR 32*tn.
+template <class Cfg, bool B_KN = false>
 struct Ring16Mainloop {
   using acc_t = float4v;
+  static constexpr int KN_PITCH = Cfg::BN * 2;                   // bytes per K row of a [K][N] half tile
+  // Source pointers a lane holds for its B tile loads.  [N][K]: one per load.  [K][N]: load i
+  // fetches K row 8*i + r0 (r0 < 8 fixed per lane), whose chunk XOR depends on i%2 only, so
+  // b_src[i] = b_src2[i % 2] + (i / 2) * 16 rows: two pointers and a scalar offset.
+  static constexpr int B_SRCS = B_KN ? 2 : Cfg::B_DMA;
+  static_assert(!B_KN || (Cfg::NW == 4 && Cfg::B_DMA % 2 == 0), "[K][N] load pattern");
+  static_assert(!B_KN || (Cfg::WTN == 128 && Cfg::BN * Cfg::BK * 2 == Cfg::B_BYTES), "[K][N] layout is written for 128-column wavefront tiles");
   static_assert(Cfg::BK == 64, "two K=32 substeps per K tile");
   static_assert(Cfg::A_BYTES == Cfg::B_BYTES, "ring slots are one size");
   static constexpr int NSLOT = 5;
@@ -658,10 +689,21 @@ struct Ring16Mainloop {
     return s;
   }
 
-  template <int N>
-  static __device__ __forceinline__ void issue_all(const half_t *const (&src)[N], int k_elem, int slot_off, int wave) {
-    static_for<0, N>([&](auto I) {
-      lds_dma16(src[I.value] + k_elem, lds() + slot_off + (I.value * Cfg::NW + wave) * 1024);
+  // Source of tile load l: src[l] + k_elem, or for the two-pointer form of a [K][N] operand
+  // src[l % 2] + k_elem + (l / 2) * 16 K rows of bmul elements.
+  template <bool KN2, int N>
+  static __device__ __forceinline__ const half_t *load_src(const half_t *const (&src)[N], int l, int k_elem, int bmul) {
+    if constexpr (KN2) {
+      return src[l & 1] + (k_elem + (l >> 1) * 16 * bmul);
+    } else {
+      return src[l] + k_elem;
+    }
+  }
+  template <bool KN2, int NLOAD, int N>
+  static __device__ __forceinline__ void issue_all(const half_t *const (&src)[N], int k_elem, int slot_off, int wave,
+                                                   int bmul = 1) {
+    static_for<0, NLOAD>([&](auto I) {
+      lds_dma16(load_src<KN2>(src, I.value, k_elem, bmul), lds() + slot_off + (I.value * Cfg::NW + wave) * 1024);
     });
   }
 
@@ -670,7 +712,14 @@ struct Ring16Mainloop {
   template <int I>
   static __device__ __forceinline__ void read_frag(half8 (&a)[TM], half8 (&b)[TN], uint32_t ra, uint32_t rb) {
     if constexpr (I < TN) {
-      b[I] = lds_read_b128<I * 16 * Cfg::CPR * 16>(rb);
+      if constexpr (B_KN) {
+        const uint32_t addr = rb ^ (I * 32);
+        const half4 lo = lds_read_tr_b64<0>(addr);
+        const half4 hi = lds_read_tr_b64<4 * KN_PITCH>(addr);
+        b[I] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      } else {
+        b[I] = lds_read_b128<I * 16 * Cfg::CPR * 16>(rb);
+      }
     } else {
       a[I - TN] = lds_read_b128<(I - TN) * 16 * Cfg::CPR * 16>(ra);
     }
@@ -722,10 +771,10 @@ struct Ring16Mainloop {
   // One substep: PER_SUB MFMAs on fragment buffer SUB; interleaved with them the
   // reads of the NEXT substep's fragments (LDS addresses ra, rb) into the other
   // buffer and the tile loads into the slot at byte offset ws.
-  template <int SUB, int NLOAD, bool FULL>
+  template <int SUB, int NLOAD, bool FULL, bool KN2 = false, int NSRC>
   static __device__ __forceinline__ void substep(half8 (&a)[2][TM], half8 (&b)[2][TN],
-                                                 const half_t *const (&src)[NLOAD], int k_elem, uint32_t ra,
-                                                 uint32_t rb, int ws, int wave, int live_m) {
+                                                 const half_t *const (&src)[NSRC], int k_elem, uint32_t ra,
+                                                 uint32_t rb, int ws, int wave, int live_m, int bmul = 1) {
     // what goes out behind MFMA i
     auto behind = [&](auto II) {
       constexpr int i = II.value;
@@ -733,7 +782,7 @@ struct Ring16Mainloop {
         read_frag<i / READ_EVERY>(a[SUB ^ 1], b[SUB ^ 1], ra, rb);
       if constexpr (i % Cfg::DMA_EVERY == 1 && i / Cfg::DMA_EVERY < NLOAD) {
         constexpr int l = i / Cfg::DMA_EVERY;
-        lds_dma16(src[l] + k_elem, lds() + ws + (l * Cfg::NW + wave) * 1024);
+        lds_dma16(load_src<KN2>(src, l, k_elem, bmul), lds() + ws + (l * Cfg::NW + wave) * 1024);
       }
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -752,13 +801,13 @@ struct Ring16Mainloop {
     });
   }
 
-  // K tile kt in ring phase ph; k2: K element offset of the K tile that the loads
-  // of this step fetch (A into the fifth slot, B into the slot A(kt) leaves).
+  // K tile kt in ring phase ph; k2 / kb2: element offset from the A / B sources of the K
+  // tile that the loads of this step fetch (A into the fifth slot, B into the slot A(kt) leaves).
   template <bool FULL>
   static __device__ __forceinline__ void step(half8 (&a)[2][TM], half8 (&b)[2][TN],
                                               const half_t *const (&a_src)[Cfg::A_DMA],
-                                              const half_t *const (&b_src)[Cfg::B_DMA], const int (&a_off)[2],
-                                              const int (&b_off)[2], int k2, int ph, int wave, int live_m) {
+                                              const half_t *const (&b_src)[B_SRCS], const int (&a_off)[2],
+                                              const int (&b_off)[2], int k2, int kb2, int ph, int wave, int live_m, int bmul) {
     const Slots s = slots_of(ph);
     const uint32_t base = lds_addr();
     frags_ready(a[0], b[0]);
@@ -772,22 +821,24 @@ struct Ring16Mainloop {
     frags_ready(a[1], b[1]);
     __builtin_amdgcn_sched_barrier(0);
     // K half 1; fetch the fragments of K half 0 of tile kt+1; load B(kt+2) into A(kt)'s slot
-    substep<1, Cfg::B_DMA, FULL>(a, b, b_src, k2, base + s.na + a_off[0], base + s.nb + b_off[0], s.a, wave,
-                                 live_m);
+    substep<1, Cfg::B_DMA, FULL, B_KN>(a, b, b_src, kb2, base + s.na + a_off[0], base + s.nb + b_off[0], s.a, wave,
+                                       live_m, bmul);
   }
 
   // `steps` consecutive K-tile steps starting in ring phase `phase` (updated).
-  // Step i loads the K tile at element offset min(k2_first + i*BK, k2_max).
+  // Step i loads the K tile at element offset min(k2_first + i*BK, k2_max); bmul: elements
+  // between consecutive K rows of a [K][N] B operand.
   template <bool FULL>
   static __device__ __forceinline__ void k_range(half8 (&a)[2][TM], half8 (&b)[2][TN],
                                                  const half_t *const (&a_src)[Cfg::A_DMA],
-                                                 const half_t *const (&b_src)[Cfg::B_DMA], const int (&a_off)[2],
+                                                 const half_t *const (&b_src)[B_SRCS], const int (&a_off)[2],
                                                  const int (&b_off)[2], int steps, int k2_first, int k2_max,
-                                                 int &phase, int wave, int live_m) {
+                                                 int &phase, int wave, int live_m, int bmul = 1) {
     int ph = phase;
     int k2 = k2_first;
     for (int i = 0; i < steps; ++i) {
-      step<FULL>(a, b, a_src, b_src, a_off, b_off, k2 < k2_max ? k2 : k2_max, ph, wave, live_m);
+      const int kc = k2 < k2_max ? k2 : k2_max;
+      step<FULL>(a, b, a_src, b_src, a_off, b_off, kc, B_KN ? kc * bmul : kc, ph, wave, live_m, bmul);
       k2 += Cfg::BK;
       ph = ph == NSLOT - 1 ? 0 : ph + 1;
     }
@@ -804,9 +855,27 @@ struct Ring16Mainloop {
     for (int sub = 0; sub < 2; ++sub) {
       const int c = sub * 4 + (lane >> 4);
       a_off[sub] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
-      b_off[sub] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
+      if constexpr (B_KN) {
+        // source lane j of its group of 16 points at K row 8*group + j/4, columns 4*(j%4) ..
+        const int j = lane & 15;
+        const int row = sub * 32 + 8 * (lane >> 4) + (j >> 2);
+        b_off[sub] = row * KN_PITCH + (wave % Cfg::WN) * (Cfg::WTN * 2) + (kn_swz(row) << 5) + ((j & 3) << 3);
+      } else {
+        b_off[sub] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
+      }
     }
   }
+  // 32-byte chunk XOR of K row `row` of a [K][N] half tile
+  static __device__ __forceinline__ int kn_swz(int row) { return (row & 3) | (((row >> 3) & 1) << 2); }
+  // Global column (elements, inside the tile's BN columns) that LDS position
+  // (row, 16-byte unit u of the row) of a [K][N] half tile holds.
+  static __device__ __forceinline__ int kn_col(int row, int u) {
+    const int chunk = u >> 1;                                     // 32-byte chunk of the row
+    return (chunk >> 3) * Cfg::WTN + (((chunk & 7) ^ kn_swz(row)) << 4) + ((u & 1) << 3);
+  }
+  // K row and 16-byte unit of tile load i of this lane for a [K][N] half tile (two rows per load).
+  static __device__ __forceinline__ int kn_dma_row(int i, int tid) { return 2 * (i * Cfg::NW + (tid >> 6)) + ((tid & 63) >> 5); }
+  static __device__ __forceinline__ int kn_dma_unit(int tid) { return tid & 31; }
 
   // The tile's rows [0, rows) are split between the two rows of wavefronts: the
   // first (rows+1)/2 sit in tile rows 0 .., the rest in tile rows WTM .., so a
@@ -835,13 +904,14 @@ struct Ring16Mainloop {
   // the fragments of K half 0 of tile 0 into a[0], b[0].
   static __device__ __forceinline__ void prologue(half8 (&a)[2][TM], half8 (&b)[2][TN],
                                                   const half_t *const (&a_src)[Cfg::A_DMA],
-                                                  const half_t *const (&b_src)[Cfg::B_DMA], int KT,
-                                                  const int (&a_off)[2], const int (&b_off)[2], int wave) {
+                                                  const half_t *const (&b_src)[B_SRCS], int KT,
+                                                  const int (&a_off)[2], const int (&b_off)[2], int wave,
+                                                  int bmul = 1) {
     const int k1 = (KT > 1 ? 1 : 0) * Cfg::BK;
-    issue_all(a_src, 0, 0 * SLOT_BYTES, wave);
-    issue_all(b_src, 0, 1 * SLOT_BYTES, wave);
-    issue_all(a_src, k1, 2 * SLOT_BYTES, wave);
-    issue_all(b_src, k1, 3 * SLOT_BYTES, wave);
+    issue_all<false, Cfg::A_DMA>(a_src, 0, 0 * SLOT_BYTES, wave);
+    issue_all<B_KN, Cfg::B_DMA>(b_src, 0, 1 * SLOT_BYTES, wave, bmul);
+    issue_all<false, Cfg::A_DMA>(a_src, k1, 2 * SLOT_BYTES, wave);
+    issue_all<B_KN, Cfg::B_DMA>(b_src, B_KN ? k1 * bmul : k1, 3 * SLOT_BYTES, wave, bmul);
     wait_vmcnt<Cfg::A_DMA + Cfg::B_DMA>();
     block_barrier();
     const uint32_t ra = lds_addr() + a_off[0], rb = lds_addr() + SLOT_BYTES + b_off[0];
@@ -850,23 +920,24 @@ struct Ring16Mainloop {
 
   // rows: real rows of this M tile (1..BM).
   static __device__ __forceinline__ void run(const half_t *const (&a_src)[Cfg::A_DMA],
-                                             const half_t *const (&b_src)[Cfg::B_DMA], int K, int rows) {
+                                             const half_t *const (&b_src)[B_SRCS], int K, int rows,
+                                             int bmul = 1) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int KT = K / Cfg::BK;
     const int live_m = live_blocks(rows);
     int a_off[2], b_off[2];
     frag_offsets(a_off, b_off);
     half8 a[2][TM], b[2][TN];
-    prologue(a, b, a_src, b_src, KT, a_off, b_off, wave);
+    prologue(a, b, a_src, b_src, KT, a_off, b_off, wave, bmul);
     int phase = 0;
     reserve();
     zero_acc();
     acc_settle();
     // past the end of K the last K tile is fetched again into slots nobody reads
     if (live_m == TM) {
-      k_range<true>(a, b, a_src, b_src, a_off, b_off, KT, 2 * Cfg::BK, (KT - 1) * Cfg::BK, phase, wave, live_m);
+      k_range<true>(a, b, a_src, b_src, a_off, b_off, KT, 2 * Cfg::BK, (KT - 1) * Cfg::BK, phase, wave, live_m, bmul);
     } else {
-      k_range<false>(a, b, a_src, b_src, a_off, b_off, KT, 2 * Cfg::BK, (KT - 1) * Cfg::BK, phase, wave, live_m);
+      k_range<false>(a, b, a_src, b_src, a_off, b_off, KT, 2 * Cfg::BK, (KT - 1) * Cfg::BK, phase, wave, live_m, bmul);
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     wait_vmcnt<0>();

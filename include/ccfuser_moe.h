@@ -55,7 +55,9 @@ const char *ccf_last_error(void);
 /*
  * Tuning knobs (no counterpart in the reference).  "gemm_variant" selects the
  * grouped-GEMM main-loop variant used by the FFN entry points; -1 restores
- * the default.  "gate_waves" (4 or 16) caps the gate
+ * the default.  "dgrad_transpose" (0/1) makes the backward's input-gradient GEMM run on a
+ * transposed copy of the weight instead of reading the stored one.
+ * "gate_waves" (4 or 16) caps the gate
  * kernel's wavefronts per workgroup.  Process-wide; not meant to be changed
  * while work is in flight.
  */

@@ -44,8 +44,22 @@ def _case(T, d, f, E, k, seed, skew=False):
     (257, 256, 1024, 3, 1, -1, False, 2),
     (64, 256, 256, 16, 2, -1, False, 3),      # every expert far below one K tile of rows
     (700, 256, 512, 4, 2, -1, True, 4),       # one large expert, one empty
+    (200, 320, 576, 4, 2, -1, False, 5),      # widths that are no multiple of 256: transposed-weight path, partial tiles
+    (1500, 512, 768, 2, 1, -1, False, 6),     # several M tiles per expert
 ])
-def test_ffn_backward_stages(T, d, f, E, k, cap, skew, seed):
+@pytest.mark.parametrize("transpose", [0, 1])
+def test_ffn_backward_stages(T, d, f, E, k, cap, skew, seed, transpose):
+    """transpose=0: input gradients read the stored weight as [K][N] where the width allows;
+    transpose=1: always on a transposed copy."""
+    from ccfuser_amd import ops
+    ops.set_option("dgrad_transpose", transpose)
+    try:
+        _ffn_backward_stages(T, d, f, E, k, cap, skew, seed)
+    finally:
+        ops.set_option("dgrad_transpose", 0)
+
+
+def _ffn_backward_stages(T, d, f, E, k, cap, skew, seed):
     from ccfuser_amd import ops
     _say(f"ffn backward T={T} d={d} f={f} E={E} k={k} cap={cap} skew={skew}")
     p = _case(T, d, f, E, k, seed, skew)
