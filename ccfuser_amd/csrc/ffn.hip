@@ -236,7 +236,11 @@ __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v e
     int g = row0 + rc;
     if constexpr (kSeg) g -= ent[0] * p.seg_rows;      // sorted row j of expert e is row j - e*seg_rows of A
     else if (p.a_rows) g = p.a_rows[g];
-    a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(g)) * static_cast<uint32_t>(lda) + ML::dma_chunk(r) * 8;
+    if constexpr (kSeg) {
+      a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(g)) * static_cast<uint32_t>(lda) + ML::dma_chunk(r) * 8;
+    } else {
+      a_src[i] = p.A + static_cast<size_t>(g) * p.K + ML::dma_chunk(r) * 8;
+    }
   }
   if constexpr (kKN) {
     // B is [E, K, N]: K row r of the tile, the columns LDS unit u of that row holds (N % BN == 0)
@@ -252,7 +256,11 @@ __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v e
     for (int i = 0; i < Cfg::B_DMA; ++i) {
       const int r = ML::dma_row(i);
       const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-      b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r) * 8;
+      if constexpr (kSeg) {
+        b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r) * 8;
+      } else {
+        b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r) * 8;
+      }
     }
   }
 }
@@ -508,8 +516,12 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
         } else {
           asm volatile("" : "+v"(next_row[i]));       // requested before step 0, complete at its barrier
         }
-        a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(next_row[i])) * static_cast<uint32_t>(lda) +
-                   ML::dma_chunk(r, tid1) * 8;
+        if constexpr (kSeg) {
+          a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(next_row[i])) * static_cast<uint32_t>(lda) +
+                     ML::dma_chunk(r, tid1) * 8;
+        } else {
+          a_src[i] = p.A + static_cast<size_t>(next_row[i]) * p.K + ML::dma_chunk(r, tid1) * 8;
+        }
       }
       if constexpr (kKN) {
 #pragma unroll
@@ -522,7 +534,11 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
         for (int i = 0; i < Cfg::B_DMA; ++i) {
           const int r = ML::dma_row(i, tid1);
           const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-          b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r, tid1) * 8;
+          if constexpr (kSeg) {
+            b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r, tid1) * 8;
+          } else {
+            b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r, tid1) * 8;
+          }
         }
       }
     }
