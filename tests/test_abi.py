@@ -74,6 +74,21 @@ def test_argument_errors_are_codes_not_crashes(lib):
     rc = lib.ccf_moe_forward(p, p, p, p, p, p, p, 4, 64, 64, 2, 1, -1, p, None, None, None, None,
                              None, p, 16, None)
     assert rc == 3
+    # backward entry points and the block planner
+    assert lib.ccf_ffn_backward_workspace_bytes(8192, 8, 4096, 14336) > 8 * 4096 * 14336 * 2
+    assert lib.ccf_ffn_backward_workspace_bytes(8192, 0, 4096, 14336) == 0
+    rc = lib.ccf_ffn2_backward(None, p, None, p, 8, 2, 64, 64, p, p, p, p, p, 1 << 30, None)
+    assert rc == 1 and b"null" in lib.ccf_last_error()
+    rc = lib.ccf_ffn2_backward(p, p, None, p, 8, 2, 64, 96, p, p, p, p, p, 1 << 30, None)
+    assert rc == 2 and b"multiples of 64" in lib.ccf_last_error()
+    rc = lib.ccf_ffn1_backward(p, p, None, None, p, 8, 2, 64, 64, p, p, p, p, p, 16, None)
+    assert rc == 3 and b"workspace" in lib.ccf_last_error()
+    rc = lib.ccf_combine_backward(p, p, p, None, 4, 2, 60, p, p, None)
+    assert rc == 2
+    rc = lib.ccf_plan_blocks(p, 2000, 64, 0, 8, p, p, p, p, p, p, p, None)
+    assert rc == 2 and b"exceeds" in lib.ccf_last_error()
+    rc = lib.ccf_plan_blocks(None, 4, 64, 0, 8, p, p, p, p, p, p, p, None)
+    assert rc == 1
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
