@@ -39,7 +39,8 @@ SIGNATURES = {
     "ccf_ffn2_forward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
     "ccf_combine_backward": (_i, [_p, _p, _p, _p, _i, _i, _i, _p, _p, _p]),
     "ccf_ffn_backward_workspace_bytes": (_sz, [_i, _i, _i, _i]),
-    "ccf_ffn2_backward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
+    "ccf_ffn1_forward_keep": (_i, [_p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
+    "ccf_ffn2_backward": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
     "ccf_ffn1_backward": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
     "ccf_moe_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "ccf_moe_forward": (_i, [_p] * 7 + [_i] * 6 + [_p] * 6 + [_p, _sz, _p]),

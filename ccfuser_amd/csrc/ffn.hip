@@ -159,6 +159,7 @@ struct GroupedArgs {
   const half_t *B;          // [E, N, K]
   const half_t *bias;       // [E, N]
   half_t *C;                // [*, N]
+  half_t *C2;               // [*, N] in sorted row order: the pre-activation, written by epilogue 2, read by epilogue 3
   const int32_t *c_rows;    // row of C for sorted row j, or NULL (identity)
   const half_t *row_scale;  // [rows] or NULL; NULL with the GELU epilogue
   const int32_t *plan;
@@ -197,6 +198,32 @@ __device__ __forceinline__ float gelu_erf(float v) {
   // 0.5*v + |v| * 0.5*erf(|z|)
   return fmaf(fabsf(v), half_erf, 0.5f * v);
 }
+
+// Derivative of the erf GELU, Phi(v) + v*phi(v), with the same erf polynomial.
+__device__ __forceinline__ float gelu_erf_grad(float v) {
+  const float u = fminf(fabsf(v), 4.2426406871192851464f);
+  const float t = u * u;
+  float q = 1.1253530e-10f * 0.5f;
+  q = fmaf(q, t, -1.0743734e-08f * 0.5f);
+  q = fmaf(q, t, 4.5365911e-07f * 0.5f);
+  q = fmaf(q, t, -1.1292428e-05f * 0.5f);
+  q = fmaf(q, t, 1.8718123e-04f * 0.5f);
+  q = fmaf(q, t, -2.2188006e-03f * 0.5f);
+  q = fmaf(q, t, 1.9636238e-02f * 0.5f);
+  q = fmaf(q, t, -1.3269384e-01f * 0.5f);
+  q = fmaf(q, t, 7.9780629e-01f * 0.5f);
+  const float half_erf = copysignf(fminf(q * u, 0.5f), v);        // 0.5 * erf(v / sqrt2)
+  // phi(v) = exp(-v^2/2) / sqrt(2 pi) = exp2(-v^2 * log2(e)/2) * 0.3989...
+  const float pdf = 0.3989422804014327f * __builtin_amdgcn_exp2f(-0.72134752044448170368f * v * v);
+  return fmaf(v, pdf, 0.5f + half_erf);
+}
+
+// Epilogue forms of the grouped GEMM.
+//   0  C = (acc + bias) * row_scale
+//   1  C = gelu(acc + bias)
+//   2  as 1, and C2 = acc + bias (the pre-activation a later backward needs)
+//   3  C = (acc + bias) * gelu'(C2): an input gradient taken straight through the GELU
+constexpr int kEpiPlain = 0, kEpiGelu = 1, kEpiGeluKeep = 2, kEpiGeluGrad = 3;
 
 // Row of the tile's row range [0, rows) that tile row r (0 .. BM-1) holds; padded
 // tile rows repeat a real one.  The 16x16x32 kernels give the upper and the
@@ -277,7 +304,7 @@ __device__ __forceinline__ int k_tiles_of(const GroupedArgs &p, int e) {
 
 // Epilogue of the 16x16x32 accumulator layout: bias (+ GELU) (+ row scale),
 // fp16, 8-byte stores through the row index.
-template <class Cfg, bool kGelu>
+template <class Cfg, int kEpi>
 __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0, int rows, int n0) {
   using R = Ring16Mainloop<Cfg>;
   constexpr int TM = R::TM, TN = R::TN;
@@ -312,25 +339,38 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
       const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
       const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
       half_t *dst = p.C + crow * p.N;
+      half_t *row2 = p.C2 + static_cast<size_t>(j) * p.N;           // epilogues 2 and 3 only
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) {
-        half4 o;
+        half4 o, pre = {0, 0, 0, 0};
+        if (kEpi == kEpiGeluGrad && col[tn] < p.N) pre = *reinterpret_cast<const half4 *>(row2 + col[tn]);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           float x = v[tn][c] + bias_v[tn][c];
-          if (kGelu) x = gelu_erf(x);                 // FFN1: no row scale
-          else x *= sc;
+          if (kEpi == kEpiGelu || kEpi == kEpiGeluKeep) {
+            if (kEpi == kEpiGeluKeep) pre[c] = static_cast<half_t>(x);
+            x = gelu_erf(x);                          // FFN1: no row scale
+          } else if (kEpi == kEpiGeluGrad) {
+            x *= gelu_erf_grad(static_cast<float>(pre[c]));
+          } else {
+            x *= sc;
+          }
           o[c] = static_cast<half_t>(x);
         }
-        if (col[tn] < p.N) *reinterpret_cast<half4 *>(dst + col[tn]) = o;
+        if (col[tn] < p.N) {
+          *reinterpret_cast<half4 *>(dst + col[tn]) = o;
+          if (kEpi == kEpiGeluKeep) *reinterpret_cast<half4 *>(row2 + col[tn]) = pre;
+        }
       }
     }
   });
 }
 
-template <class Cfg, bool kGelu, bool kSeg = false, bool kKN = false>
+template <class Cfg, int kEpi, bool kSeg = false, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_kernel(GroupedArgs p) {
+  constexpr bool kGelu = kEpi == kEpiGelu;
+  static_assert(kEpi <= kEpiGelu || Cfg::SCHED == 4, "epilogues 2 and 3 exist for the 16x16x32 kernels only");
   using ML = GemmMainloop<Cfg>;
   const int4v ent = reinterpret_cast<const int4v *>(p.plan)[blockIdx.x];
   const int e = ent[0];
@@ -347,7 +387,7 @@ grouped_gemm_kernel(GroupedArgs p) {
   const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
   if constexpr (Cfg::SCHED == 4) {
     Ring16Mainloop<Cfg, kKN>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, rows, p.N);
-    epilogue16<Cfg, kGelu>(p, e, row0, rows, n0);
+    epilogue16<Cfg, kEpi>(p, e, row0, rows, n0);
     return;
   } else {
   typename ML::acc_t acc[Cfg::TM][Cfg::TN];
@@ -422,7 +462,7 @@ grouped_gemm_kernel(GroupedArgs p) {
 // the first barrier covers them); steps 0 .. KT-3 run with this tile's sources;
 // then the sources of the next tile are computed and the last two steps load
 // its K tiles 0 and 1.
-template <class Cfg, bool kGelu, bool kSeg = false, bool kKN = false>
+template <class Cfg, int kEpi, bool kSeg = false, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   using ML = GemmMainloop<Cfg>;
@@ -548,7 +588,7 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul);
     }
     R::acc_settle();
-    epilogue16<Cfg, kGelu>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
+    epilogue16<Cfg, kEpi>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
     R::acc_settle();
     if (!has_next) break;
     ent = nent;
@@ -592,9 +632,16 @@ constexpr int kPersistentMinKT = 4;
 const Launch kVariants[] = {CCF_VARIANT(Cfg0), CCF_VARIANT(Cfg1), CCF_VARIANT(Cfg2), CCF_VARIANT(Cfg3),
                             CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5), CCF_VARIANT_P(Cfg5),
                             // B stored [E, K, N] (input gradients on the stored weight); not selectable
-                            {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, false, false, true>, nullptr,
-                             grouped_gemm_persistent_kernel<Cfg5, false, false, true>, nullptr}};
-constexpr int kKnVariant = 7;
+                            {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiPlain, false, true>,
+                             grouped_gemm_kernel<Cfg5, kEpiGeluGrad, false, true>,
+                             grouped_gemm_persistent_kernel<Cfg5, kEpiPlain, false, true>,
+                             grouped_gemm_persistent_kernel<Cfg5, kEpiGeluGrad, false, true>},
+                            // training forms of the default kernels: "plain" = GELU that keeps the
+                            // pre-activation, "gelu" slot = input gradient through the GELU; not selectable
+                            {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiGeluKeep>,
+                             grouped_gemm_kernel<Cfg5, kEpiGeluGrad>, grouped_gemm_persistent_kernel<Cfg5, kEpiGeluKeep>,
+                             grouped_gemm_persistent_kernel<Cfg5, kEpiGeluGrad>}};
+constexpr int kKnVariant = 7, kTrainVariant = 8;
 #undef CCF_VARIANT
 #undef CCF_VARIANT_P
 
@@ -624,12 +671,16 @@ size_t plan_bytes(int max_rows, int E, int n_max) {
 }
 
 int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets, int max_rows, int E,
-                 int N, int K, const half_t *B, const half_t *bias, bool gelu, half_t *C,
+                 int N, int K, const half_t *B, const half_t *bias, int epi, half_t *C,
                  const int32_t *c_rows, const half_t *row_scale, int32_t *plan, hipStream_t stream,
-                 const char *what, bool b_kn = false) {
+                 const char *what, bool b_kn = false, half_t *C2 = nullptr) {
   CCF_REQUIRE(A && offsets && B && C && plan, CCF_ERR_ARG, "%s: null pointer", what);
+  const bool gelu = epi != kEpiPlain;
+  CCF_REQUIRE(epi >= kEpiPlain && epi <= kEpiGeluGrad && (epi < kEpiGeluKeep || (C2 && aligned16(C2))), CCF_ERR_ARG,
+              "%s: epilogue %d needs the pre-activation buffer", what, epi);
   // b_kn: B is [E, K, N] (the stored weight of the layer whose input gradient this is); Cfg5 kernels only
-  CCF_REQUIRE(!b_kn || (N % Cfg5::BN == 0 && !gelu && static_cast<long long>(K) * N < (1ll << 31)), CCF_ERR_SHAPE,
+  CCF_REQUIRE(!b_kn || (N % Cfg5::BN == 0 && (epi == kEpiPlain || epi == kEpiGeluGrad) &&
+                        static_cast<long long>(K) * N < (1ll << 31)), CCF_ERR_SHAPE,
               "%s: the [K][N] weight form needs N=%d to be a multiple of %d", what, N, Cfg5::BN);
   CCF_REQUIRE(max_rows >= 0 && E > 0 && N > 0 && K > 0, CCF_ERR_ARG, "%s: bad size", what);
   CCF_REQUIRE(E <= 1024, CCF_ERR_SHAPE, "%s: num_expert=%d exceeds 1024", what, E);
@@ -639,7 +690,9 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
               "%s: operands must be 16-byte aligned", what);
   CCF_REQUIRE(!(gelu && row_scale), CCF_ERR_ARG, "%s: the GELU epilogue takes no row scale", what);
   if (max_rows == 0) return CCF_OK;
-  const Launch &v = kVariants[b_kn ? kKnVariant : g_variant];
+  const Launch &v = kVariants[b_kn ? kKnVariant : (epi >= kEpiGeluKeep ? kTrainVariant : g_variant)];
+  // which of the entry's two kernels: the K-N and training entries hold the GELU-gradient form in the second slot
+  const bool second = b_kn ? epi == kEpiGeluGrad : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu);
   const int max_tiles = max_tiles_for(max_rows, E, v.bm);
   const int n_tiles_n = (N + v.bn - 1) / v.bn;
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, offsets, E, v.bm, max_tiles,
@@ -651,6 +704,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.B = B;
   p.bias = bias;
   p.C = C;
+  p.C2 = C2;
   p.c_rows = c_rows;
   p.row_scale = row_scale;
   p.plan = plan;
@@ -664,10 +718,10 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;                // wgs is a multiple of 8
-    hipLaunchKernelGGL(gelu ? v.persistent_gelu : v.persistent_plain, dim3(static_cast<unsigned>(g)),
+    hipLaunchKernelGGL(second ? v.persistent_gelu : v.persistent_plain, dim3(static_cast<unsigned>(g)),
                        dim3(v.threads), 0, stream, p, static_cast<int>(wgs / 8));
   } else {
-    hipLaunchKernelGGL(gelu ? v.gelu : v.plain, dim3(static_cast<unsigned>(wgs)), dim3(v.threads), 0,
+    hipLaunchKernelGGL(second ? v.gelu : v.plain, dim3(static_cast<unsigned>(wgs)), dim3(v.threads), 0,
                        stream, p);
   }
   return check_launch(what);
@@ -693,6 +747,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.B = B;
   p.bias = nullptr;
   p.C = C;
+  p.C2 = nullptr;
   p.c_rows = nullptr;
   p.row_scale = nullptr;
   p.plan = plan;
@@ -762,7 +817,7 @@ int linear_backward(const half_t *grad_out, const int32_t *g_rows, const half_t 
                     const int32_t *in_rows, const int32_t *offsets, int max_rows, int E, int n_in,
                     int n_out, const half_t *w, half_t *grad_in, const int32_t *gi_rows,
                     half_t *grad_w, half_t *grad_b, void *workspace, size_t workspace_bytes,
-                    int d, int f, hipStream_t stream, const char *what) {
+                    int d, int f, hipStream_t stream, const char *what, const half_t *gelu_pre = nullptr) {
   CCF_REQUIRE(grad_out && in && offsets && w && grad_in && grad_w && grad_b, CCF_ERR_ARG,
               "%s: null pointer", what);
   CCF_REQUIRE(max_rows >= 0 && E > 0 && E <= 1024 && d > 0 && f > 0, CCF_ERR_ARG, "%s: bad size", what);
@@ -780,8 +835,11 @@ int linear_backward(const half_t *grad_out, const int32_t *g_rows, const half_t 
   if (!kn) {
     if (int rc = launch_transpose_weights(w, ws.w_t, E, n_out, n_in, stream)) return rc;
   }
+  // gelu_pre: the input was gelu(gelu_pre); the gradient is then taken through the GELU in the epilogue
+  CCF_REQUIRE(!gelu_pre || !gi_rows, CCF_ERR_ARG, "%s: the GELU gradient needs rows in expert order", what);
   if (int rc = grouped_gemm(grad_out, g_rows, offsets, max_rows, E, n_in, n_out, kn ? w : ws.w_t, nullptr,
-                            false, grad_in, gi_rows, nullptr, ws.plan_rows, stream, what, kn))
+                            gelu_pre ? kEpiGeluGrad : kEpiPlain, grad_in, gi_rows, nullptr, ws.plan_rows, stream,
+                            what, kn, const_cast<half_t *>(gelu_pre)))
     return rc;
   // weight and bias gradients
   if (int rc = launch_kseg(offsets, E, max_rows, n_out, ws.n_blk, ws.k_seg, ws.row_off, ws.blk_row0,
@@ -837,7 +895,7 @@ extern "C" int ccf_ffn1_forward(const void *x, const int32_t *src_row, const int
               "ffn1: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   return grouped_gemm(static_cast<const half_t *>(x), src_row, offsets, max_rows, num_expert, d_ffn,
                       d_model, static_cast<const half_t *>(w1), static_cast<const half_t *>(b1),
-                      apply_gelu != 0, static_cast<half_t *>(h), dst_row, nullptr,
+                      apply_gelu != 0 ? kEpiGelu : kEpiPlain, static_cast<half_t *>(h), dst_row, nullptr,
                       static_cast<int32_t *>(workspace), as_stream(stream), "ffn1");
 }
 
@@ -851,7 +909,7 @@ extern "C" int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int
   CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
               "ffn2: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   return grouped_gemm(static_cast<const half_t *>(h), src_row, offsets, max_rows, num_expert, d_model,
-                      d_ffn, static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), false,
+                      d_ffn, static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), kEpiPlain,
                       static_cast<half_t *>(y), dst_row, static_cast<const half_t *>(row_scale),
                       static_cast<int32_t *>(workspace), as_stream(stream), "ffn2");
 }
@@ -861,7 +919,24 @@ extern "C" size_t ccf_ffn_backward_workspace_bytes(int max_rows, int num_expert,
   return ccf::carve_backward(nullptr, max_rows, num_expert, d_model, d_ffn).bytes;
 }
 
-extern "C" int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const int32_t *dst_row,
+extern "C" int ccf_ffn1_forward_keep(const void *x, const int32_t *src_row, const int32_t *offsets,
+                                     int max_rows, int num_expert, int d_model, int d_ffn,
+                                     const void *w1, const void *b1, void *h_pre, void *act,
+                                     void *workspace, size_t workspace_bytes, ccf_stream_t stream) {
+  using namespace ccf;
+  const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
+  CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
+              "ffn1_keep: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  CCF_REQUIRE(h_pre && act, CCF_ERR_ARG, "ffn1_keep: null output");
+  return grouped_gemm(static_cast<const half_t *>(x), src_row, offsets, max_rows, num_expert, d_ffn,
+                      d_model, static_cast<const half_t *>(w1), static_cast<const half_t *>(b1),
+                      kEpiGeluKeep, static_cast<half_t *>(act), nullptr, nullptr,
+                      static_cast<int32_t *>(workspace), as_stream(stream), "ffn1_keep", false,
+                      static_cast<half_t *>(h_pre));
+}
+
+extern "C" int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const void *h_pre,
+                                 const int32_t *dst_row,
                                  const int32_t *offsets, int max_rows, int num_expert, int d_model,
                                  int d_ffn, const void *w2, void *grad_act, void *grad_w2,
                                  void *grad_b2, void *workspace, size_t workspace_bytes,
@@ -873,7 +948,7 @@ extern "C" int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const
                          d_ffn, d_model, static_cast<const half_t *>(w2),
                          static_cast<half_t *>(grad_act), nullptr, static_cast<half_t *>(grad_w2),
                          static_cast<half_t *>(grad_b2), workspace, workspace_bytes, d_model, d_ffn,
-                         as_stream(stream), "ffn2_backward");
+                         as_stream(stream), "ffn2_backward", static_cast<const half_t *>(h_pre));
 }
 
 extern "C" int ccf_ffn1_backward(const void *grad_h, const void *x, const int32_t *src_row,

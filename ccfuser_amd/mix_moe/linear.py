@@ -118,6 +118,50 @@ class MixMOELinear2(Function):
         return g_act, None, None, grad_w, grad_b
 
 
+class MixMOEFusedFFN(Function):
+    """Both expert linears with the erf GELU between them as one differentiable step:
+    ``y_flat[pos[j]] = gelu(x[pos[j] // k] @ W1[e]^T + b1[e]) @ W2[e]^T + b2[e]``.
+
+    The reference keeps the activation a separate torch op between its two functions
+    (mix_moe/mix_moe/transformer.py:82-91) so that autograd differentiates it; here the
+    first GEMM's epilogue applies the GELU and also stores the pre-activation, so the
+    forward has no activation pass.  The backward applies GELU' with torch's elementwise
+    kernel: the input-gradient GEMM can multiply by it in its epilogue
+    (``ops.ffn2_backward(h_pre=...)``), but that epilogue runs with the matrix pipe idle
+    and measures slower (config 3: +0.21 ms against 0.14 ms for the separate pass)."""
+
+    @staticmethod
+    def forward(ctx, input_buf, pos, moe_inp_block_infos, w1, b1, w2, b2):
+        src_row, dst_row, offsets, max_rows, n_flat = _routing(pos, moe_inp_block_infos)
+        E = offsets.numel() - 1
+        may_drop = bool(moe_inp_block_infos.get("may_drop", True))
+        act, h_pre = ops.ffn1_keep(input_buf, src_row, offsets, max_rows, w1.detach()[:E], b1.detach()[:E])
+        y = (torch.zeros if may_drop else torch.empty)(n_flat, w2.shape[1], dtype=input_buf.dtype,
+                                                       device=input_buf.device)
+        ops.ffn2(act, dst_row, offsets, max_rows, w2.detach()[:E], b2.detach()[:E], y)
+        ctx.save_for_backward(input_buf, w1, w2, act, h_pre, src_row, dst_row, offsets,
+                              moe_inp_block_infos.get("inv_pos"))
+        ctx.sizes = (max_rows, n_flat, may_drop)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        input_buf, w1, w2, act, h_pre, src_row, dst_row, offsets, inv_pos = ctx.saved_tensors
+        max_rows, n_flat, may_drop = ctx.sizes
+        E = offsets.numel() - 1
+        grad_w2, grad_b2 = _param_grads(w2, E)
+        grad_act, _, _ = ops.ffn2_backward(grad_y.contiguous(), act, dst_row, offsets, max_rows,
+                                           w2.detach()[:E], grad_w2[:E], grad_b2[:E], may_drop=may_drop)
+        grad_h = torch.ops.aten.gelu_backward(grad_act, h_pre)
+        grad_w1, grad_b1 = _param_grads(w1, E)
+        g_flat, _, _ = ops.ffn1_backward(grad_h, input_buf, src_row, dst_row, offsets, max_rows,
+                                         w1.detach()[:E], n_flat, grad_w1[:E], grad_b1[:E], may_drop=may_drop)
+        top_k = n_flat // input_buf.shape[0]
+        ones = torch.ones(n_flat, dtype=g_flat.dtype, device=g_flat.device)
+        grad_in = ops.combine(g_flat, ones, top_k, inv_pos)
+        return grad_in, None, None, grad_w1, grad_b1, grad_w2, grad_b2
+
+
 class FMoELinear(nn.Module):
     """Parameter container for E experts: weight [E, out, in], bias [E, out]
     (reference linear.py:177-233)."""

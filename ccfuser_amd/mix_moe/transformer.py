@@ -5,7 +5,7 @@ import torch.nn as nn
 
 from .. import ops
 from .layers import MixMOE
-from .linear import FMoELinear, MixMOEInstance, MixMOELinear1, MixMOELinear2
+from .linear import FMoELinear, MixMOEFusedFFN, MixMOEInstance, MixMOELinear1, MixMOELinear2
 
 _COMPAT_KEYS = ("expert_ids", "local_expert_id_indexs", "ranks", "lens", "start_addrs",
                 "remote_block_num", "total_block_num", "expert_block_ids", "expert_block_id_idxs")
@@ -77,15 +77,20 @@ class _Expert(nn.Module):
         self.htoh4 = FMoELinear(num_expert, d_model, d_hidden, bias=True, rank=rank)
         self.h4toh = FMoELinear(num_expert, d_hidden, d_model, bias=True, rank=rank)
         self.activation = activation
+        self.fuse_training = True     # False: the reference's three steps (linear, torch activation, linear)
 
     def _gelu_is_fusable(self):
         return isinstance(self.activation, nn.GELU) and getattr(self.activation, "approximate", "none") == "none"
 
     def forward(self, inp, pos, moe_inp_block_infos):
-        # fused into the first GEMM's epilogue only when nothing will be differentiated:
-        # the fused form keeps no pre-activation for the GELU's backward
         wants_grad = torch.is_grad_enabled() and (inp.requires_grad or self.htoh4.weight.requires_grad)
-        fuse = self._gelu_is_fusable() and not wants_grad
+        fuse = self._gelu_is_fusable()
+        if fuse and wants_grad and self.fuse_training:
+            # one differentiable step: the GELU and its derivative live in GEMM epilogues
+            return MixMOEFusedFFN.apply(inp, pos, moe_inp_block_infos, self.htoh4.weight, self.htoh4.bias,
+                                        self.h4toh.weight, self.h4toh.bias)
+        # the inference epilogue keeps no pre-activation, so it is used only when nothing is differentiated
+        fuse = fuse and not wants_grad
         x = MixMOELinear1.apply(inp, pos, moe_inp_block_infos, self.htoh4.weight, self.htoh4.bias, fuse)
         if not fuse:
             x = self.activation(x)

@@ -246,6 +246,31 @@ def ffn1(x: torch.Tensor, src_row: Optional[torch.Tensor], offsets: torch.Tensor
     return h
 
 
+def ffn1_keep(x: torch.Tensor, src_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
+              w1: torch.Tensor, b1: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(act, h_pre), both [max_rows, f]: ``ffn1`` with the GELU, keeping the pre-activation
+    for the backward."""
+    _check(x, "x", dtype=torch.float16, ndim=2)
+    _check_expert(w1, b1, "ffn1")
+    _check(offsets, "offsets", dtype=torch.int32, ndim=1)
+    E, f, d = w1.shape
+    if x.shape[1] != d or offsets.numel() != E + 1:
+        raise ValueError("ffn1_keep: x/offsets do not match the weight shape")
+    if src_row is not None:
+        _check(src_row, "src_row", dtype=torch.int32, ndim=1)
+        if src_row.numel() < max_rows:
+            raise ValueError("ffn1_keep: src_row shorter than max_rows")
+    elif x.shape[0] < max_rows:
+        raise ValueError("ffn1_keep: x has fewer rows than max_rows")
+    act = torch.empty(max_rows, f, dtype=x.dtype, device=x.device)
+    h_pre = torch.empty_like(act)
+    with torch.cuda.device(x.device):
+        ws = _workspace(_lib.lib().ccf_ffn_workspace_bytes(max_rows, E, d, f), x)
+        _lib.call("ccf_ffn1_forward_keep", _ptr(x), _ptr(src_row), _ptr(offsets), int(max_rows), E, d, f,
+                  _ptr(w1), _ptr(b1), _ptr(h_pre), _ptr(act), _ptr(ws), ws.numel(), _stream(x))
+    return act, h_pre
+
+
 def ffn2(h: torch.Tensor, dst_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
          w2: torch.Tensor, b2: torch.Tensor, y: torch.Tensor,
          row_scale: Optional[torch.Tensor] = None,
@@ -321,11 +346,16 @@ def _grad_outputs(w: torch.Tensor, grad_w: Optional[torch.Tensor], grad_b: Optio
 def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optional[torch.Tensor],
                   offsets: torch.Tensor, max_rows: int, w2: torch.Tensor,
                   grad_w: Optional[torch.Tensor] = None, grad_b: Optional[torch.Tensor] = None,
-                  may_drop: bool = True):
+                  may_drop: bool = True, h_pre: Optional[torch.Tensor] = None):
     """(grad_act [max_rows, f], grad_w2 [E, d, f], grad_b2 [E, d]) of ``ffn2``.
     Rows of ``grad_act`` past ``offsets[-1]`` are zero (``may_drop=False`` promises there
-    are none and skips the zero fill)."""
+    are none and skips the zero fill).  With ``h_pre`` (``act = gelu(h_pre)``, from
+    ``ffn1_keep``) the first result is the gradient of ``h_pre`` instead."""
     _check(grad_y_flat, "grad_y_flat", dtype=torch.float16, ndim=2)
+    if h_pre is not None:
+        _check(h_pre, "h_pre", dtype=torch.float16, ndim=2)
+        if h_pre.shape != act.shape:
+            raise ValueError("ffn2_backward: h_pre and act differ in shape")
     _check(act, "act", dtype=torch.float16, ndim=2)
     _check(w2, "ffn2 weight", dtype=torch.float16, ndim=3)
     _check(offsets, "offsets", dtype=torch.int32, ndim=1)
@@ -343,7 +373,7 @@ def ffn2_backward(grad_y_flat: torch.Tensor, act: torch.Tensor, dst_row: Optiona
     g_w, g_b = _grad_outputs(w2, grad_w, grad_b)
     with torch.cuda.device(dev):
         ws = _backward_ws(max_rows, E, d, f, act)
-        _lib.call("ccf_ffn2_backward", _ptr(grad_y_flat), _ptr(act), _ptr(dst_row), _ptr(offsets),
+        _lib.call("ccf_ffn2_backward", _ptr(grad_y_flat), _ptr(act), _ptr(h_pre), _ptr(dst_row), _ptr(offsets),
                   int(max_rows), E, d, f, _ptr(w2), _ptr(g_act), _ptr(g_w), _ptr(g_b), _ptr(ws),
                   ws.numel(), _stream(act))
     return g_act, g_w, g_b

@@ -298,6 +298,20 @@ int ccf_combine_backward(const void *grad_out, const void *y_flat, const void *s
                          const int32_t *inv_pos, int tokens, int top_k, int hidden,
                          void *grad_y_flat, void *grad_score, ccf_stream_t stream);
 
+/*
+ * ccf_ffn1_forward with the erf GELU, for a forward whose backward will follow:
+ * act = gelu(x[src_row] * w1[e]^T + b1[e]) as ccf_ffn1_forward(apply_gelu = 1)
+ * writes it, and the pre-activation besides, both [max_rows, d_ffn] in expert
+ * order.  The reference's first_gemm_forward (mix_moe/csrc/mix_moe.h:236-298)
+ * returns the pre-activation and applies the activation as a separate torch op
+ * (mix_moe/mix_moe/transformer.py:88), which keeps both for autograd the same way.
+ * Workspace: ccf_ffn_workspace_bytes.
+ */
+int ccf_ffn1_forward_keep(const void *x, const int32_t *src_row, const int32_t *offsets,
+                          int max_rows, int num_expert, int d_model, int d_ffn,
+                          const void *w1, const void *b1, void *h_pre, void *act,
+                          void *workspace, size_t workspace_bytes, ccf_stream_t stream);
+
 /* Workspace of ccf_ffn1_backward / ccf_ffn2_backward (transposed weight, transposed
  * and padded activations, tile plans, bias partial sums).  No counterpart in the
  * reference, whose backward allocates its temporaries per call
@@ -315,13 +329,19 @@ size_t ccf_ffn_backward_workspace_bytes(int max_rows, int num_expert, int d_mode
  * reference returns it uninitialised, 489).
  *   grad_y_flat fp16 [n_flat, d_model]  gradient of ccf_ffn2_forward's y
  *   act         fp16 [max_rows, d_ffn]  the forward's input, expert order
+ *   h_pre       fp16 [max_rows, d_ffn] or NULL.  Given (from ccf_ffn1_forward_keep,
+ *               act = gelu(h_pre)), grad_act is taken through the GELU in the GEMM's
+ *               epilogue and is the gradient of h_pre, ready for ccf_ffn1_backward
+ *               (the reference leaves the activation's backward to autograd,
+ *               mix_moe/mix_moe/transformer.py:88)
  *   dst_row, offsets                    as in the forward
  *   w2          fp16 [E, d_model, d_ffn]
  *   grad_act    fp16 [max_rows, d_ffn]  out; rows >= offsets[E] untouched
  *   grad_w2     fp16 [E, d_model, d_ffn], grad_b2 fp16 [E, d_model]  out
  * d_model and d_ffn must be multiples of 64.
  */
-int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const int32_t *dst_row,
+int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const void *h_pre,
+                      const int32_t *dst_row,
                       const int32_t *offsets, int max_rows, int num_expert, int d_model,
                       int d_ffn, const void *w2, void *grad_act, void *grad_w2,
                       void *grad_b2, void *workspace, size_t workspace_bytes,

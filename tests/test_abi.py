@@ -77,12 +77,14 @@ def test_argument_errors_are_codes_not_crashes(lib):
     # backward entry points and the block planner
     assert lib.ccf_ffn_backward_workspace_bytes(8192, 8, 4096, 14336) > 8 * 4096 * 14336 * 2
     assert lib.ccf_ffn_backward_workspace_bytes(8192, 0, 4096, 14336) == 0
-    rc = lib.ccf_ffn2_backward(None, p, None, p, 8, 2, 64, 64, p, p, p, p, p, 1 << 30, None)
+    rc = lib.ccf_ffn2_backward(None, p, None, None, p, 8, 2, 64, 64, p, p, p, p, p, 1 << 30, None)
     assert rc == 1 and b"null" in lib.ccf_last_error()
-    rc = lib.ccf_ffn2_backward(p, p, None, p, 8, 2, 64, 96, p, p, p, p, p, 1 << 30, None)
+    rc = lib.ccf_ffn2_backward(p, p, None, None, p, 8, 2, 64, 96, p, p, p, p, p, 1 << 30, None)
     assert rc == 2 and b"multiples of 64" in lib.ccf_last_error()
     rc = lib.ccf_ffn1_backward(p, p, None, None, p, 8, 2, 64, 64, p, p, p, p, p, 16, None)
     assert rc == 3 and b"workspace" in lib.ccf_last_error()
+    rc = lib.ccf_ffn1_forward_keep(p, None, p, 8, 2, 64, 64, p, p, None, p, p, 1 << 30, None)
+    assert rc == 1
     rc = lib.ccf_combine_backward(p, p, p, None, 4, 2, 60, p, p, None)
     assert rc == 2
     rc = lib.ccf_plan_blocks(p, 2000, 64, 0, 8, p, p, p, p, p, p, p, None)

@@ -94,6 +94,19 @@ def _ffn_backward_stages(T, d, f, E, k, cap, skew, seed):
     assert float(ga[R:].abs().max()) == 0.0 if R < n else True
     _close(gw2, gw2_ref, "grad_w2")
     _close(gb2, gb2_ref, "grad_b2")
+    # the same call taking the gradient through the GELU: act = gelu(h_pre)
+    hp16 = ref["h_pre"].half()
+    hp_pad = torch.zeros(n, f, dtype=torch.float16)
+    hp_pad[:R] = hp16
+    gh_ref = O.gelu_backward(ga_ref, hp16)
+    gh_fused, gw2_b, _ = ops.ffn2_backward(gy16.cuda(), a_pad.cuda(), rt["dst_row"], rt["offsets"], n,
+                                           p["w2"].cuda(), h_pre=hp_pad.cuda())
+    _close(gh_fused[:R], gh_ref, "grad_h through the GELU")
+    assert torch.equal(gw2_b, gw2)
+    # and the forward that keeps the pre-activation
+    act_k, hpre_k = ops.ffn1_keep(p["x"].cuda(), rt["src_row"], rt["offsets"], n, p["w1"].cuda(), p["b1"].cuda())
+    _close(hpre_k[:R], ref["h_pre"], "h_pre")
+    _close(act_k[:R], ref["act_fwd"], "act")
 
     # first GEMM backward
     gh16 = ref["h"].half()
@@ -151,6 +164,14 @@ def test_module_backward_matches_oracle(T, d, f, E, k, cf, seed):
     mlp(x2).backward(grad_out.cuda())
     _close(x2.grad, ref["x"], "grad_x (async)")
     _close(mlp.experts.h4toh.weight.grad[:E], ref["w2"], "grad_w2 (async)")
+    # the reference's three steps (linear, torch GELU, linear) give the same gradients
+    mlp.zero_grad()
+    mlp.experts.fuse_training = False
+    x3 = p["x"].cuda().requires_grad_(True)
+    mlp(x3).backward(grad_out.cuda())
+    _close(x3.grad, ref["x"], "grad_x (unfused)")
+    _close(mlp.experts.htoh4.weight.grad[:E], ref["w1"], "grad_w1 (unfused)")
+    _close(mlp.experts.htoh4.bias.grad[:E], ref["b1"], "grad_b1 (unfused)")
     mlp.close()
 
 
