@@ -207,3 +207,37 @@ def test_full_size_properties(workloads, name):
             h = O.gelu_exact(t["w1"][e].float() @ t["x"][tok].float() + t["b1"][e].float())
             acc += float(score_ref[tok, s]) * (t["w2"][e].float() @ h + t["b2"][e].float())
         assert (out[tok].cpu().float() - acc).abs().max() <= MAX_ABS
+
+
+def test_forward_replays_from_a_hip_graph(workloads):
+    """The whole-layer call allocates nothing and never synchronises, so it can be captured
+    into a HIP graph.  Replayed several times with fresh inputs, with eager work and
+    synchronisations between the replays, every replay must equal the eager result bit for bit
+    (routing changes with the input, so the graph's kernels must pick the new tile plan up)."""
+    from ccfuser_amd import ops
+    wl = workloads("c2_gshard", 1024)
+    t = wl.tensors
+    T, d, f, E, k = wl.tokens, wl.d_model, wl.d_ffn, wl.num_expert, wl.top_k
+    params = [t[n].cuda() for n in ("wg", "bg", "w1", "b1", "w2", "b2")]
+    x_static = t["x"].cuda().clone()
+    ws = ops.moe_workspace(T, d, f, E, k, "cuda")
+    _say(f"graph replay T={T} d={d} f={f} E={E} k={k}")
+    side = torch.cuda.Stream()                               # default priority
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):                                   # warm-up outside the capture
+            ops.moe_forward(x_static, *params, k, wl.capacity, workspace=ws)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out_static = ops.moe_forward(x_static, *params, k, wl.capacity, workspace=ws)
+    g = torch.Generator().manual_seed(99)
+    for rep in range(4):
+        x_new = torch.randn(T, d, generator=g).half().cuda()
+        eager = ops.moe_forward(x_new, *params, k, wl.capacity)      # own workspace, eager
+        torch.cuda.synchronize()
+        x_static.copy_(x_new)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, eager), f"replay {rep} differs from the eager call"
