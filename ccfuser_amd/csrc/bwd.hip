@@ -6,8 +6,10 @@
 // (`grad_out.transpose(-2, -1).contiguous()`, mix_moe.h:343, 492) for the weight
 // gradients.  Here both become calls of the one grouped GEMM, whose operands
 // must have the contraction index contiguous:
-//   * input gradients contract over the weight's rows, so the weight is
-//     transposed once per call (transpose_weights);
+//   * input gradients contract over the weight's rows: the GEMM's main loop reads
+//     the stored weight as a [K][N] operand through transposing LDS reads
+//     (gemm_tile.h, B_KN), or, for widths that are no multiple of its column
+//     tile, runs on a copy transposed here (transpose_weights);
 //   * weight gradients contract over an expert's rows, so the two activation
 //     matrices are transposed into [columns, padded rows] with every expert's
 //     rows starting at a multiple of 64 and zero-filled up to a multiple of 64
@@ -190,7 +192,25 @@ combine_backward_kernel(const half_t *__restrict__ grad_out, const half_t *__res
   if (lane == 0) grad_score[i] = static_cast<half_t>(dot);
 }
 
+// dst[0 .. n) = 0, 16 bytes per lane (n a multiple of 8 halves, dst 16-byte aligned)
+__global__ void __launch_bounds__(256)
+zero_kernel(half_t *__restrict__ dst, size_t chunks) {
+  const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (size_t c = blockIdx.x * 256ull + threadIdx.x; c < chunks; c += static_cast<size_t>(gridDim.x) * 256)
+    reinterpret_cast<half8 *>(dst)[c] = z;
+}
+
 }  // namespace
+
+// A fill kernel rather than a memset node: the call may sit inside a captured graph.
+int launch_zero(half_t *dst, size_t halves, hipStream_t stream) {
+  if (halves == 0) return CCF_OK;
+  const size_t chunks = halves / 8;
+  const size_t blocks = (chunks + 255) / 256;
+  hipLaunchKernelGGL(zero_kernel, dim3(static_cast<unsigned>(blocks < 4096 ? (blocks ? blocks : 1) : 4096)), dim3(256),
+                     0, stream, dst, chunks);
+  return check_launch("zero_kernel");
+}
 
 int padded_rows(int max_rows, int E) {
   return static_cast<int>(round_up(static_cast<size_t>(max_rows) + static_cast<size_t>(kPadK) * E, kTile));

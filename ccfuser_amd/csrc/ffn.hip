@@ -808,6 +808,15 @@ BackwardWs carve_backward(void *base, int max_rows, int E, int d, int f) {
   return w;
 }
 
+// No rows at all: the parameter gradients are zero and there is no input gradient.
+int zero_param_grads(void *grad_w, void *grad_b, int E, int n_out, int n_in, hipStream_t stream) {
+  CCF_REQUIRE(grad_w && grad_b && E > 0 && n_out > 0 && n_in > 0, CCF_ERR_ARG, "backward: null pointer or bad size");
+  CCF_REQUIRE(n_out % 8 == 0 && n_in % 8 == 0 && aligned16(grad_w) && aligned16(grad_b), CCF_ERR_SHAPE,
+              "backward: widths must be multiples of 8 and buffers 16-byte aligned");
+  if (int rc = launch_zero(static_cast<half_t *>(grad_w), static_cast<size_t>(E) * n_out * n_in, stream)) return rc;
+  return launch_zero(static_cast<half_t *>(grad_b), static_cast<size_t>(E) * n_out, stream);
+}
+
 // One expert linear layer's backward.  Forward was out[c_row(j)] = in[a_row(j)] * w[e]^T + b[e]
 // with w [E, n_out, n_in].  Given grad_out rows (through g_rows) and the forward's input rows
 // (through in_rows):
@@ -942,7 +951,7 @@ extern "C" int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const
                                  void *grad_b2, void *workspace, size_t workspace_bytes,
                                  ccf_stream_t stream) {
   using namespace ccf;
-  if (max_rows == 0) return CCF_OK;
+  if (max_rows == 0) return zero_param_grads(grad_w2, grad_b2, num_expert, d_model, d_ffn, as_stream(stream));
   return linear_backward(static_cast<const half_t *>(grad_y_flat), dst_row,
                          static_cast<const half_t *>(act), nullptr, offsets, max_rows, num_expert,
                          d_ffn, d_model, static_cast<const half_t *>(w2),
@@ -957,7 +966,7 @@ extern "C" int ccf_ffn1_backward(const void *grad_h, const void *x, const int32_
                                  void *grad_x_flat, void *grad_w1, void *grad_b1, void *workspace,
                                  size_t workspace_bytes, ccf_stream_t stream) {
   using namespace ccf;
-  if (max_rows == 0) return CCF_OK;
+  if (max_rows == 0) return zero_param_grads(grad_w1, grad_b1, num_expert, d_ffn, d_model, as_stream(stream));
   return linear_backward(static_cast<const half_t *>(grad_h), nullptr, static_cast<const half_t *>(x),
                          src_row, offsets, max_rows, num_expert, d_model, d_ffn,
                          static_cast<const half_t *>(w1), static_cast<half_t *>(grad_x_flat), dst_row,

@@ -231,3 +231,22 @@ def test_full_size_backward_properties(workloads, name):
     # no atomics anywhere: a second run gives the same bits
     _, gw2_again, gb2_again = ops.ffn2_backward(gy.cuda(), act.cuda(), rt["dst_row"], rt["offsets"], n, w2.cuda())
     assert torch.equal(gw2_again.cpu(), gw2) and torch.equal(gb2_again.cpu(), gb2)
+
+
+def test_backward_without_rows():
+    """No routed rows (every slot dropped): parameter gradients are zero, not left unwritten."""
+    from ccfuser_amd import ops
+    E, d, f = 4, 256, 512
+    w1 = torch.randn(E, f, d).half().cuda()
+    w2 = torch.randn(E, d, f).half().cuda()
+    offsets = torch.zeros(E + 1, dtype=torch.int32, device="cuda")
+    empty_f = torch.empty(0, f, dtype=torch.float16, device="cuda")
+    empty_d = torch.empty(0, d, dtype=torch.float16, device="cuda")
+    gw2 = torch.full_like(w2, 7.0)
+    gb2 = torch.full((E, d), 7.0, dtype=torch.float16, device="cuda")
+    ga, _, _ = ops.ffn2_backward(empty_d, empty_f, None, offsets, 0, w2, gw2, gb2)
+    assert ga.shape == (0, f) and float(gw2.abs().max()) == 0.0 and float(gb2.abs().max()) == 0.0
+    gw1 = torch.full_like(w1, 7.0)
+    gb1 = torch.full((E, f), 7.0, dtype=torch.float16, device="cuda")
+    gx, _, _ = ops.ffn1_backward(empty_f, empty_d, None, None, offsets, 0, w1, 0, gw1, gb1)
+    assert gx.shape == (0, d) and float(gw1.abs().max()) == 0.0 and float(gb1.abs().max()) == 0.0
