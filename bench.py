@@ -190,6 +190,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3_mixtral")
     ap.add_argument("--gemm-variant", type=int, default=None)
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="ccf_set_option before the run (tuning knobs), may repeat")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (a known HBM traffic, for scaling "
@@ -214,6 +216,9 @@ def main():
     lib = _lib.lib()
     if a.gemm_variant is not None:
         ops.set_option("gemm_variant", a.gemm_variant)
+    for item in a.option:
+        name, _, value = item.partition("=")
+        ops.set_option(name, int(value))
 
     wl = make_workload(a.workload)
     if wl.dtype != torch.float16:

@@ -170,6 +170,7 @@ struct GroupedArgs {
   // of BK, at least four K tiles) and rows e*seg_rows .. of C.  NULL otherwise.
   const int32_t *k_seg;
   int lda, ldb, seg_rows;
+  int stagger;              // persistent form: start delay per group of four workgroups, in units of 512 clocks
 };
 
 // erf-form GELU, 0.5*v*(1+erf(v/sqrt2)) = 0.5*(v + |v| erf(|z|)), z = v/sqrt2.
@@ -304,7 +305,7 @@ __device__ __forceinline__ int k_tiles_of(const GroupedArgs &p, int e) {
 
 // Epilogue of the 16x16x32 accumulator layout: bias (+ GELU) (+ row scale),
 // fp16, 8-byte stores through the row index.
-template <class Cfg, int kEpi>
+template <class Cfg, int kEpi, bool kPlainRows = false>     // kPlainRows: no row index, no row scale
 __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0, int rows, int n0) {
   using R = Ring16Mainloop<Cfg>;
   constexpr int TM = R::TM, TN = R::TN;
@@ -319,6 +320,17 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
     if (p.bias && col[tn] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn]);
 #pragma unroll
     for (int c = 0; c < 4; ++c) bias_v[tn][c] = static_cast<float>(bv[c]);
+  }
+  // Row data of all TM row blocks is looked up before the first accumulator is touched: one
+  // memory round trip for the tile instead of one per row block (padded tile rows look up the
+  // real row they repeat, so every index is in range).
+  int crow_v[TM];
+  float sc_v[TM];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int j = row0 + R::local_row(acc16_row<Cfg>(tm, tid), rows);
+    crow_v[tm] = (!kPlainRows && p.c_rows) ? p.c_rows[j] : j;
+    sc_v[tm] = (!kPlainRows && p.row_scale) ? static_cast<float>(p.row_scale[j]) : 1.0f;
   }
   static_for<0, TM>([&](auto T) {
     constexpr int tm = T.value;
@@ -336,8 +348,8 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
     });
     if (real) {
       const int j = row0 + lr;
-      const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
-      const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
+      const size_t crow = static_cast<size_t>(crow_v[tm]);
+      const float sc = sc_v[tm];
       half_t *dst = p.C + crow * p.N;
       half_t *row2 = p.C2 + static_cast<size_t>(j) * p.N;           // epilogues 2 and 3 only
 #pragma unroll
@@ -387,7 +399,7 @@ grouped_gemm_kernel(GroupedArgs p) {
   const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
   if constexpr (Cfg::SCHED == 4) {
     Ring16Mainloop<Cfg, kKN>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, rows, p.N);
-    epilogue16<Cfg, kEpi>(p, e, row0, rows, n0);
+    epilogue16<Cfg, kEpi, kSeg>(p, e, row0, rows, n0);
     return;
   } else {
   typename ML::acc_t acc[Cfg::TM][Cfg::TN];
@@ -476,6 +488,14 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   int4v ent = plan[slot_j * 8 + xcd];
   if (ent[0] < 0) return;                             // the used slots of an XCD are a prefix
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (p.stagger) {
+    // Workgroups all run tiles of equal length, so without this they reach their epilogues
+    // together and the stores of 256 tiles hit memory at once.  Four workgroups that share a
+    // weight tile (slots 4q .. 4q+3 of an XCD) keep in step; the eight such groups of an XCD
+    // start a little apart.
+    const int group = ((blockIdx.x >> 3) >> 2) & 7;
+    for (int i = 0; i < group * p.stagger; ++i) __builtin_amdgcn_s_sleep(8);
+  }
 
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
@@ -588,7 +608,7 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul);
     }
     R::acc_settle();
-    epilogue16<Cfg, kEpi>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
+    epilogue16<Cfg, kEpi, kSeg>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
     R::acc_settle();
     if (!has_next) break;
     ent = nent;
@@ -613,6 +633,7 @@ using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 8, 4>;   // 4 wavefronts of 128x1
 
 constexpr int kDefaultVariant = 6;
 int g_variant = kDefaultVariant;
+int g_stagger = 0;            // start delay between groups of workgroups in the persistent kernels (x 512 clocks)
 int g_dgrad_transpose = 0;   // 1: input gradients always on a transposed copy of the weight
 
 struct Launch {
@@ -713,6 +734,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.k_seg = nullptr;
   p.lda = p.ldb = K;
   p.seg_rows = 0;
+  p.stagger = g_stagger;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
@@ -757,6 +779,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.lda = lda;
   p.ldb = ldb;
   p.seg_rows = M;
+  p.stagger = g_stagger;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   const int grid = persistent_grid();
@@ -875,6 +898,11 @@ extern "C" int ccf_set_option(const char *name, int value) {
     CCF_REQUIRE(value >= -1 && value < kNumVariants, CCF_ERR_ARG, "set_option: gemm_variant %d outside -1..%d",
                 value, kNumVariants - 1);
     g_variant = value < 0 ? kDefaultVariant : value;     // -1: back to the default
+    return CCF_OK;
+  }
+  if (!strcmp(name, "stagger")) {
+    CCF_REQUIRE(value >= 0 && value <= 64, CCF_ERR_ARG, "set_option: stagger %d outside 0..64", value);
+    g_stagger = value;
     return CCF_OK;
   }
   if (!strcmp(name, "dgrad_transpose")) {
