@@ -170,7 +170,6 @@ struct GroupedArgs {
   // of BK, at least four K tiles) and rows e*seg_rows .. of C.  NULL otherwise.
   const int32_t *k_seg;
   int lda, ldb, seg_rows;
-  int stagger;              // persistent form: start delay per group of four workgroups, in units of 512 clocks
 };
 
 // erf-form GELU, 0.5*v*(1+erf(v/sqrt2)) = 0.5*(v + |v| erf(|z|)), z = v/sqrt2.
@@ -488,15 +487,6 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   int4v ent = plan[slot_j * 8 + xcd];
   if (ent[0] < 0) return;                             // the used slots of an XCD are a prefix
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  if (p.stagger) {
-    // Workgroups all run tiles of equal length, so without this they reach their epilogues
-    // together and the stores of 256 tiles hit memory at once.  Four workgroups that share a
-    // weight tile (slots 4q .. 4q+3 of an XCD) keep in step; the eight such groups of an XCD
-    // start a little apart.
-    const int group = ((blockIdx.x >> 3) >> 2) & 7;
-    for (int i = 0; i < group * p.stagger; ++i) __builtin_amdgcn_s_sleep(8);
-  }
-
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
   tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
@@ -633,7 +623,6 @@ using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 8, 4>;   // 4 wavefronts of 128x1
 
 constexpr int kDefaultVariant = 6;
 int g_variant = kDefaultVariant;
-int g_stagger = 0;            // start delay between groups of workgroups in the persistent kernels (x 512 clocks)
 int g_dgrad_transpose = 0;   // 1: input gradients always on a transposed copy of the weight
 
 struct Launch {
@@ -734,7 +723,6 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.k_seg = nullptr;
   p.lda = p.ldb = K;
   p.seg_rows = 0;
-  p.stagger = g_stagger;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
@@ -779,7 +767,6 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.lda = lda;
   p.ldb = ldb;
   p.seg_rows = M;
-  p.stagger = g_stagger;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   const int grid = persistent_grid();
@@ -898,11 +885,6 @@ extern "C" int ccf_set_option(const char *name, int value) {
     CCF_REQUIRE(value >= -1 && value < kNumVariants, CCF_ERR_ARG, "set_option: gemm_variant %d outside -1..%d",
                 value, kNumVariants - 1);
     g_variant = value < 0 ? kDefaultVariant : value;     // -1: back to the default
-    return CCF_OK;
-  }
-  if (!strcmp(name, "stagger")) {
-    CCF_REQUIRE(value >= 0 && value <= 64, CCF_ERR_ARG, "set_option: stagger %d outside 0..64", value);
-    g_stagger = value;
     return CCF_OK;
   }
   if (!strcmp(name, "dgrad_transpose")) {
