@@ -302,6 +302,20 @@ __device__ __forceinline__ int k_tiles_of(const GroupedArgs &p, int e) {
   }
 }
 
+// x, y: this lane's four columns of two neighbouring 16-column blocks.  Lanes 16 apart swap
+// (v_permlane16_swap: the odd 16-lane rows of the first operand with the even rows of the
+// second), so that an even row ends with columns 4q .. 4q+7 of the first block and an odd
+// row with columns 4(q-1) .. 4(q-1)+7 of the second, in order.
+__device__ __forceinline__ half8 pair_exchange(half4 x, half4 y) {
+  typedef unsigned uint2v __attribute__((ext_vector_type(2)));
+  const uint2v xv = __builtin_bit_cast(uint2v, x), yv = __builtin_bit_cast(uint2v, y);
+  const uint2v r0 = __builtin_amdgcn_permlane16_swap(xv[0], yv[0], false, false);
+  const uint2v r1 = __builtin_amdgcn_permlane16_swap(xv[1], yv[1], false, false);
+  typedef unsigned uint4v __attribute__((ext_vector_type(4)));
+  const uint4v all = {r0[0], r1[0], r0[1], r1[1]};
+  return __builtin_bit_cast(half8, all);
+}
+
 // Epilogue of the 16x16x32 accumulator layout: bias (+ GELU) (+ row scale),
 // fp16, 8-byte stores through the row index.
 template <class Cfg, int kEpi, bool kPlainRows = false>     // kPlainRows: no row index, no row scale
@@ -345,11 +359,31 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
       v[tn][2] = R::template acc_get<tm, tn, 2>();
       v[tn][3] = R::template acc_get<tm, tn, 3>();
     });
-    if (real) {
-      const int j = row0 + lr;
-      const size_t crow = static_cast<size_t>(crow_v[tm]);
-      const float sc = sc_v[tm];
-      half_t *dst = p.C + crow * p.N;
+    const int j = row0 + lr;
+    const float sc = sc_v[tm];
+    half_t *dst = p.C + static_cast<size_t>(crow_v[tm]) * p.N;
+    if constexpr (kEpi == kEpiPlain) {
+      // A lane holds columns 4q .. 4q+3 of every 16-column block (q = lane / 16).  Lanes q and
+      // q^1 of a row trade halves of a pair of blocks, after which the even one holds eight
+      // consecutive columns of the first block and the odd one of the second: half as many
+      // stores, 16 bytes each.  A store costs per instruction and cache line touched, not per
+      // byte: 64 eight-byte stores per lane took 9.6 us of a tile's epilogue, 32 sixteen-byte
+      // ones 3.4.  Every lane takes part in the exchange, padded rows included.  (The GELU
+      // epilogues are bound by their arithmetic, which hides the stores: they keep the plain form.)
+      const int q = (tid & 63) >> 4;
+#pragma unroll
+      for (int tp = 0; tp < TN / 2; ++tp) {
+        half4 o[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            o[h][c] = static_cast<half_t>((v[2 * tp + h][c] + bias_v[2 * tp + h][c]) * sc);
+        const int c16 = col[2 * tp] - 4 * q + (q & 1) * 16 + 4 * (q & 2);   // first of this lane's 8 columns
+        const half8 out = pair_exchange(o[0], o[1]);
+        if (real && c16 < p.N) *reinterpret_cast<half8 *>(dst + c16) = out;
+      }
+    } else if (real) {
       half_t *row2 = p.C2 + static_cast<size_t>(j) * p.N;           // epilogues 2 and 3 only
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) {
@@ -358,13 +392,11 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           float x = v[tn][c] + bias_v[tn][c];
-          if (kEpi == kEpiGelu || kEpi == kEpiGeluKeep) {
-            if (kEpi == kEpiGeluKeep) pre[c] = static_cast<half_t>(x);
-            x = gelu_erf(x);                          // FFN1: no row scale
-          } else if (kEpi == kEpiGeluGrad) {
+          if (kEpi == kEpiGeluGrad) {
             x *= gelu_erf_grad(static_cast<float>(pre[c]));
           } else {
-            x *= sc;
+            if (kEpi == kEpiGeluKeep) pre[c] = static_cast<half_t>(x);
+            x = gelu_erf(x);                          // FFN1: no row scale
           }
           o[c] = static_cast<half_t>(x);
         }
