@@ -318,7 +318,7 @@ __device__ __forceinline__ half8 pair_exchange(half4 x, half4 y) {
 
 // Epilogue of the 16x16x32 accumulator layout: bias (+ GELU) (+ row scale),
 // fp16, 8-byte stores through the row index.
-template <class Cfg, int kEpi, bool kPlainRows = false>     // kPlainRows: no row index, no row scale
+template <class Cfg, int kEpi, bool kPlainRows = false>     // kPlainRows: no row index, no row scale, no bias
 __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0, int rows, int n0) {
   using R = Ring16Mainloop<Cfg>;
   constexpr int TM = R::TM, TN = R::TN;
@@ -378,7 +378,8 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
         for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int c = 0; c < 4; ++c)
-            o[h][c] = static_cast<half_t>((v[2 * tp + h][c] + bias_v[2 * tp + h][c]) * sc);
+            o[h][c] = static_cast<half_t>(kPlainRows ? v[2 * tp + h][c]          // weight gradients: no bias, no scale
+                                                     : (v[2 * tp + h][c] + bias_v[2 * tp + h][c]) * sc);
         const int c16 = col[2 * tp] - 4 * q + (q & 1) * 16 + 4 * (q & 2);   // first of this lane's 8 columns
         const half8 out = pair_exchange(o[0], o[1]);
         if (real && c16 < p.N) *reinterpret_cast<half8 *>(dst + c16) = out;
