@@ -31,8 +31,8 @@ PEAK_HBM_GBS = 8000.0
 # profiles/grouped_gemm_<workload>_hbm_traffic.txt.  Counters cannot be read from inside a
 # normal run, so a workload without a profile reports null.
 MEASURED_TRAFFIC_KIB = {
-    ("c3_mixtral", "ffn1"): {"FETCH_SIZE": 905033.9, "WRITE_SIZE": 229379.0},
-    ("c3_mixtral", "ffn2"): {"FETCH_SIZE": 1026989.9, "WRITE_SIZE": 65536.2},
+    ("c3_mixtral", "ffn1"): {"FETCH_SIZE": 923101.2, "WRITE_SIZE": 229378.9},
+    ("c3_mixtral", "ffn2"): {"FETCH_SIZE": 1026486.6, "WRITE_SIZE": 65536.1},
 }
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 
