@@ -172,20 +172,19 @@ struct GroupedArgs {
   int lda, ldb, seg_rows;
 };
 
-// erf-form GELU, 0.5*v*(1+erf(v/sqrt2)) = 0.5*(v + |v| erf(|z|)), z = v/sqrt2.
-// erf(|z|) is an odd minimax polynomial z*Q(z^2) (degree 8 in z^2, fitted on
-// [0, 3]; beyond 3, where 1 - erf < 2.3e-5, z is clamped and the result capped
-// at 1).  Measured in fp32 against the exact function over [-8, 8]: erf within
-// 2.8e-5, GELU within 6.2e-5 absolute, an eighth of the fp16 rounding step of
-// a result of magnitude 1.  14 full-rate instructions and no transcendental
-// (the library erff is ~40, the exp-based form 15 plus rcp and exp at quarter
-// rate); the FFN1 epilogue applies it to 256 values per lane and tile.
+// erf-form GELU, v * Phi(v) with Phi(v) = 0.5 + 0.5*erf(v/sqrt2) = 0.5 + u*Q(u^2), u = v
+// clamped to +-3*sqrt2 (beyond it 1 - erf < 2.3e-5).  0.5*erf(u/sqrt2) is an odd minimax
+// polynomial u*Q(u^2) of degree 8 in u^2, fitted on [0, 3] in z = u/sqrt2 with the 1/sqrt2
+// and the 0.5 folded into the coefficients.  Measured in fp32 against the exact function:
+// within 1.4e-5 for |v| <= 2, 5.9e-5 for |v| <= 8 (at -8 the result is -2e-5 instead of -0),
+// an eighth of the fp16 rounding step of a result of magnitude 1.  12 full-rate instructions
+// with the fp16 conversion and no transcendental (the library erff is ~40, the exp-based form
+// 15 plus rcp and exp at quarter rate); the FFN1 epilogue applies it to 256 values per lane
+// and tile and is bound by this arithmetic.
 __device__ __forceinline__ float gelu_erf(float v) {
-  // u = |v| clamped at 3*sqrt2; the 1/sqrt2 of z = u/sqrt2 is folded into the coefficients:
-  // erf(z) = u * Q'(u^2) with c'_k = c_k / sqrt2^(2k+1)
-  const float u = fminf(fabsf(v), 4.2426406871192851464f);
+  const float u = __builtin_amdgcn_fmed3f(v, -4.2426406871192851464f, 4.2426406871192851464f);
   const float t = u * u;
-  float q = 1.1253530e-10f * 0.5f;                 // 0.5 * c'_8 .. the 0.5 of GELU is folded in too
+  float q = 1.1253530e-10f * 0.5f;
   q = fmaf(q, t, -1.0743734e-08f * 0.5f);
   q = fmaf(q, t, 4.5365911e-07f * 0.5f);
   q = fmaf(q, t, -1.1292428e-05f * 0.5f);
@@ -194,9 +193,7 @@ __device__ __forceinline__ float gelu_erf(float v) {
   q = fmaf(q, t, 1.9636238e-02f * 0.5f);
   q = fmaf(q, t, -1.3269384e-01f * 0.5f);
   q = fmaf(q, t, 7.9780629e-01f * 0.5f);
-  const float half_erf = fminf(q * u, 0.5f);       // 0.5 * erf(|z|)
-  // 0.5*v + |v| * 0.5*erf(|z|)
-  return fmaf(fabsf(v), half_erf, 0.5f * v);
+  return v * fmaf(u, q, 0.5f);
 }
 
 // Derivative of the erf GELU, Phi(v) + v*phi(v), with the same erf polynomial.
