@@ -828,23 +828,24 @@ BackwardWs carve_backward(void *base, int max_rows, int E, int d, int f) {
   const int big = d > f ? d : f;
   w.ld_t = padded_rows(max_rows, E);
   w.n_blk = w.ld_t / 64;
-  char *p = static_cast<char *>(base);
+  // offsets are added to the base as integers: the size query passes a null base
+  uintptr_t p = reinterpret_cast<uintptr_t>(base);
   auto take = [&](size_t bytes) {
-    char *r = p;
+    void *r = reinterpret_cast<void *>(p);
     p += round_up(bytes, 256);
     return r;
   };
-  w.plan_rows = reinterpret_cast<int32_t *>(take(plan_bytes(max_rows, E, big)));
-  w.plan_w = reinterpret_cast<int32_t *>(take(plan_bytes(E * big, E, big)));
-  w.k_seg = reinterpret_cast<int32_t *>(take(sizeof(int32_t) * (E + 1)));
-  w.row_off = reinterpret_cast<int32_t *>(take(sizeof(int32_t) * (E + 1)));
-  w.blk_row0 = reinterpret_cast<int32_t *>(take(sizeof(int32_t) * w.n_blk));
-  w.blk_cnt = reinterpret_cast<int32_t *>(take(sizeof(int32_t) * w.n_blk));
-  w.w_t = reinterpret_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(E) * d * f));
-  w.a_t = reinterpret_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(big) * w.ld_t));
-  w.b_t = reinterpret_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(big) * w.ld_t));
-  w.partial = reinterpret_cast<float *>(take(sizeof(float) * static_cast<size_t>(w.n_blk) * big));
-  w.bytes = static_cast<size_t>(p - static_cast<char *>(base));
+  w.plan_rows = static_cast<int32_t *>(take(plan_bytes(max_rows, E, big)));
+  w.plan_w = static_cast<int32_t *>(take(plan_bytes(E * big, E, big)));
+  w.k_seg = static_cast<int32_t *>(take(sizeof(int32_t) * (E + 1)));
+  w.row_off = static_cast<int32_t *>(take(sizeof(int32_t) * (E + 1)));
+  w.blk_row0 = static_cast<int32_t *>(take(sizeof(int32_t) * w.n_blk));
+  w.blk_cnt = static_cast<int32_t *>(take(sizeof(int32_t) * w.n_blk));
+  w.w_t = static_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(E) * d * f));
+  w.a_t = static_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(big) * w.ld_t));
+  w.b_t = static_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(big) * w.ld_t));
+  w.partial = static_cast<float *>(take(sizeof(float) * static_cast<size_t>(w.n_blk) * big));
+  w.bytes = static_cast<size_t>(p - reinterpret_cast<uintptr_t>(base));
   return w;
 }
 
