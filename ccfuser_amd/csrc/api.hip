@@ -174,12 +174,17 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
                              w.ffn_ws, w.ffn_bytes, stream)))
     return rc;
   mark_stage(3, st);
+  // top-1 without a capacity limit: every token has one slot, its score is exactly 1 (the softmax of
+  // one logit) and its flat row is its token row, so FFN2 writes the layer output itself
+  const bool direct = top_k == 1 && capacity < 0;
   if ((rc = ccf_ffn2_forward(w.h, nullptr, w.dst_row, w.offsets, n, num_expert, d_model, d_ffn, w2, b2,
-                             nullptr, w.y_flat, w.ffn_ws, w.ffn_bytes, stream)))
+                             nullptr, direct ? out : w.y_flat, w.ffn_ws, w.ffn_bytes, stream)))
     return rc;
   mark_stage(4, st);
-  if ((rc = ccf_combine(w.y_flat, w.score, w.inv_pos, out, tokens, top_k, d_model, stream)))
-    return rc;
+  if (!direct) {
+    if ((rc = ccf_combine(w.y_flat, w.score, w.inv_pos, out, tokens, top_k, d_model, stream)))
+      return rc;
+  }
   mark_stage(5, st);
   // optional copies of the routing results (device to device, same stream)
   hipError_t e = hipSuccess;

@@ -241,3 +241,25 @@ def test_forward_replays_from_a_hip_graph(workloads):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out_static, eager), f"replay {rep} differs from the eager call"
+
+
+def test_top1_output_written_by_ffn2_equals_the_staged_path(workloads):
+    """With top-1 and no capacity limit the fused call lets FFN2 write the layer output (the
+    score is exactly 1); the staged path, which runs the combine kernel, must give the same bits."""
+    from ccfuser_amd import ops
+    wl = workloads("c5_skewed", 2048)
+    t = wl.tensors
+    assert wl.top_k == 1 and wl.capacity < 0
+    args = [t[n].cuda() for n in ("x", "wg", "bg", "w1", "b1", "w2", "b2")]
+    _say(f"top-1 direct output T={wl.tokens}")
+    fused, r = ops.moe_forward(*args, 1, -1, return_routing=True)
+    assert bool((r["score"] == 1.0).all())
+    x, wg, bg, w1, b1, w2, b2 = args
+    idx, score = ops.gate_topk_softmax(x, wg, bg, 1)
+    rt = ops.route(idx.reshape(-1), wl.num_expert, 1, -1)
+    n = wl.tokens
+    h = ops.ffn1(x, rt["src_row"], rt["offsets"], n, w1, b1, gelu=True)
+    y = torch.empty(n, wl.d_model, dtype=torch.float16, device="cuda")
+    ops.ffn2(h, rt["dst_row"], rt["offsets"], n, w2, b2, y)
+    staged = ops.combine(y, score.reshape(-1), 1, rt["inv_pos"])
+    assert torch.equal(fused, staged)
