@@ -250,3 +250,20 @@ def test_backward_without_rows():
     gb1 = torch.full((E, f), 7.0, dtype=torch.float16, device="cuda")
     gx, _, _ = ops.ffn1_backward(empty_f, empty_d, None, None, offsets, 0, w1, 0, gw1, gb1)
     assert gx.shape == (0, d) and float(gw1.abs().max()) == 0.0 and float(gb1.abs().max()) == 0.0
+
+
+def _random_shapes(count, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    out = []
+    for i in range(count):
+        E = r(1, 9)
+        out.append((r(1, 600), 64 * r(1, 10), 64 * r(1, 10), E, min(r(1, 3), E), [-1, -1, r(0, 200)][r(0, 2)], 100 + i))
+    return out
+
+
+@pytest.mark.parametrize("T,d,f,E,k,cap,seed", _random_shapes(10, 4242))
+def test_ffn_backward_random_shapes(T, d, f, E, k, cap, seed):
+    """Widths from 64 to 640 in steps of 64 (one K tile, partial M and N tiles, both weight
+    forms), 1 to 600 tokens, 1 to 9 experts, top-1 to top-3, with and without capacity."""
+    _ffn_backward_stages(T, d, f, E, k, cap, False, seed)
