@@ -289,11 +289,29 @@ __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v e
   }
 }
 
+// Loads through the scalar cache of data no kernel in flight writes (the tile plan, the K
+// ranges), complete on return.  Inside the tile loop the compiler would use vector loads for
+// them (the kernel's own stores might alias), and a vector load queues behind the epilogue's
+// stores.
+typedef int int2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ int4v scalar_load4(const int4v *q) {
+  int4v r;
+  asm volatile("s_load_dwordx4 %0, %1, 0x0\n s_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(q) : "memory");
+  return r;
+}
+__device__ __forceinline__ int2v scalar_load2(const int32_t *q) {
+  int2v r;
+  asm volatile("s_load_dwordx2 %0, %1, 0x0\n s_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(q) : "memory");
+  return r;
+}
+
 // K tiles of expert e's contraction.
 template <class Cfg, bool kSeg>
 __device__ __forceinline__ int k_tiles_of(const GroupedArgs &p, int e) {
   if constexpr (kSeg) {
-    return __builtin_amdgcn_readfirstlane((p.k_seg[e + 1] - p.k_seg[e]) / Cfg::BK);
+    const int eu = __builtin_amdgcn_readfirstlane(e);
+    const int2v r = scalar_load2(p.k_seg + eu);
+    return (r[1] - r[0]) / Cfg::BK;
   } else {
     return p.K / Cfg::BK;
   }
@@ -516,6 +534,14 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   if (slot_j >= slots_per_xcd) return;
   int4v ent = plan[slot_j * 8 + xcd];
   if (ent[0] < 0) return;                             // the used slots of an XCD are a prefix
+  // Plan entries are read through uniform indices (scalar loads, which do not queue behind the
+  // epilogue's stores) and one tile ahead of their use: `ahead` is the entry after the next one.
+  auto entry_at = [&](int j) {
+    int4v t = int4v{-1, 0, 0, 0};
+    if (j < slots_per_xcd) t = scalar_load4(plan + __builtin_amdgcn_readfirstlane(j * 8 + xcd));
+    return t;
+  };
+  int4v ahead = entry_at(slot_j + stride);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
@@ -530,15 +556,9 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   for (;;) {
     // the entry after this one; without one, the tail steps re-fetch this tile's first K tiles
     const int nj = slot_j + stride;
-    int4v nent = ent;
-    bool has_next = false;
-    if (nj < slots_per_xcd) {
-      const int4v t = plan[nj * 8 + xcd];
-      if (t[0] >= 0) {
-        nent = t;
-        has_next = true;
-      }
-    }
+    const bool has_next = ahead[0] >= 0;
+    const int4v nent = has_next ? ahead : ent;
+    ahead = has_next ? entry_at(nj + stride) : ahead;  // used by the next tile: its latency hides under this one
     const int n_row0 = nent[1], n_rows = nent[2];
     const int KT = k_tiles_of<Cfg, kSeg>(p, ent[0]);
     const int k_end = KT * Cfg::BK;
