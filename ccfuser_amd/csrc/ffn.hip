@@ -170,6 +170,9 @@ struct GroupedArgs {
   // of BK, at least four K tiles) and rows e*seg_rows .. of C.  NULL otherwise.
   const int32_t *k_seg;
   int lda, ldb, seg_rows;
+  // split-K tail (see tail_kernel): header {tiles, parts per tile}, entries, fp32 partial tiles
+  const int32_t *tail;
+  float *partial;
 };
 
 // erf-form GELU, v * Phi(v) with Phi(v) = 0.5 + 0.5*erf(v/sqrt2) = 0.5 + u*Q(u^2), u = v
@@ -658,6 +661,168 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   wait_vmcnt<0>();
 }
 
+
+// ---- split-K tail -----------------------------------------------------------------
+// Tiles all take about the same time, so a launch whose tile count is no multiple of the
+// workgroup count ends with a round in which most CUs idle: config 3's FFN2 has 592 tiles for
+// 256 workgroups, 2.3 rounds that cost 3.  tail_kernel takes the tiles of each XCD's last,
+// partly filled round out of the plan and, when they are few enough to matter (at most half
+// a round), cuts each into S parts along K, S = workgroups / tiles (at most 8, at least four
+// K tiles per part).  The parts run as one more launch, one workgroup each, and leave raw
+// fp32 accumulators in a scratch area; splitk_reduce adds a tile's parts in part order and
+// applies the epilogue.  The area sits in front of the plan in the caller's workspace:
+//   [0, 16)              header: tiles R, parts S
+//   [256, 256 + 16*256)  entries {expert, row0, rows, tile_n | part << 16 | S << 24}, part-major per tile
+//   [kTailHead, ...)     256 partial tiles of 256 x 256 fp32
+constexpr int kTailMaxParts = 256;
+constexpr size_t kTailHead = 256 + 16 * kTailMaxParts;
+constexpr size_t kTailBytes = kTailHead + static_cast<size_t>(kTailMaxParts) * 256 * 256 * 4;
+
+__global__ void __launch_bounds__(256)
+tail_kernel(int32_t *__restrict__ plan, int slots_per_xcd, int persistent_wgs, int k_tiles,
+            int32_t *__restrict__ tail) {
+  __shared__ int s_used[8], s_full[8], s_base[9];
+  const int spx = persistent_wgs >> 3;                 // persistent workgroups per XCD
+  int4v *entry = reinterpret_cast<int4v *>(plan);
+  int4v *tent = reinterpret_cast<int4v *>(tail + 64);
+  if (threadIdx.x < 8) {
+    // the used slots of an XCD are a prefix: first slot j with an idle entry
+    const int x = threadIdx.x;
+    int lo = 0, hi = slots_per_xcd;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (entry[mid * 8 + x][0] >= 0) lo = mid + 1; else hi = mid;
+    }
+    s_used[x] = lo;
+    s_full[x] = lo / spx * spx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int r = 0;
+    for (int x = 0; x < 8; ++x) { s_base[x] = r; r += s_used[x] - s_full[x]; }
+    s_base[8] = r;
+  }
+  __syncthreads();
+  const int R = s_base[8];
+  int S = R > 0 ? persistent_wgs / R : 0;
+  S = S > 8 ? 8 : S;
+  S = S > k_tiles / 4 ? k_tiles / 4 : S;
+  if (R == 0 || R * 2 > persistent_wgs || S < 2 || R * S > kTailMaxParts) {
+    if (threadIdx.x == 0) { tail[0] = 0; tail[1] = 0; }
+    return;                                            // the plan stays as it is
+  }
+  if (threadIdx.x == 0) { tail[0] = R; tail[1] = S; }
+  for (int x = 0; x < 8; ++x) {
+    const int rx = s_used[x] - s_full[x];
+    for (int i = threadIdx.x; i < rx; i += blockDim.x) {
+      const int4v e = entry[(s_full[x] + i) * 8 + x];
+      entry[(s_full[x] + i) * 8 + x] = int4v{-1, 0, 0, 0};
+      const int t = s_base[x] + i;
+      for (int part = 0; part < S; ++part) tent[t * S + part] = int4v{e[0], e[1], e[2], e[3] | (part << 16) | (S << 24)};
+    }
+  }
+}
+
+// K tiles [first, first + count) of part `part` of S over k_tiles K tiles.
+__device__ __forceinline__ void part_range(int k_tiles, int part, int S, int &first, int &count) {
+  const int base = k_tiles / S, rem = k_tiles % S;
+  count = base + (part < rem ? 1 : 0);
+  first = part * base + (part < rem ? part : rem);
+}
+
+// One part of one tail tile per workgroup: the main loop over its K range, raw accumulators out.
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
+grouped_gemm_tail_kernel(GroupedArgs p) {
+  using R = Ring16Mainloop<Cfg>;
+  const int tiles = p.tail[0], S = p.tail[1];
+  if (static_cast<int>(blockIdx.x) >= tiles * S) return;
+  int4v ent = reinterpret_cast<const int4v *>(p.tail + 64)[blockIdx.x];
+  const int part = (ent[3] >> 16) & 0xff;
+  ent[3] &= 0xffff;
+  int first, count;
+  part_range(p.K / Cfg::BK, part, S, first, count);
+  const half_t *a_src[Cfg::A_DMA];
+  const half_t *b_src[Cfg::B_DMA];
+  tile_sources<Cfg>(p, ent, a_src, b_src);
+#pragma unroll
+  for (int i = 0; i < Cfg::A_DMA; ++i) a_src[i] += first * Cfg::BK;
+#pragma unroll
+  for (int i = 0; i < Cfg::B_DMA; ++i) b_src[i] += first * Cfg::BK;
+  R::run(a_src, b_src, count * Cfg::BK, ent[2]);
+  float *out = p.partial + static_cast<size_t>(blockIdx.x) * (Cfg::BM * Cfg::BN);
+  const int tid = fresh_tid();
+  static_for<0, R::TM>([&](auto T) {
+    constexpr int tm = T.value;
+    const int tr = acc16_row<Cfg>(tm, tid);
+    static_for<0, R::TN>([&](auto J) {
+      constexpr int tn = J.value;
+      float4v v;
+      v[0] = R::template acc_get<tm, tn, 0>();
+      v[1] = R::template acc_get<tm, tn, 1>();
+      v[2] = R::template acc_get<tm, tn, 2>();
+      v[3] = R::template acc_get<tm, tn, 3>();
+      *reinterpret_cast<float4v *>(out + tr * Cfg::BN + acc16_col4<Cfg>(tn, tid)) = v;
+    });
+  });
+}
+
+// out tile = sum of its S partial tiles (in part order) + bias, then the epilogue kEpi of the
+// grouped GEMM.  grid (kTailMaxParts, BM / 16): block (t, q) does tile rows 16q .. 16q+15 of
+// tail tile t, a thread four rows of four columns.
+template <class Cfg, int kEpi>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(GroupedArgs p) {
+  using R = Ring16Mainloop<Cfg>;
+  const int tiles = p.tail[0], S = p.tail[1];
+  const int t = blockIdx.x;
+  if (t >= tiles) return;
+  const int4v ent = reinterpret_cast<const int4v *>(p.tail + 64)[t * S];
+  const int e = ent[0], row0 = ent[1], rows = ent[2], n0 = (ent[3] & 0xffff) * Cfg::BN;
+  const float *part0 = p.partial + static_cast<size_t>(t) * S * (Cfg::BM * Cfg::BN);
+  const int c4 = threadIdx.x & 63;                     // which group of four columns
+  const int col = n0 + 4 * c4;
+  if (col >= p.N) return;
+  float bias_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (p.bias) {
+    const half4 bv = *reinterpret_cast<const half4 *>(p.bias + static_cast<size_t>(e) * p.N + col);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) bias_v[c] = static_cast<float>(bv[c]);
+  }
+  float4v acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+  const int r_first = blockIdx.y * 16 + (threadIdx.x >> 6);
+  for (int s = 0; s < S; ++s) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      acc[i] += *reinterpret_cast<const float4v *>(part0 + static_cast<size_t>(s) * (Cfg::BM * Cfg::BN) +
+                                                   (r_first + 4 * i) * Cfg::BN + 4 * c4);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r_first + 4 * i;
+    if (!R::row_is_real(r, rows)) continue;
+    const int j = row0 + R::local_row(r, rows);
+    const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
+    const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
+    half4 o, pre;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float x = acc[i][c] + bias_v[c];
+      if (kEpi == kEpiGelu || kEpi == kEpiGeluKeep) {
+        pre[c] = static_cast<half_t>(x);
+        x = gelu_erf(x);
+      } else {
+        x *= sc;
+      }
+      o[c] = static_cast<half_t>(x);
+    }
+    *reinterpret_cast<half4 *>(p.C + crow * p.N + col) = o;
+    if (kEpi == kEpiGeluKeep) *reinterpret_cast<half4 *>(p.C2 + static_cast<size_t>(j) * p.N + col) = pre;
+  }
+}
+
 // ---- variants -------------------------------------------------------------------
 // 256x256x64 tiles throughout (the most flop per byte pulled from L2 that the
 // register file allows).  What differs is how the tile loads are pipelined and
@@ -673,7 +838,9 @@ using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 8, 4>;   // 4 wavefronts of 128x1
 
 constexpr int kDefaultVariant = 6;
 int g_variant = kDefaultVariant;
-int g_dgrad_transpose = 0;   // 1: input gradients always on a transposed copy of the weight
+int g_dgrad_transpose = 0;
+int g_split_tail = 1;        // 0: the last round of tiles is not cut along K
+int g_split_tail_min_kt = 128;   // 1: input gradients always on a transposed copy of the weight
 
 struct Launch {
   int bm, bn, threads;
@@ -725,16 +892,20 @@ int max_tiles_for(int max_rows, int E, int bm) { return (max_rows + bm - 1) / bm
 
 constexpr int kMinBN = 128;
 
+// Workspace of one grouped GEMM: the split-K tail area, then the tile plan.
 size_t plan_bytes(int max_rows, int E, int n_max) {
-  return round_up(sizeof(int32_t) * plan_ints(launched_wgs(max_tiles_for(max_rows, E, kMinBM),
-                                                            (n_max + kMinBN - 1) / kMinBN)), 256);
+  return kTailBytes + round_up(sizeof(int32_t) * plan_ints(launched_wgs(max_tiles_for(max_rows, E, kMinBM),
+                                                                         (n_max + kMinBN - 1) / kMinBN)), 256);
 }
 
 int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets, int max_rows, int E,
                  int N, int K, const half_t *B, const half_t *bias, int epi, half_t *C,
-                 const int32_t *c_rows, const half_t *row_scale, int32_t *plan, hipStream_t stream,
+                 const int32_t *c_rows, const half_t *row_scale, int32_t *workspace, hipStream_t stream,
                  const char *what, bool b_kn = false, half_t *C2 = nullptr) {
-  CCF_REQUIRE(A && offsets && B && C && plan, CCF_ERR_ARG, "%s: null pointer", what);
+  CCF_REQUIRE(A && offsets && B && C && workspace, CCF_ERR_ARG, "%s: null pointer", what);
+  int32_t *tail = workspace;                                                        // header and entries
+  float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + kTailHead);
+  int32_t *plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(workspace) + kTailBytes);
   const bool gelu = epi != kEpiPlain;
   CCF_REQUIRE(epi >= kEpiPlain && epi <= kEpiGeluGrad && (epi < kEpiGeluKeep || (C2 && aligned16(C2))), CCF_ERR_ARG,
               "%s: epilogue %d needs the pre-activation buffer", what, epi);
@@ -773,13 +944,33 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.k_seg = nullptr;
   p.lda = p.ldb = K;
   p.seg_rows = 0;
+  p.tail = tail;
+  p.partial = partial;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;                // wgs is a multiple of 8
+    // the last, partly filled round is cut along K and spread over all workgroups (forward forms)
+    // (worth its three small launches only where a tile is long: K of 8192 and more)
+    const bool split = g_split_tail && !b_kn && epi <= kEpiGeluKeep && g == grid && grid <= kTailMaxParts &&
+                       v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= g_split_tail_min_kt;
+    if (split) {
+      hipLaunchKernelGGL(tail_kernel, dim3(1), dim3(256), 0, stream, plan, static_cast<int>(wgs / 8), grid, K / 64, tail);
+      if (int rc = check_launch("tail_kernel")) return rc;
+    }
     hipLaunchKernelGGL(second ? v.persistent_gelu : v.persistent_plain, dim3(static_cast<unsigned>(g)),
                        dim3(v.threads), 0, stream, p, static_cast<int>(wgs / 8));
+    if (split) {
+      if (int rc = check_launch(what)) return rc;
+      hipLaunchKernelGGL(grouped_gemm_tail_kernel<Cfg5>, dim3(grid), dim3(Cfg5::THREADS), 0, stream, p);
+      if (int rc = check_launch("grouped_gemm_tail_kernel")) return rc;
+      const dim3 rgrid(grid, Cfg5::BM / 16);
+      if (epi == kEpiPlain) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiPlain>), rgrid, dim3(256), 0, stream, p);
+      else if (epi == kEpiGelu) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGelu>), rgrid, dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGeluKeep>), rgrid, dim3(256), 0, stream, p);
+      return check_launch("splitk_reduce_kernel");
+    }
   } else {
     hipLaunchKernelGGL(second ? v.gelu : v.plain, dim3(static_cast<unsigned>(wgs)), dim3(v.threads), 0,
                        stream, p);
@@ -790,9 +981,10 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
 // C[e*M + m, n] = sum over k in [k_seg[e], k_seg[e+1]) of A[m, k] * B[n, k]: the weight
 // gradient of expert e from the two transposed activation matrices.  row_off[e] = e*M.
 int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const int32_t *k_seg,
-                      const int32_t *row_off, int E, int M, int N, half_t *C, int32_t *plan,
+                      const int32_t *row_off, int E, int M, int N, half_t *C, int32_t *workspace,
                       hipStream_t stream, const char *what) {
-  CCF_REQUIRE(A && B && k_seg && row_off && C && plan, CCF_ERR_ARG, "%s: null pointer", what);
+  CCF_REQUIRE(A && B && k_seg && row_off && C && workspace, CCF_ERR_ARG, "%s: null pointer", what);
+  int32_t *plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(workspace) + kTailBytes);
   CCF_REQUIRE(lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0, CCF_ERR_SHAPE, "%s: strides and N must be multiples of 8", what);
   CCF_REQUIRE(static_cast<long long>(E) * M < (1ll << 31), CCF_ERR_SHAPE, "%s: output too tall", what);
   const int max_rows = E * M;
@@ -817,6 +1009,8 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.lda = lda;
   p.ldb = ldb;
   p.seg_rows = M;
+  p.tail = nullptr;
+  p.partial = nullptr;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   const int grid = persistent_grid();
@@ -936,6 +1130,11 @@ extern "C" int ccf_set_option(const char *name, int value) {
     CCF_REQUIRE(value >= -1 && value < kNumVariants, CCF_ERR_ARG, "set_option: gemm_variant %d outside -1..%d",
                 value, kNumVariants - 1);
     g_variant = value < 0 ? kDefaultVariant : value;     // -1: back to the default
+    return CCF_OK;
+  }
+  if (!strcmp(name, "split_tail")) {         // 0 = off, 1 = default, n > 1: for K of n K tiles and more
+    g_split_tail = value != 0;
+    g_split_tail_min_kt = value > 1 ? value : 128;
     return CCF_OK;
   }
   if (!strcmp(name, "dgrad_transpose")) {

@@ -55,7 +55,8 @@ const char *ccf_last_error(void);
 /*
  * Tuning knobs (no counterpart in the reference).  "gemm_variant" selects the
  * grouped-GEMM main-loop variant used by the FFN entry points; -1 restores
- * the default.  "dgrad_transpose" (0/1) makes the backward's input-gradient GEMM run on a
+ * the default.  "split_tail" (0 = off, 1 = default, n > 1 = for K of n*64 and more) cuts the
+ * tiles of a launch's last, partly filled round along K.  "dgrad_transpose" (0/1) makes the backward's input-gradient GEMM run on a
  * transposed copy of the weight instead of reading the stored one.
  * "gate_waves" (4 or 16) caps the gate
  * kernel's wavefronts per workgroup.  Process-wide; not meant to be changed

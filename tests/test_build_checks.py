@@ -27,7 +27,7 @@ def test_no_compiler_values_in_accumulation_registers(tmp_path):
     assert res.returncode == 0, res.stderr[-2000:]
     text = out.read_text()
     # kernels built on Ring16Mainloop: SCHED = 4 in the GemmCfg mangling, plain and persistent
-    kernels = re.findall(r"^(_ZN3ccf\S*GemmCfgILi256ELi256ELi64ELi2ELi2ELi2ELi1ELi8ELi4EEE\S*):[^\n]*\n(.*?)s_endpgm",
+    kernels = re.findall(r"^(_ZN3ccf\S*grouped_gemm\S*GemmCfgILi256ELi256ELi64ELi2ELi2ELi2ELi1ELi8ELi4EEE\S*):[^\n]*\n(.*?)s_endpgm",
                          text, flags=re.S | re.M)
     assert len(kernels) >= 4, [k for k, _ in kernels]
     for name, body in kernels:

@@ -294,3 +294,56 @@ def test_ffn_special_cases():
     pre = ops.ffn1(dev(x), None, off, R, dev(w1), dev(b1), gelu=False)
     ref = x.float() @ w1[0].float().t() + b1.float()
     assert O.max_abs_err(pre.cpu(), ref) <= MAX_ABS
+
+
+def test_split_k_tail_all_epilogues():
+    """The last, partly filled round of tiles is cut along K and reduced by a separate kernel.
+    By default that happens for K >= 8192 only; here it is forced on a small K so that the
+    reduction's three epilogues (plain with row index and scale, GELU, GELU keeping the
+    pre-activation) are compared with the oracle and with the unsplit kernels."""
+    from ccfuser_amd import ops
+    g = torch.Generator().manual_seed(21)
+    R, d, f, E = 8192, 2048, 2048, 6           # 16+ M tiles x 8 N tiles: more tiles than workgroups, a ragged last round
+    x = (torch.randn(R, d, generator=g)).half()
+    w1 = (torch.randn(E, f, d, generator=g) * 0.05).half()
+    b1 = (torch.randn(E, f, generator=g) * 0.05).half()
+    w2 = (torch.randn(E, d, f, generator=g) * 0.02).half()
+    b2 = (torch.randn(E, d, generator=g) * 0.05).half()
+    idx = torch.randint(0, E, (R,), generator=g)
+    r = ops.route(dev(idx), E, 1, -1)
+    off = r["offsets"].cpu()
+    pos = r["pos"].cpu()
+    scale = (torch.rand(R, generator=g) + 0.5).half()
+    _say(f"split-K tail R={R} d={d} f={f} E={E} counts={r['counts'].tolist()}")
+    results = {}
+    for mode in (0, 4):
+        ops.set_option("split_tail", mode)
+        try:
+            h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True)
+            act, pre = ops.ffn1_keep(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1))
+            y = torch.zeros(R, d, dtype=torch.float16, device="cuda")
+            ops.ffn2(h, r["dst_row"], r["offsets"], R, dev(w2), dev(b2), y, row_scale=dev(scale))
+            results[mode] = [t.cpu() for t in (h, act, pre, y)]
+        finally:
+            ops.set_option("split_tail", 1)
+    buf = x[torch.div(pos, 1, rounding_mode="floor")].float()
+    h_ref = torch.zeros(R, f)
+    pre_ref = torch.zeros(R, f)
+    for e in range(E):
+        lo, hi = int(off[e]), int(off[e + 1])
+        pre_ref[lo:hi] = buf[lo:hi] @ w1[e].float().t() + b1[e].float()
+    h_ref = O.gelu_exact(pre_ref)
+    for mode, (h, act, pre, y) in results.items():
+        assert O.max_abs_err(h, h_ref) <= MAX_ABS and O.mean_rel_err(h, h_ref) <= MEAN_REL, mode
+        assert torch.equal(h, act), mode
+        assert O.max_abs_err(pre, pre_ref) <= MAX_ABS, mode
+    y_ref = torch.zeros(R, d)
+    hq = results[4][0].float()
+    for e in range(E):
+        lo, hi = int(off[e]), int(off[e + 1])
+        y_ref[pos[lo:hi]] = (hq[lo:hi] @ w2[e].float().t() + b2[e].float()) * scale[lo:hi].float()[:, None]
+    assert O.max_abs_err(results[4][3], y_ref) <= MAX_ABS and O.mean_rel_err(results[4][3], y_ref) <= MEAN_REL
+    # split and unsplit differ only in summation order (and do differ: the split path ran)
+    assert O.max_abs_err(results[4][3], results[0][3].float()) <= MAX_ABS
+    assert O.max_abs_err(results[4][0], results[0][0].float()) <= MAX_ABS
+    assert not torch.equal(results[4][3], results[0][3]) and not torch.equal(results[4][0], results[0][0])
