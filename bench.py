@@ -186,9 +186,11 @@ def bench_backward(a, wl, ops):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c3_mixtral")
+    ap.add_argument("--stage-events", choices=("timed", "after"), default="timed",
+                    help="record the per-stage HIP events inside the timed steps, or in a second pass of the same steps")
     ap.add_argument("--gemm-variant", type=int, default=None)
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="ccf_set_option before the run (tuning knobs), may repeat")
@@ -261,20 +263,30 @@ def main():
             _lib.call("ccf_moe_forward", *ptrs, T, d, f, E, k, wl.capacity, out.data_ptr(), None,
                       None, None, None, offsets.data_ptr(), ws.data_ptr(), ws.numel(), stream)
 
+        events = [[ev.create() for _ in range(6)] for _ in range(K)]
+        arrs = [(ctypes.c_void_p * 6)(*row) for row in events]
         for _ in range(W):
             run()
         torch.cuda.synchronize()
-        routed = int(offsets[-1].item())
-        events = [[ev.create() for _ in range(6)] for _ in range(K)]
-        arrs = [(ctypes.c_void_p * 6)(*row) for row in events]
-        torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(K):
-            _lib.call("ccf_moe_forward_set_events", arrs[i], 6)
+            if a.stage_events == "timed":
+                _lib.call("ccf_moe_forward_set_events", arrs[i], 6)
             run()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
+        if a.stage_events == "after":
+            # the same K steps once more, now with an event recorded between the stages
+            t1 = time.perf_counter()
+            for i in range(K):
+                _lib.call("ccf_moe_forward_set_events", arrs[i], 6)
+                run()
+            torch.cuda.synchronize()
+            wall_events = time.perf_counter() - t1
+        else:
+            wall_events = wall
         _lib.call("ccf_moe_forward_set_events", None, 0)
+        routed = int(offsets[-1].item())
         stage_names = ("gate", "route", "ffn1", "ffn2", "combine")
         stage_ms = {n: sum(ev.elapsed_ms(events[i][s], events[i][s + 1]) for i in range(K)) / K
                     for s, n in enumerate(stage_names)}
@@ -303,6 +315,7 @@ def main():
     }
     if stage_ms is not None:
         line["stages_ms"] = stage_ms
+        line["ms_per_step_with_stage_events"] = wall_events / K * 1e3
         dom = "ffn1" if stage_ms["ffn1"] >= stage_ms["ffn2"] else "ffn2"
         ach = (flops / 2) / (stage_ms[dom] * 1e-3) / 1e12
         line["roofline"] = {"kernel": f"grouped_gemm_persistent_kernel ({dom})", "bound": "mfma",

@@ -15,6 +15,8 @@
 // blocks on the host in Python (mix_moe/mix_moe/transformer.py:150-250) and
 // copies seven arrays to the device per call; here a one-workgroup kernel
 // derives the tile list from the offsets on the device.
+#include <limits.h>
+
 #include "ccf_common.h"
 #include "gemm_tile.h"
 
@@ -34,6 +36,16 @@ __host__ __device__ inline long long launched_wgs(int max_tiles, int n_tiles_n) 
 }
 
 constexpr int kOrderGroupM = 8;
+
+// Scratch of the split last round, in front of the plan in the caller's workspace:
+//   [0, 16)              header: tile slots T (a multiple of 8; slot t belongs to XCD t % 8), parts S
+//   [256, 256 + 16*256)  entries {expert, row0, rows, tile_n | part << 16 | S << 24} by workgroup
+//                        id: part s of tile slot t at (t % 8) + 8 * ((t / 8) * S + s); expert -1 = none
+//   [kTailHead, ...)     256 partial tiles of 256 x 256 fp32, by the same workgroup id
+constexpr int kTailMaxParts = 256;
+constexpr int kTailMaxTiles = kTailMaxParts / 2;     // tile slots: every tile has at least two parts
+constexpr size_t kTailHead = 256 + 16 * kTailMaxParts;
+constexpr size_t kTailBytes = kTailHead + static_cast<size_t>(kTailMaxParts) * 256 * 256 * 4;
 
 // Rows of M tile i of an expert with cnt rows in nt = ceil(cnt / BM) tiles.  When
 // the last tile would hold at most BM/2 rows, it and the one before it share
@@ -63,7 +75,9 @@ __device__ inline void tile_rows(int cnt, int nt, int i, int BM, int &first_row,
 // where they also even out the end of the launch.
 __global__ void __launch_bounds__(1024)
 plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, int max_rows,
-            int n_tiles_n, int32_t *__restrict__ plan) {
+            int n_tiles_n, int32_t *__restrict__ plan, int spx, int k_tiles, int32_t *__restrict__ tail) {
+  __shared__ int s_full[8];        // split last round: slots of XCD x from s_full[x] on go to the tail list
+  __shared__ int s_parts;          // parts per tail tile, 0 = no split
   __shared__ int s_off[1025];
   __shared__ int s_long[1025];     // exclusive scan of long M tiles per expert
   __shared__ int s_short[1025];    // exclusive scan of short M tiles per expert (0 or 1 each)
@@ -98,6 +112,9 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   int4v *entry = reinterpret_cast<int4v *>(plan);
   for (long long b = threadIdx.x; b < wgs; b += blockDim.x) entry[b] = int4v{-1, 0, 0, 0};
+  int4v *tent = reinterpret_cast<int4v *>(tail + 64);
+  if (tail)
+    for (int b = threadIdx.x; b < kTailMaxParts; b += blockDim.x) tent[b] = int4v{-1, 0, 0, 0};
   __syncthreads();
   // Hardware hands consecutive workgroup ids to the 8 XCDs in turn, so XCD x
   // runs ids x, x+8, ... in order.  Each class is cut into eight equal
@@ -109,6 +126,48 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
   const long long total_short = static_cast<long long>(s_short[E]) * n_tiles_n;
   const long long per_long = (total_long + 7) / 8;
   const long long per_short = (total_short + 7) / 8;
+  // The split last round (see "split-K tail" below).  XCD x holds used_x tiles; with spx
+  // persistent workgroups per XCD the last used_x % spx of them form a partly filled round.
+  // When that round is at most half full on every XCD, its tiles leave the plan: tile i of
+  // XCD x's last round, part s of S, becomes tail entry x + 8 * (i * S + s), the workgroup id
+  // that the hardware places on the same XCD, so the patch of neighbouring tiles keeps sharing
+  // its operands through that XCD's L2 (parts of the same K range walk K in step).
+  if (threadIdx.x == 0) {
+    int max_r = 0;
+    for (int x = 0; x < 8; ++x) {
+      long long nl_x = total_long - x * per_long, ns_x = total_short - x * per_short;
+      nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
+      ns_x = ns_x < 0 ? 0 : (ns_x > per_short ? per_short : ns_x);
+      const int used = static_cast<int>(nl_x + ns_x);
+      const int full = spx > 0 ? used / spx * spx : used;
+      s_full[x] = full;
+      max_r = (used - full) > max_r ? (used - full) : max_r;
+    }
+    int S = 0;
+    if (tail && spx > 0 && max_r > 0 && max_r * 2 <= spx) {
+      S = spx / max_r;
+      S = S > 8 ? 8 : S;
+      S = S > k_tiles / 4 ? k_tiles / 4 : S;           // at least four K tiles per part
+      S = (S >= 2 && 8 * max_r * S <= kTailMaxParts) ? S : 0;
+    }
+    s_parts = S;
+    if (!S)
+      for (int x = 0; x < 8; ++x) s_full[x] = INT_MAX;
+    if (tail) { tail[0] = S ? 8 * max_r : 0; tail[1] = S; }
+  }
+  __syncthreads();
+  const int S = s_parts;
+  // slot j of XCD x: into the plan, or cut into S parts on the tail list
+  auto place = [&](long long j, long long x, int4v v) {
+    const long long b = j * 8 + x;
+    if (j >= s_full[x]) {
+      const int i = static_cast<int>(j) - s_full[x];
+      for (int part = 0; part < S; ++part)
+        tent[x + 8 * (i * S + part)] = int4v{v[0], v[1], v[2], v[3] | (part << 16) | (S << 24)};
+    } else if (b < wgs) {
+      entry[b] = v;
+    }
+  };
   // one wavefront per expert
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
   for (int e = wave; e < E; e += nwave) {
@@ -132,10 +191,9 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
       const int i = run_first + in_run % run_size;               // M tile within the expert
       const int tn = in_run / run_size;
       const long long logical = first + l;
-      const long long b = (logical % per_long) * 8 + logical / per_long;   // hardware id
       int first_row, rows;
       tile_rows(cnt, nl, i, BM, first_row, rows);
-      if (b < wgs) entry[b] = int4v{e, lo + first_row, rows, tn};
+      place(logical % per_long, logical / per_long, int4v{e, lo + first_row, rows, tn});   // hardware id = slot * 8 + XCD
     }
     if (ns) {
       const int i = nl;                                          // the expert's last M tile
@@ -145,8 +203,7 @@ plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, i
         const long long x = logical / per_short;
         long long nl_x = total_long - x * per_long;              // long tiles on this XCD
         nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
-        const long long b = (nl_x + logical % per_short) * 8 + x;
-        if (b < wgs) entry[b] = int4v{e, lo + i * BM, cnt - i * BM, tn};
+        place(nl_x + logical % per_short, x, int4v{e, lo + i * BM, cnt - i * BM, tn});
       }
     }
   }
@@ -665,63 +722,13 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
 // ---- split-K tail -----------------------------------------------------------------
 // Tiles all take about the same time, so a launch whose tile count is no multiple of the
 // workgroup count ends with a round in which most CUs idle: config 3's FFN2 has 592 tiles for
-// 256 workgroups, 2.3 rounds that cost 3.  tail_kernel takes the tiles of each XCD's last,
-// partly filled round out of the plan and, when they are few enough to matter (at most half
-// a round), cuts each into S parts along K, S = workgroups / tiles (at most 8, at least four
-// K tiles per part).  The parts run as one more launch, one workgroup each, and leave raw
-// fp32 accumulators in a scratch area; splitk_reduce adds a tile's parts in part order and
-// applies the epilogue.  The area sits in front of the plan in the caller's workspace:
-//   [0, 16)              header: tiles R, parts S
-//   [256, 256 + 16*256)  entries {expert, row0, rows, tile_n | part << 16 | S << 24}, part-major per tile
-//   [kTailHead, ...)     256 partial tiles of 256 x 256 fp32
-constexpr int kTailMaxParts = 256;
-constexpr size_t kTailHead = 256 + 16 * kTailMaxParts;
-constexpr size_t kTailBytes = kTailHead + static_cast<size_t>(kTailMaxParts) * 256 * 256 * 4;
-
-__global__ void __launch_bounds__(256)
-tail_kernel(int32_t *__restrict__ plan, int slots_per_xcd, int persistent_wgs, int k_tiles,
-            int32_t *__restrict__ tail) {
-  __shared__ int s_used[8], s_full[8], s_base[9];
-  const int spx = persistent_wgs >> 3;                 // persistent workgroups per XCD
-  int4v *entry = reinterpret_cast<int4v *>(plan);
-  int4v *tent = reinterpret_cast<int4v *>(tail + 64);
-  if (threadIdx.x < 8) {
-    // the used slots of an XCD are a prefix: first slot j with an idle entry
-    const int x = threadIdx.x;
-    int lo = 0, hi = slots_per_xcd;
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (entry[mid * 8 + x][0] >= 0) lo = mid + 1; else hi = mid;
-    }
-    s_used[x] = lo;
-    s_full[x] = lo / spx * spx;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int r = 0;
-    for (int x = 0; x < 8; ++x) { s_base[x] = r; r += s_used[x] - s_full[x]; }
-    s_base[8] = r;
-  }
-  __syncthreads();
-  const int R = s_base[8];
-  int S = R > 0 ? persistent_wgs / R : 0;
-  S = S > 8 ? 8 : S;
-  S = S > k_tiles / 4 ? k_tiles / 4 : S;
-  if (R == 0 || R * 2 > persistent_wgs || S < 2 || R * S > kTailMaxParts) {
-    if (threadIdx.x == 0) { tail[0] = 0; tail[1] = 0; }
-    return;                                            // the plan stays as it is
-  }
-  if (threadIdx.x == 0) { tail[0] = R; tail[1] = S; }
-  for (int x = 0; x < 8; ++x) {
-    const int rx = s_used[x] - s_full[x];
-    for (int i = threadIdx.x; i < rx; i += blockDim.x) {
-      const int4v e = entry[(s_full[x] + i) * 8 + x];
-      entry[(s_full[x] + i) * 8 + x] = int4v{-1, 0, 0, 0};
-      const int t = s_base[x] + i;
-      for (int part = 0; part < S; ++part) tent[t * S + part] = int4v{e[0], e[1], e[2], e[3] | (part << 16) | (S << 24)};
-    }
-  }
-}
+// 256 workgroups, 2.3 rounds that cost 3.  plan_kernel therefore keeps the tiles of each XCD's
+// last, partly filled round out of the plan when they are few enough to matter (at most half a
+// round) and cuts each into S parts along K, S = workgroups per XCD / tiles (at most 8, at
+// least four K tiles per part).  The parts run as one more launch, one workgroup each, and
+// leave raw fp32 accumulators in a scratch area; splitk_reduce adds a tile's parts in part
+// order and applies the epilogue.  The area sits in front of the plan in the caller's workspace
+// (kTailHead, kTailBytes above).
 
 // K tiles [first, first + count) of part `part` of S over k_tiles K tiles.
 __device__ __forceinline__ void part_range(int k_tiles, int part, int S, int &first, int &count) {
@@ -731,25 +738,28 @@ __device__ __forceinline__ void part_range(int k_tiles, int part, int S, int &fi
 }
 
 // One part of one tail tile per workgroup: the main loop over its K range, raw accumulators out.
-template <class Cfg>
+template <class Cfg, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_tail_kernel(GroupedArgs p) {
-  using R = Ring16Mainloop<Cfg>;
+  using R = Ring16Mainloop<Cfg, kKN>;
+  const int bmul = kKN ? p.N : 1;                      // elements between K rows of a [K][N] B
   const int tiles = p.tail[0], S = p.tail[1];
   if (static_cast<int>(blockIdx.x) >= tiles * S) return;
   int4v ent = reinterpret_cast<const int4v *>(p.tail + 64)[blockIdx.x];
+  if (ent[0] < 0) return;                              // this XCD's last round had fewer tiles
   const int part = (ent[3] >> 16) & 0xff;
   ent[3] &= 0xffff;
   int first, count;
   part_range(p.K / Cfg::BK, part, S, first, count);
   const half_t *a_src[Cfg::A_DMA];
-  const half_t *b_src[Cfg::B_DMA];
-  tile_sources<Cfg>(p, ent, a_src, b_src);
+  constexpr int NB = kKN ? 2 : Cfg::B_DMA;
+  const half_t *b_src[NB];
+  tile_sources<Cfg, false, kKN>(p, ent, a_src, b_src);
 #pragma unroll
   for (int i = 0; i < Cfg::A_DMA; ++i) a_src[i] += first * Cfg::BK;
 #pragma unroll
-  for (int i = 0; i < Cfg::B_DMA; ++i) b_src[i] += first * Cfg::BK;
-  R::run(a_src, b_src, count * Cfg::BK, ent[2]);
+  for (int i = 0; i < NB; ++i) b_src[i] += static_cast<size_t>(first * Cfg::BK) * bmul;
+  R::run(a_src, b_src, count * Cfg::BK, ent[2], bmul);
   float *out = p.partial + static_cast<size_t>(blockIdx.x) * (Cfg::BM * Cfg::BN);
   const int tid = fresh_tid();
   static_for<0, R::TM>([&](auto T) {
@@ -768,8 +778,9 @@ grouped_gemm_tail_kernel(GroupedArgs p) {
 }
 
 // out tile = sum of its S partial tiles (in part order) + bias, then the epilogue kEpi of the
-// grouped GEMM.  grid (kTailMaxParts, BM / 16): block (t, q) does tile rows 16q .. 16q+15 of
-// tail tile t, a thread four rows of four columns.
+// grouped GEMM.  grid (kTailMaxTiles, BM / 16): block (t, q) does tile rows 16q .. 16q+15 of
+// tile slot t, a thread four rows of four columns.  It runs at the speed the partial tiles
+// stream back in (config 3, FFN2: 63 MB in 13 us).
 template <class Cfg, int kEpi>
 __global__ void __launch_bounds__(256)
 splitk_reduce_kernel(GroupedArgs p) {
@@ -777,9 +788,10 @@ splitk_reduce_kernel(GroupedArgs p) {
   const int tiles = p.tail[0], S = p.tail[1];
   const int t = blockIdx.x;
   if (t >= tiles) return;
-  const int4v ent = reinterpret_cast<const int4v *>(p.tail + 64)[t * S];
+  const int first_wg = (t & 7) + 8 * ((t >> 3) * S);   // workgroup id of part 0; part s is 8 s further
+  const int4v ent = reinterpret_cast<const int4v *>(p.tail + 64)[first_wg];
   const int e = ent[0], row0 = ent[1], rows = ent[2], n0 = (ent[3] & 0xffff) * Cfg::BN;
-  const float *part0 = p.partial + static_cast<size_t>(t) * S * (Cfg::BM * Cfg::BN);
+  if (e < 0) return;
   const int c4 = threadIdx.x & 63;                     // which group of four columns
   const int col = n0 + 4 * c4;
   if (col >= p.N) return;
@@ -793,11 +805,11 @@ splitk_reduce_kernel(GroupedArgs p) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
   const int r_first = blockIdx.y * 16 + (threadIdx.x >> 6);
+  const float *src = p.partial + static_cast<size_t>(first_wg) * (Cfg::BM * Cfg::BN) + r_first * Cfg::BN + 4 * c4;
   for (int s = 0; s < S; ++s) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      acc[i] += *reinterpret_cast<const float4v *>(part0 + static_cast<size_t>(s) * (Cfg::BM * Cfg::BN) +
-                                                   (r_first + 4 * i) * Cfg::BN + 4 * c4);
+      acc[i] += *reinterpret_cast<const float4v *>(src + static_cast<size_t>(8 * s) * (Cfg::BM * Cfg::BN) + 4 * i * Cfg::BN);
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -838,9 +850,10 @@ using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 8, 4>;   // 4 wavefronts of 128x1
 
 constexpr int kDefaultVariant = 6;
 int g_variant = kDefaultVariant;
-int g_dgrad_transpose = 0;
+int g_dgrad_transpose = 0;   // 1: input gradients always on a transposed copy of the weight
 int g_split_tail = 1;        // 0: the last round of tiles is not cut along K
-int g_split_tail_min_kt = 128;   // 1: input gradients always on a transposed copy of the weight
+constexpr int kSplitTailMinKT = 64;
+int g_split_tail_min_kt = kSplitTailMinKT;
 
 struct Launch {
   int bm, bn, threads;
@@ -926,8 +939,16 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   const bool second = b_kn ? epi == kEpiGeluGrad : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu);
   const int max_tiles = max_tiles_for(max_rows, E, v.bm);
   const int n_tiles_n = (N + v.bn - 1) / v.bn;
+  const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
+  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
+  const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
+  // the last, partly filled round is cut along K and spread over all workgroups (forward forms;
+  // worth its two small launches only where a tile is long: K of 4096 and more)
+  const bool split = g_split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && grid >= 8 && grid <= wgs &&
+                     grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN &&
+                     K / 64 >= g_split_tail_min_kt;
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, offsets, E, v.bm, max_tiles,
-                     max_rows, n_tiles_n, plan);
+                     max_rows, n_tiles_n, plan, split ? grid / 8 : 0, K / 64, split ? tail : nullptr);
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
   p.A = A;
@@ -946,26 +967,16 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.seg_rows = 0;
   p.tail = tail;
   p.partial = partial;
-  const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
-  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
-  const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;                // wgs is a multiple of 8
-    // the last, partly filled round is cut along K and spread over all workgroups (forward forms)
-    // (worth its three small launches only where a tile is long: K of 8192 and more)
-    const bool split = g_split_tail && !b_kn && epi <= kEpiGeluKeep && g == grid && grid <= kTailMaxParts &&
-                       v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= g_split_tail_min_kt;
-    if (split) {
-      hipLaunchKernelGGL(tail_kernel, dim3(1), dim3(256), 0, stream, plan, static_cast<int>(wgs / 8), grid, K / 64, tail);
-      if (int rc = check_launch("tail_kernel")) return rc;
-    }
     hipLaunchKernelGGL(second ? v.persistent_gelu : v.persistent_plain, dim3(static_cast<unsigned>(g)),
                        dim3(v.threads), 0, stream, p, static_cast<int>(wgs / 8));
     if (split) {
       if (int rc = check_launch(what)) return rc;
-      hipLaunchKernelGGL(grouped_gemm_tail_kernel<Cfg5>, dim3(grid), dim3(Cfg5::THREADS), 0, stream, p);
+      if (b_kn) hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, true>), dim3(grid), dim3(Cfg5::THREADS), 0, stream, p);
+      else hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, false>), dim3(grid), dim3(Cfg5::THREADS), 0, stream, p);
       if (int rc = check_launch("grouped_gemm_tail_kernel")) return rc;
-      const dim3 rgrid(grid, Cfg5::BM / 16);
+      const dim3 rgrid(kTailMaxTiles, Cfg5::BM / 16);
       if (epi == kEpiPlain) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiPlain>), rgrid, dim3(256), 0, stream, p);
       else if (epi == kEpiGelu) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGelu>), rgrid, dim3(256), 0, stream, p);
       else hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGeluKeep>), rgrid, dim3(256), 0, stream, p);
@@ -991,7 +1002,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const int max_tiles = max_tiles_for(max_rows, E, Cfg5::BM);
   const int n_tiles_n = (N + Cfg5::BN - 1) / Cfg5::BN;
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, row_off, E, Cfg5::BM, max_tiles,
-                     max_rows, n_tiles_n, plan);
+                     max_rows, n_tiles_n, plan, 0, 0, static_cast<int32_t *>(nullptr));
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
   p.A = A;
@@ -1134,7 +1145,7 @@ extern "C" int ccf_set_option(const char *name, int value) {
   }
   if (!strcmp(name, "split_tail")) {         // 0 = off, 1 = default, n > 1: for K of n K tiles and more
     g_split_tail = value != 0;
-    g_split_tail_min_kt = value > 1 ? value : 128;
+    g_split_tail_min_kt = value > 1 ? value : kSplitTailMinKT;
     return CCF_OK;
   }
   if (!strcmp(name, "dgrad_transpose")) {

@@ -59,6 +59,33 @@ def test_ffn_backward_stages(T, d, f, E, k, cap, skew, seed, transpose):
         ops.set_option("dgrad_transpose", 0)
 
 
+@pytest.mark.parametrize("transpose", [0, 1])
+def test_ffn_backward_stages_with_split_last_round(transpose):
+    """Input gradients with the last, partly filled round of tiles cut along K (forced on a
+    short K; by default it takes K >= 4096): 36 M tiles x 8 N tiles on 256 workgroups, in both
+    weight forms, against the oracle; and the split path did run (bits differ from unsplit)."""
+    from ccfuser_amd import ops
+    T, d, f, E, k = 4096, 2048, 2048, 6, 2
+    ops.set_option("dgrad_transpose", transpose)
+    ops.set_option("split_tail", 4)
+    try:
+        _ffn_backward_stages(T, d, f, E, k, -1, False, 7)
+        g = torch.Generator().manual_seed(77)
+        n = T * k
+        rt = ops.route(torch.randint(0, E, (n,), generator=g).cuda(), E, k, -1)
+        gy = torch.randn(n, d, generator=g).half().cuda()
+        act = torch.randn(n, f, generator=g).half().cuda()
+        w2 = (torch.randn(E, d, f, generator=g) * 0.05).half().cuda()
+        ga_split = ops.ffn2_backward(gy, act, rt["dst_row"], rt["offsets"], n, w2)[0]
+        ops.set_option("split_tail", 0)
+        ga_whole = ops.ffn2_backward(gy, act, rt["dst_row"], rt["offsets"], n, w2)[0]
+        assert O.max_abs_err(ga_split.cpu(), ga_whole.float().cpu()) <= MAX_ABS
+        assert not torch.equal(ga_split, ga_whole)
+    finally:
+        ops.set_option("dgrad_transpose", 0)
+        ops.set_option("split_tail", 1)
+
+
 def _ffn_backward_stages(T, d, f, E, k, cap, skew, seed):
     from ccfuser_amd import ops
     _say(f"ffn backward T={T} d={d} f={f} E={E} k={k} cap={cap} skew={skew}")
