@@ -10,6 +10,7 @@
 // in place through the row index) and keeps only the activation h and the
 // un-permuted expert output in a caller-owned HBM workspace.
 #include "ccf_common.h"
+#include "plan.h"
 
 namespace ccf {
 
@@ -166,19 +167,25 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
                                   w.score, nullptr, stream)))
     return rc;
   mark_stage(1, st);
-  if ((rc = ccf_route(w.idx, n, num_expert, top_k, capacity, w.counts, w.offsets, w.pos, w.src_row,
-                      w.dst_row, w.inv_pos, w.idx_kept, w.route_ws, w.route_bytes, stream)))
+  // the tile plans of both GEMMs are built by two more workgroups of the routing stage's last
+  // launch (they need the offsets only), which saves the GEMMs a small launch each
+  PlanReq plans[2];
+  const bool planned = forward_plan_request(1, n, num_expert, d_model, d_ffn, w.ffn_ws, &plans[0]) &&
+                       forward_plan_request(2, n, num_expert, d_model, d_ffn, w.ffn_ws, &plans[1]);
+  if ((rc = route_with_plans(w.idx, n, num_expert, top_k, capacity, w.counts, w.offsets, w.pos, w.src_row,
+                             w.dst_row, w.inv_pos, w.idx_kept, w.route_ws, w.route_bytes, st, plans,
+                             planned ? 2 : 0)))
     return rc;
   mark_stage(2, st);
-  if ((rc = ccf_ffn1_forward(x, w.src_row, nullptr, w.offsets, n, num_expert, d_model, d_ffn, w1, b1, 1, w.h,
-                             w.ffn_ws, w.ffn_bytes, stream)))
+  if ((rc = ffn1_forward(x, w.src_row, nullptr, w.offsets, n, num_expert, d_model, d_ffn, w1, b1, 1, w.h,
+                         w.ffn_ws, w.ffn_bytes, st, planned)))
     return rc;
   mark_stage(3, st);
   // top-1 without a capacity limit: every token has one slot, its score is exactly 1 (the softmax of
   // one logit) and its flat row is its token row, so FFN2 writes the layer output itself
   const bool direct = top_k == 1 && capacity < 0;
-  if ((rc = ccf_ffn2_forward(w.h, nullptr, w.dst_row, w.offsets, n, num_expert, d_model, d_ffn, w2, b2,
-                             nullptr, direct ? out : w.y_flat, w.ffn_ws, w.ffn_bytes, stream)))
+  if ((rc = ffn2_forward(w.h, nullptr, w.dst_row, w.offsets, n, num_expert, d_model, d_ffn, w2, b2,
+                         nullptr, direct ? out : w.y_flat, w.ffn_ws, w.ffn_bytes, st, planned)))
     return rc;
   mark_stage(4, st);
   if (!direct) {

@@ -15,198 +15,19 @@
 // blocks on the host in Python (mix_moe/mix_moe/transformer.py:150-250) and
 // copies seven arrays to the device per call; here a one-workgroup kernel
 // derives the tile list from the offsets on the device.
-#include <limits.h>
-
 #include "ccf_common.h"
 #include "gemm_tile.h"
+#include "plan.h"
 
 namespace ccf {
 namespace {
 
 // ---- tile plan ---------------------------------------------------------------
-// The plan is one 16-byte entry per launched workgroup, indexed by the hardware
-// workgroup id: {expert, first sorted row, rows in the M tile, N tile}, expert
-// = -1 for workgroups with nothing to do.  A workgroup learns its whole
-// assignment from a single load.
-__host__ __device__ inline size_t plan_ints(long long wgs) { return 4 * static_cast<size_t>(wgs); }
-
-__host__ __device__ inline long long launched_wgs(int max_tiles, int n_tiles_n) {
-  long long w = static_cast<long long>(max_tiles) * n_tiles_n;
-  return ((w + 7) / 8 + 2) * 8;                   // per XCD: a share of each of the two tile classes, rounded up
-}
-
-constexpr int kOrderGroupM = 8;
-
-// Scratch of the split last round, in front of the plan in the caller's workspace:
-//   [0, 16)              header: tile slots T (a multiple of 8; slot t belongs to XCD t % 8), parts S
-//   [256, 256 + 16*256)  entries {expert, row0, rows, tile_n | part << 16 | S << 24} by workgroup
-//                        id: part s of tile slot t at (t % 8) + 8 * ((t / 8) * S + s); expert -1 = none
-//   [kTailHead, ...)     256 partial tiles of 256 x 256 fp32, by the same workgroup id
-constexpr int kTailMaxParts = 256;
-constexpr int kTailMaxTiles = kTailMaxParts / 2;     // tile slots: every tile has at least two parts
-constexpr size_t kTailHead = 256 + 16 * kTailMaxParts;
-constexpr size_t kTailBytes = kTailHead + static_cast<size_t>(kTailMaxParts) * 256 * 256 * 4;
-
-// Rows of M tile i of an expert with cnt rows in nt = ceil(cnt / BM) tiles.  When
-// the last tile would hold at most BM/2 rows, it and the one before it share
-// their rows evenly instead: a nearly empty tile still streams a whole weight
-// panel, on its own and from HBM (its siblings have long passed), which costs
-// about as much as a full tile; two half-full tiles run in step with their
-// siblings, share the panel in L2, and skip half of their MFMAs.
-__device__ inline void tile_rows(int cnt, int nt, int i, int BM, int &first_row, int &rows) {
-  const int last = cnt - (nt - 1) * BM;
-  if (nt >= 2 && last <= BM / 2 && i >= nt - 2) {
-    const int both = BM + last;
-    const int h = (both + 1) / 2;
-    first_row = (nt - 2) * BM + (i == nt - 2 ? 0 : h);
-    rows = i == nt - 2 ? h : both - h;
-  } else {
-    first_row = i * BM;
-    rows = (cnt - i * BM) < BM ? (cnt - i * BM) : BM;
-  }
-}
-
-// Tiles come in two classes.  A "long" M tile holds more than BM/2 rows; a
-// "short" one is the only tile of an expert with at most BM/2 rows, skips most
-// of its MFMAs and ends early.  Workgroups that share an
-// XCD share weight and token tiles through its L2 only while they walk K in
-// step, and a workgroup that ends early puts every later one on its CU out of
-// step, so all long tiles are launched first and the short ones after them,
-// where they also even out the end of the launch.
+// build_plan() (plan.h) in a launch of its own; the layer's forward call lets the routing
+// stage build both of its plans instead.
 __global__ void __launch_bounds__(1024)
-plan_kernel(const int32_t *__restrict__ offsets, int E, int BM, int max_tiles, int max_rows,
-            int n_tiles_n, int32_t *__restrict__ plan, int spx, int k_tiles, int32_t *__restrict__ tail) {
-  __shared__ int s_full[8];        // split last round: slots of XCD x from s_full[x] on go to the tail list
-  __shared__ int s_parts;          // parts per tail tile, 0 = no split
-  __shared__ int s_off[1025];
-  __shared__ int s_long[1025];     // exclusive scan of long M tiles per expert
-  __shared__ int s_short[1025];    // exclusive scan of short M tiles per expert (0 or 1 each)
-  for (int e = threadIdx.x; e <= E; e += blockDim.x) {
-    int v = offsets[e];
-    s_off[e] = v < max_rows ? v : max_rows;          // never plan past the caller's bound
-  }
-  __syncthreads();
-  if (threadIdx.x < 64) {
-    const int lane = threadIdx.x;
-    int carry_l = 0, carry_s = 0;
-    for (int e0 = 0; e0 < E; e0 += 64) {
-      const int e = e0 + lane;
-      int cnt = e < E ? s_off[e + 1] - s_off[e] : 0;
-      cnt = cnt > 0 ? cnt : 0;
-      const int nt = (cnt + BM - 1) / BM;
-      const int ns = (nt == 1 && cnt <= BM / 2) ? 1 : 0;        // a short tile only when it is the expert's only one
-      const int nl = nt - ns;
-      int inc_l = nl, inc_s = ns;
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        int ol = __shfl_up(inc_l, off, 64);
-        int os = __shfl_up(inc_s, off, 64);
-        if (lane >= off) { inc_l += ol; inc_s += os; }
-      }
-      if (e < E) { s_long[e] = carry_l + inc_l - nl; s_short[e] = carry_s + inc_s - ns; }
-      carry_l += __shfl(inc_l, 63, 64);
-      carry_s += __shfl(inc_s, 63, 64);
-    }
-    if (lane == 0) { s_long[E] = carry_l; s_short[E] = carry_s; }
-  }
-  const long long wgs = launched_wgs(max_tiles, n_tiles_n);
-  int4v *entry = reinterpret_cast<int4v *>(plan);
-  for (long long b = threadIdx.x; b < wgs; b += blockDim.x) entry[b] = int4v{-1, 0, 0, 0};
-  int4v *tent = reinterpret_cast<int4v *>(tail + 64);
-  if (tail)
-    for (int b = threadIdx.x; b < kTailMaxParts; b += blockDim.x) tent[b] = int4v{-1, 0, 0, 0};
-  __syncthreads();
-  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn, so XCD x
-  // runs ids x, x+8, ... in order.  Each class is cut into eight equal
-  // contiguous runs of logical tile ids, one per XCD (one L2): with nl long
-  // tiles on XCD x, its slot j is long tile x*per_long + j for j < nl, else
-  // short tile x*per_short + (j - nl).  The used slots of an XCD are a prefix:
-  // the first idle entry ends its list.
-  const long long total_long = static_cast<long long>(s_long[E]) * n_tiles_n;
-  const long long total_short = static_cast<long long>(s_short[E]) * n_tiles_n;
-  const long long per_long = (total_long + 7) / 8;
-  const long long per_short = (total_short + 7) / 8;
-  // The split last round (see "split-K tail" below).  XCD x holds used_x tiles; with spx
-  // persistent workgroups per XCD the last used_x % spx of them form a partly filled round.
-  // When that round is at most half full on every XCD, its tiles leave the plan: tile i of
-  // XCD x's last round, part s of S, becomes tail entry x + 8 * (i * S + s), the workgroup id
-  // that the hardware places on the same XCD, so the patch of neighbouring tiles keeps sharing
-  // its operands through that XCD's L2 (parts of the same K range walk K in step).
-  if (threadIdx.x == 0) {
-    int max_r = 0;
-    for (int x = 0; x < 8; ++x) {
-      long long nl_x = total_long - x * per_long, ns_x = total_short - x * per_short;
-      nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
-      ns_x = ns_x < 0 ? 0 : (ns_x > per_short ? per_short : ns_x);
-      const int used = static_cast<int>(nl_x + ns_x);
-      const int full = spx > 0 ? used / spx * spx : used;
-      s_full[x] = full;
-      max_r = (used - full) > max_r ? (used - full) : max_r;
-    }
-    int S = 0;
-    if (tail && spx > 0 && max_r > 0 && max_r * 2 <= spx) {
-      S = spx / max_r;
-      S = S > 8 ? 8 : S;
-      S = S > k_tiles / 4 ? k_tiles / 4 : S;           // at least four K tiles per part
-      S = (S >= 2 && 8 * max_r * S <= kTailMaxParts) ? S : 0;
-    }
-    s_parts = S;
-    if (!S)
-      for (int x = 0; x < 8; ++x) s_full[x] = INT_MAX;
-    if (tail) { tail[0] = S ? 8 * max_r : 0; tail[1] = S; }
-  }
-  __syncthreads();
-  const int S = s_parts;
-  // slot j of XCD x: into the plan, or cut into S parts on the tail list
-  auto place = [&](long long j, long long x, int4v v) {
-    const long long b = j * 8 + x;
-    if (j >= s_full[x]) {
-      const int i = static_cast<int>(j) - s_full[x];
-      for (int part = 0; part < S; ++part)
-        tent[x + 8 * (i * S + part)] = int4v{v[0], v[1], v[2], v[3] | (part << 16) | (S << 24)};
-    } else if (b < wgs) {
-      entry[b] = v;
-    }
-  };
-  // one wavefront per expert
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
-  for (int e = wave; e < E; e += nwave) {
-    const int lo = s_off[e];
-    int cnt = s_off[e + 1] - lo;
-    cnt = cnt > 0 ? cnt : 0;
-    const int nl = s_long[e + 1] - s_long[e];
-    const int ns = s_short[e + 1] - s_short[e];
-    // Launch order of an expert's long tiles: runs of up to kOrderGroupM M
-    // tiles, and inside a run the M tile varies fastest.  The ~32 workgroups an
-    // XCD runs at a time (consecutive logical ids) then form a patch of a M
-    // tiles x 32/a N tiles of ONE expert: a weight tile is pulled from HBM once
-    // for a M tiles, a token tile once for 32/a N tiles, and HBM traffic per
-    // patch, which goes as 1/a + a/32, is near its minimum for a = 4..8.
-    const long long first = static_cast<long long>(s_long[e]) * n_tiles_n;
-    for (int l = lane; l < nl * n_tiles_n; l += 64) {
-      const int run = l / (kOrderGroupM * n_tiles_n);            // which run of M tiles
-      const int run_first = run * kOrderGroupM;
-      const int run_size = (nl - run_first) < kOrderGroupM ? (nl - run_first) : kOrderGroupM;
-      const int in_run = l - run * kOrderGroupM * n_tiles_n;
-      const int i = run_first + in_run % run_size;               // M tile within the expert
-      const int tn = in_run / run_size;
-      const long long logical = first + l;
-      int first_row, rows;
-      tile_rows(cnt, nl, i, BM, first_row, rows);
-      place(logical % per_long, logical / per_long, int4v{e, lo + first_row, rows, tn});   // hardware id = slot * 8 + XCD
-    }
-    if (ns) {
-      const int i = nl;                                          // the expert's last M tile
-      const long long first_s = static_cast<long long>(s_short[e]) * n_tiles_n;
-      for (int tn = lane; tn < n_tiles_n; tn += 64) {
-        const long long logical = first_s + tn;
-        const long long x = logical / per_short;
-        long long nl_x = total_long - x * per_long;              // long tiles on this XCD
-        nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
-        place(nl_x + logical % per_short, x, int4v{e, lo + i * BM, cnt - i * BM, tn});
-      }
-    }
-  }
+plan_kernel(PlanReq rq, const int32_t *__restrict__ offsets, int E) {
+  build_plan(rq, offsets, E);
 }
 
 // ---- grouped GEMM kernel -------------------------------------------------------
@@ -905,20 +726,67 @@ int max_tiles_for(int max_rows, int E, int bm) { return (max_rows + bm - 1) / bm
 
 constexpr int kMinBN = 128;
 
-// Workspace of one grouped GEMM: the split-K tail area, then the tile plan.
-size_t plan_bytes(int max_rows, int E, int n_max) {
-  return kTailBytes + round_up(sizeof(int32_t) * plan_ints(launched_wgs(max_tiles_for(max_rows, E, kMinBM),
-                                                                         (n_max + kMinBN - 1) / kMinBN)), 256);
+// Workspace of one grouped GEMM: the split-K tail area, then the tile plan.  A second plan
+// (region 1: header and entries of its own, then the plan; the partial tiles are shared) follows
+// in the forward workspace, so that the plans of both GEMMs of a layer can exist at once.
+size_t plan_only_bytes(int max_rows, int E, int n_max) {
+  return round_up(sizeof(int32_t) * plan_ints(launched_wgs(max_tiles_for(max_rows, E, kMinBM),
+                                                           (n_max + kMinBN - 1) / kMinBN)), 256);
+}
+size_t plan_bytes(int max_rows, int E, int n_max) { return kTailBytes + plan_only_bytes(max_rows, E, n_max); }
+size_t forward_ws_bytes(int max_rows, int E, int n_max) {
+  return plan_bytes(max_rows, E, n_max) + kTailHead + plan_only_bytes(max_rows, E, n_max);
 }
 
+// Everything the launches of one grouped GEMM derive from its sizes, and the request that
+// builds its plan.
+struct GemmSetup {
+  const Launch *v;
+  bool second, split;
+  int grid;
+  long long wgs;
+  int32_t *tail, *plan;
+  float *partial;
+  PlanReq req;
+};
+
+GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void *workspace, int region) {
+  GemmSetup g;
+  char *ws = static_cast<char *>(workspace);
+  g.partial = reinterpret_cast<float *>(ws + kTailHead);
+  if (region == 0) {
+    g.tail = reinterpret_cast<int32_t *>(ws);                                       // header and entries
+    g.plan = reinterpret_cast<int32_t *>(ws + kTailBytes);
+  } else {
+    g.tail = reinterpret_cast<int32_t *>(ws + plan_bytes(max_rows, E, N > K ? N : K));
+    g.plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.tail) + kTailHead);
+  }
+  const bool gelu = epi != kEpiPlain;
+  g.v = &kVariants[b_kn ? kKnVariant : (epi >= kEpiGeluKeep ? kTrainVariant : g_variant)];
+  const Launch &v = *g.v;
+  // which of the entry's two kernels: the K-N and training entries hold the GELU-gradient form in the second slot
+  g.second = b_kn ? epi == kEpiGeluGrad : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu);
+  const int max_tiles = max_tiles_for(max_rows, E, v.bm);
+  const int n_tiles_n = (N + v.bn - 1) / v.bn;
+  g.wgs = launched_wgs(max_tiles, n_tiles_n);                   // worst-case tile count
+  g.grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
+  // the last, partly filled round is cut along K and spread over all workgroups (forward forms;
+  // worth its two small launches only where a tile is long: K of 4096 and more)
+  g.split = g_split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && g.grid >= 8 && g.grid <= g.wgs &&
+            g.grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= g_split_tail_min_kt;
+  g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, g.plan,
+                  g.split ? g.tail : nullptr};
+  return g;
+}
+
+// plan_ready: the plan (and the split list) of this very call was already built in `region`
+// by forward_plan_request()'s request.
 int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets, int max_rows, int E,
                  int N, int K, const half_t *B, const half_t *bias, int epi, half_t *C,
-                 const int32_t *c_rows, const half_t *row_scale, int32_t *workspace, hipStream_t stream,
-                 const char *what, bool b_kn = false, half_t *C2 = nullptr) {
+                 const int32_t *c_rows, const half_t *row_scale, void *workspace, hipStream_t stream,
+                 const char *what, bool b_kn = false, half_t *C2 = nullptr, int region = 0,
+                 bool plan_ready = false) {
   CCF_REQUIRE(A && offsets && B && C && workspace, CCF_ERR_ARG, "%s: null pointer", what);
-  int32_t *tail = workspace;                                                        // header and entries
-  float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + kTailHead);
-  int32_t *plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(workspace) + kTailBytes);
   const bool gelu = epi != kEpiPlain;
   CCF_REQUIRE(epi >= kEpiPlain && epi <= kEpiGeluGrad && (epi < kEpiGeluKeep || (C2 && aligned16(C2))), CCF_ERR_ARG,
               "%s: epilogue %d needs the pre-activation buffer", what, epi);
@@ -934,22 +802,18 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
               "%s: operands must be 16-byte aligned", what);
   CCF_REQUIRE(!(gelu && row_scale), CCF_ERR_ARG, "%s: the GELU epilogue takes no row scale", what);
   if (max_rows == 0) return CCF_OK;
-  const Launch &v = kVariants[b_kn ? kKnVariant : (epi >= kEpiGeluKeep ? kTrainVariant : g_variant)];
-  // which of the entry's two kernels: the K-N and training entries hold the GELU-gradient form in the second slot
-  const bool second = b_kn ? epi == kEpiGeluGrad : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu);
-  const int max_tiles = max_tiles_for(max_rows, E, v.bm);
-  const int n_tiles_n = (N + v.bn - 1) / v.bn;
-  const long long wgs = launched_wgs(max_tiles, n_tiles_n);     // worst-case tile count
+  const GemmSetup gs = setup_gemm(max_rows, E, N, K, epi, b_kn, workspace, region);
+  const Launch &v = *gs.v;
+  const bool second = gs.second, split = gs.split;
+  const int grid = gs.grid;
+  const long long wgs = gs.wgs;
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
-  const int grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
-  // the last, partly filled round is cut along K and spread over all workgroups (forward forms;
-  // worth its two small launches only where a tile is long: K of 4096 and more)
-  const bool split = g_split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && grid >= 8 && grid <= wgs &&
-                     grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN &&
-                     K / 64 >= g_split_tail_min_kt;
-  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, offsets, E, v.bm, max_tiles,
-                     max_rows, n_tiles_n, plan, split ? grid / 8 : 0, K / 64, split ? tail : nullptr);
-  if (int rc = check_launch("plan_kernel")) return rc;
+  if (!plan_ready) {
+    hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, gs.req, offsets, E);
+    if (int rc = check_launch("plan_kernel")) return rc;
+  }
+  int32_t *plan = gs.plan, *tail = gs.tail;
+  float *partial = gs.partial;
   GroupedArgs p;
   p.A = A;
   p.a_rows = a_rows;
@@ -1001,8 +865,10 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const int max_rows = E * M;
   const int max_tiles = max_tiles_for(max_rows, E, Cfg5::BM);
   const int n_tiles_n = (N + Cfg5::BN - 1) / Cfg5::BN;
-  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, row_off, E, Cfg5::BM, max_tiles,
-                     max_rows, n_tiles_n, plan, 0, 0, static_cast<int32_t *>(nullptr));
+  const long long wgs = launched_wgs(max_tiles, n_tiles_n);
+  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
+  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream,
+                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, plan, nullptr}, row_off, E);
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
   p.A = A;
@@ -1022,8 +888,6 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.seg_rows = M;
   p.tail = nullptr;
   p.partial = nullptr;
-  const long long wgs = launched_wgs(max_tiles, n_tiles_n);
-  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   const int grid = persistent_grid();
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;
@@ -1162,21 +1026,58 @@ extern "C" int ccf_set_option(const char *name, int value) {
 
 extern "C" size_t ccf_ffn_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn) {
   if (max_rows < 0 || num_expert <= 0 || d_model <= 0 || d_ffn <= 0) return 0;
-  return ccf::plan_bytes(max_rows, num_expert, d_model > d_ffn ? d_model : d_ffn);
+  return ccf::forward_ws_bytes(max_rows, num_expert, d_model > d_ffn ? d_model : d_ffn);
 }
 
-extern "C" int ccf_ffn1_forward(const void *x, const int32_t *src_row, const int32_t *dst_row,
-                                const int32_t *offsets, int max_rows, int num_expert, int d_model,
-                                int d_ffn, const void *w1, const void *b1, int apply_gelu, void *h,
-                                void *workspace, size_t workspace_bytes, ccf_stream_t stream) {
-  using namespace ccf;
+namespace ccf {
+
+// Plan requests of the layer's two forward GEMMs (which = 1: FFN1 with GELU, 2: FFN2), for a
+// caller that builds the plans itself (the routing stage does) and then passes plan_ready.
+// False when the sizes are not ones the GEMM accepts: the caller then leaves the plan to it.
+bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, PlanReq *out) {
+  if (!workspace || max_rows <= 0 || E <= 0 || E > 1024 || d <= 0 || f <= 0 || d % 64 || f % 64) return false;
+  const int N = which == 1 ? f : d, K = which == 1 ? d : f;
+  const GemmSetup gs = setup_gemm(max_rows, E, N, K, which == 1 ? kEpiGelu : kEpiPlain, false, workspace,
+                                  which == 1 ? 0 : 1);
+  if (gs.wgs >= (1ll << 31)) return false;
+  *out = gs.req;
+  return true;
+}
+
+int ffn1_forward(const void *x, const int32_t *src_row, const int32_t *dst_row, const int32_t *offsets,
+                 int max_rows, int num_expert, int d_model, int d_ffn, const void *w1, const void *b1,
+                 int apply_gelu, void *h, void *workspace, size_t workspace_bytes, hipStream_t stream,
+                 bool plan_ready) {
   const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
   CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
               "ffn1: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   return grouped_gemm(static_cast<const half_t *>(x), src_row, offsets, max_rows, num_expert, d_ffn,
                       d_model, static_cast<const half_t *>(w1), static_cast<const half_t *>(b1),
                       apply_gelu != 0 ? kEpiGelu : kEpiPlain, static_cast<half_t *>(h), dst_row, nullptr,
-                      static_cast<int32_t *>(workspace), as_stream(stream), "ffn1");
+                      workspace, stream, "ffn1", false, nullptr, 0, plan_ready && apply_gelu != 0);
+}
+
+int ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row, const int32_t *offsets,
+                 int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
+                 const void *row_scale, void *y, void *workspace, size_t workspace_bytes,
+                 hipStream_t stream, bool plan_ready) {
+  const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
+  CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
+              "ffn2: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  return grouped_gemm(static_cast<const half_t *>(h), src_row, offsets, max_rows, num_expert, d_model,
+                      d_ffn, static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), kEpiPlain,
+                      static_cast<half_t *>(y), dst_row, static_cast<const half_t *>(row_scale),
+                      workspace, stream, "ffn2", false, nullptr, 1, plan_ready);
+}
+
+}  // namespace ccf
+
+extern "C" int ccf_ffn1_forward(const void *x, const int32_t *src_row, const int32_t *dst_row,
+                                const int32_t *offsets, int max_rows, int num_expert, int d_model,
+                                int d_ffn, const void *w1, const void *b1, int apply_gelu, void *h,
+                                void *workspace, size_t workspace_bytes, ccf_stream_t stream) {
+  return ccf::ffn1_forward(x, src_row, dst_row, offsets, max_rows, num_expert, d_model, d_ffn, w1, b1,
+                           apply_gelu, h, workspace, workspace_bytes, ccf::as_stream(stream), false);
 }
 
 extern "C" int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row,
@@ -1184,14 +1085,8 @@ extern "C" int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int
                                 int d_ffn, const void *w2, const void *b2, const void *row_scale,
                                 void *y, void *workspace, size_t workspace_bytes,
                                 ccf_stream_t stream) {
-  using namespace ccf;
-  const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
-  CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
-              "ffn2: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-  return grouped_gemm(static_cast<const half_t *>(h), src_row, offsets, max_rows, num_expert, d_model,
-                      d_ffn, static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), kEpiPlain,
-                      static_cast<half_t *>(y), dst_row, static_cast<const half_t *>(row_scale),
-                      static_cast<int32_t *>(workspace), as_stream(stream), "ffn2");
+  return ccf::ffn2_forward(h, src_row, dst_row, offsets, max_rows, num_expert, d_model, d_ffn, w2, b2,
+                           row_scale, y, workspace, workspace_bytes, ccf::as_stream(stream), false);
 }
 
 extern "C" size_t ccf_ffn_backward_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn) {
@@ -1211,7 +1106,7 @@ extern "C" int ccf_ffn1_forward_keep(const void *x, const int32_t *src_row, cons
   return grouped_gemm(static_cast<const half_t *>(x), src_row, offsets, max_rows, num_expert, d_ffn,
                       d_model, static_cast<const half_t *>(w1), static_cast<const half_t *>(b1),
                       kEpiGeluKeep, static_cast<half_t *>(act), nullptr, nullptr,
-                      static_cast<int32_t *>(workspace), as_stream(stream), "ffn1_keep", false,
+                      workspace, as_stream(stream), "ffn1_keep", false,
                       static_cast<half_t *>(h_pre));
 }
 

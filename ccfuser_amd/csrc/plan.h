@@ -1,0 +1,228 @@
+// Tile plan of a grouped GEMM: which workgroup computes which tile, derived on the
+// device from the expert offsets.  Shared by the GEMM launcher and by the routing
+// kernels, whose last launch can build the plans of the GEMMs that follow.
+#pragma once
+
+#include <limits.h>
+
+#include "ccf_common.h"
+
+namespace ccf {
+
+// ---- tile plan ---------------------------------------------------------------
+// The plan is one 16-byte entry per launched workgroup, indexed by the hardware
+// workgroup id: {expert, first sorted row, rows in the M tile, N tile}, expert
+// = -1 for workgroups with nothing to do.  A workgroup learns its whole
+// assignment from a single load.
+__host__ __device__ inline size_t plan_ints(long long wgs) { return 4 * static_cast<size_t>(wgs); }
+
+__host__ __device__ inline long long launched_wgs(int max_tiles, int n_tiles_n) {
+  long long w = static_cast<long long>(max_tiles) * n_tiles_n;
+  return ((w + 7) / 8 + 2) * 8;                   // per XCD: a share of each of the two tile classes, rounded up
+}
+
+constexpr int kOrderGroupM = 8;
+
+// Scratch of the split last round, in front of the plan in the caller's workspace:
+//   [0, 16)              header: tile slots T (a multiple of 8; slot t belongs to XCD t % 8), parts S
+//   [256, 256 + 16*256)  entries {expert, row0, rows, tile_n | part << 16 | S << 24} by workgroup
+//                        id: part s of tile slot t at (t % 8) + 8 * ((t / 8) * S + s); expert -1 = none
+//   [kTailHead, ...)     256 partial tiles of 256 x 256 fp32, by the same workgroup id
+constexpr int kTailMaxParts = 256;
+constexpr int kTailMaxTiles = kTailMaxParts / 2;     // tile slots: every tile has at least two parts
+constexpr size_t kTailHead = 256 + 16 * kTailMaxParts;
+constexpr size_t kTailBytes = kTailHead + static_cast<size_t>(kTailMaxParts) * 256 * 256 * 4;
+
+// Rows of M tile i of an expert with cnt rows in nt = ceil(cnt / BM) tiles.  When
+// the last tile would hold at most BM/2 rows, it and the one before it share
+// their rows evenly instead: a nearly empty tile still streams a whole weight
+// panel, on its own and from HBM (its siblings have long passed), which costs
+// about as much as a full tile; two half-full tiles run in step with their
+// siblings, share the panel in L2, and skip half of their MFMAs.
+__device__ inline void tile_rows(int cnt, int nt, int i, int BM, int &first_row, int &rows) {
+  const int last = cnt - (nt - 1) * BM;
+  if (nt >= 2 && last <= BM / 2 && i >= nt - 2) {
+    const int both = BM + last;
+    const int h = (both + 1) / 2;
+    first_row = (nt - 2) * BM + (i == nt - 2 ? 0 : h);
+    rows = i == nt - 2 ? h : both - h;
+  } else {
+    first_row = i * BM;
+    rows = (cnt - i * BM) < BM ? (cnt - i * BM) : BM;
+  }
+}
+
+// Tiles come in two classes.  A "long" M tile holds more than BM/2 rows; a
+// "short" one is the only tile of an expert with at most BM/2 rows, skips most
+// of its MFMAs and ends early.  Workgroups that share an
+// XCD share weight and token tiles through its L2 only while they walk K in
+// step, and a workgroup that ends early puts every later one on its CU out of
+// step, so all long tiles are launched first and the short ones after them,
+// where they also even out the end of the launch.
+// What one plan needs besides the offsets; passed by value to the kernel that builds it.
+struct PlanReq {
+  int BM, max_tiles, max_rows, n_tiles_n;
+  int spx;          // persistent workgroups per XCD when the last round may be split, else 0
+  int k_tiles;      // K tiles of a tile (bounds the parts of a split)
+  int32_t *plan;
+  int32_t *tail;    // split scratch (header and entries), or NULL
+};
+
+// Built by ONE workgroup of any size that is a multiple of 64 (all of its threads call this).
+__device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__ offsets, int E) {
+  const int BM = rq.BM, max_tiles = rq.max_tiles, max_rows = rq.max_rows, n_tiles_n = rq.n_tiles_n;
+  const int spx = rq.spx, k_tiles = rq.k_tiles;
+  int32_t *__restrict__ plan = rq.plan;
+  int32_t *__restrict__ tail = rq.tail;
+  __shared__ int s_full[8];        // split last round: slots of XCD x from s_full[x] on go to the tail list
+  __shared__ int s_parts;          // parts per tail tile, 0 = no split
+  __shared__ int s_off[1025];
+  __shared__ int s_long[1025];     // exclusive scan of long M tiles per expert
+  __shared__ int s_short[1025];    // exclusive scan of short M tiles per expert (0 or 1 each)
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) {
+    int v = offsets[e];
+    s_off[e] = v < max_rows ? v : max_rows;          // never plan past the caller's bound
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    int carry_l = 0, carry_s = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      const int e = e0 + lane;
+      int cnt = e < E ? s_off[e + 1] - s_off[e] : 0;
+      cnt = cnt > 0 ? cnt : 0;
+      const int nt = (cnt + BM - 1) / BM;
+      const int ns = (nt == 1 && cnt <= BM / 2) ? 1 : 0;        // a short tile only when it is the expert's only one
+      const int nl = nt - ns;
+      int inc_l = nl, inc_s = ns;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        int ol = __shfl_up(inc_l, off, 64);
+        int os = __shfl_up(inc_s, off, 64);
+        if (lane >= off) { inc_l += ol; inc_s += os; }
+      }
+      if (e < E) { s_long[e] = carry_l + inc_l - nl; s_short[e] = carry_s + inc_s - ns; }
+      carry_l += __shfl(inc_l, 63, 64);
+      carry_s += __shfl(inc_s, 63, 64);
+    }
+    if (lane == 0) { s_long[E] = carry_l; s_short[E] = carry_s; }
+  }
+  // the launcher checks that the worst-case tile count, and with it every count below, fits an int
+  const int wgs = static_cast<int>(launched_wgs(max_tiles, n_tiles_n));
+  int4v *entry = reinterpret_cast<int4v *>(plan);
+  for (int b = threadIdx.x; b < wgs; b += blockDim.x) entry[b] = int4v{-1, 0, 0, 0};
+  int4v *tent = reinterpret_cast<int4v *>(tail + 64);
+  if (tail)
+    for (int b = threadIdx.x; b < kTailMaxParts; b += blockDim.x) tent[b] = int4v{-1, 0, 0, 0};
+  __syncthreads();
+  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn, so XCD x
+  // runs ids x, x+8, ... in order.  Each class is cut into eight equal
+  // contiguous runs of logical tile ids, one per XCD (one L2): with nl long
+  // tiles on XCD x, its slot j is long tile x*per_long + j for j < nl, else
+  // short tile x*per_short + (j - nl).  The used slots of an XCD are a prefix:
+  // the first idle entry ends its list.
+  const int total_long = s_long[E] * n_tiles_n;
+  const int total_short = s_short[E] * n_tiles_n;
+  const int per_long = (total_long + 7) / 8;
+  const int per_short = (total_short + 7) / 8;
+  // The split last round (see "split-K tail" below).  XCD x holds used_x tiles; with spx
+  // persistent workgroups per XCD the last used_x % spx of them form a partly filled round.
+  // When that round is at most half full on every XCD, its tiles leave the plan: tile i of
+  // XCD x's last round, part s of S, becomes tail entry x + 8 * (i * S + s), the workgroup id
+  // that the hardware places on the same XCD, so the patch of neighbouring tiles keeps sharing
+  // its operands through that XCD's L2 (parts of the same K range walk K in step).
+  if (threadIdx.x == 0) {
+    int max_r = 0;
+    for (int x = 0; x < 8; ++x) {
+      int nl_x = total_long - x * per_long, ns_x = total_short - x * per_short;
+      nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
+      ns_x = ns_x < 0 ? 0 : (ns_x > per_short ? per_short : ns_x);
+      const int used = nl_x + ns_x;
+      const int full = spx > 0 ? used / spx * spx : used;
+      s_full[x] = full;
+      max_r = (used - full) > max_r ? (used - full) : max_r;
+    }
+    int S = 0;
+    if (tail && spx > 0 && max_r > 0 && max_r * 2 <= spx) {
+      S = spx / max_r;
+      S = S > 8 ? 8 : S;
+      S = S > k_tiles / 4 ? k_tiles / 4 : S;           // at least four K tiles per part
+      S = (S >= 2 && 8 * max_r * S <= kTailMaxParts) ? S : 0;
+    }
+    s_parts = S;
+    if (!S)
+      for (int x = 0; x < 8; ++x) s_full[x] = INT_MAX;
+    if (tail) { tail[0] = S ? 8 * max_r : 0; tail[1] = S; }
+  }
+  __syncthreads();
+  const int S = s_parts;
+  // slot j of XCD x: into the plan, or cut into S parts on the tail list
+  auto place = [&](int j, int x, int4v v) {
+    const int b = j * 8 + x;
+    if (j >= s_full[x]) {
+      const int i = j - s_full[x];
+      for (int part = 0; part < S; ++part)
+        tent[x + 8 * (i * S + part)] = int4v{v[0], v[1], v[2], v[3] | (part << 16) | (S << 24)};
+    } else if (b < wgs) {
+      entry[b] = v;
+    }
+  };
+  // one wavefront per expert
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
+  for (int e = wave; e < E; e += nwave) {
+    const int lo = s_off[e];
+    int cnt = s_off[e + 1] - lo;
+    cnt = cnt > 0 ? cnt : 0;
+    const int nl = s_long[e + 1] - s_long[e];
+    const int ns = s_short[e + 1] - s_short[e];
+    // Launch order of an expert's long tiles: runs of up to kOrderGroupM M
+    // tiles, and inside a run the M tile varies fastest.  The ~32 workgroups an
+    // XCD runs at a time (consecutive logical ids) then form a patch of a M
+    // tiles x 32/a N tiles of ONE expert: a weight tile is pulled from HBM once
+    // for a M tiles, a token tile once for 32/a N tiles, and HBM traffic per
+    // patch, which goes as 1/a + a/32, is near its minimum for a = 4..8.
+    const int first = s_long[e] * n_tiles_n;
+    for (int l = lane; l < nl * n_tiles_n; l += 64) {
+      const int run = l / (kOrderGroupM * n_tiles_n);            // which run of M tiles
+      const int run_first = run * kOrderGroupM;
+      const int run_size = (nl - run_first) < kOrderGroupM ? (nl - run_first) : kOrderGroupM;
+      const int in_run = l - run * kOrderGroupM * n_tiles_n;
+      const int i = run_first + in_run % run_size;               // M tile within the expert
+      const int tn = in_run / run_size;
+      const int logical = first + l;
+      int first_row, rows;
+      tile_rows(cnt, nl, i, BM, first_row, rows);
+      place(logical % per_long, logical / per_long, int4v{e, lo + first_row, rows, tn});   // hardware id = slot * 8 + XCD
+    }
+    if (ns) {
+      const int i = nl;                                          // the expert's last M tile
+      const int first_s = s_short[e] * n_tiles_n;
+      for (int tn = lane; tn < n_tiles_n; tn += 64) {
+        const int logical = first_s + tn;
+        const int x = logical / per_short;
+        int nl_x = total_long - x * per_long;              // long tiles on this XCD
+        nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
+        place(nl_x + logical % per_short, x, int4v{e, lo + i * BM, cnt - i * BM, tn});
+      }
+    }
+  }
+}
+
+// ---- the layer's forward call: plans built by the routing stage ------------------
+// ffn.hip
+bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, PlanReq *out);
+int ffn1_forward(const void *x, const int32_t *src_row, const int32_t *dst_row, const int32_t *offsets,
+                 int max_rows, int num_expert, int d_model, int d_ffn, const void *w1, const void *b1,
+                 int apply_gelu, void *h, void *workspace, size_t workspace_bytes, hipStream_t stream,
+                 bool plan_ready);
+int ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row, const int32_t *offsets,
+                 int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
+                 const void *row_scale, void *y, void *workspace, size_t workspace_bytes,
+                 hipStream_t stream, bool plan_ready);
+// route.hip: ccf_route(), whose last launch also builds n_plans (0..2) tile plans from the offsets
+int route_with_plans(const int64_t *gate_idx, int n_flat, int num_expert, int top_k, int capacity,
+                     int32_t *counts, int32_t *offsets, int64_t *pos, int32_t *src_row, int32_t *dst_row,
+                     int32_t *inv_pos, int64_t *idx_kept, void *workspace, size_t workspace_bytes,
+                     hipStream_t stream, const PlanReq *plans, int n_plans);
+
+}  // namespace ccf

@@ -16,6 +16,7 @@
 //          wavefront (ballot / popcount), then the scatter of pos and friends
 // Integer adds commute, so the results do not depend on scheduling.
 #include "ccf_common.h"
+#include "plan.h"
 
 namespace ccf {
 namespace {
@@ -140,7 +141,13 @@ pos_kernel(const int64_t *__restrict__ idx, int n, int E, int nbits, int top_k, 
            const int32_t *__restrict__ chunk_base, const int32_t *__restrict__ offsets,
            int64_t *__restrict__ pos, int32_t *__restrict__ src_row,
            int32_t *__restrict__ dst_row, int32_t *__restrict__ inv_pos,
-           int64_t *__restrict__ idx_kept) {
+           int64_t *__restrict__ idx_kept, int nchunk, PlanReq plan0, PlanReq plan1) {
+  // Workgroups past the chunks build the tile plans of the GEMMs that follow: the offsets are
+  // final since the scan, and the plans then cost no launch of their own.
+  if (static_cast<int>(blockIdx.x) >= nchunk) {
+    build_plan(blockIdx.x == static_cast<unsigned>(nchunk) ? plan0 : plan1, offsets, E);
+    return;
+  }
   extern __shared__ int s_sub[];                 // [kSub][E]
   for (int i = threadIdx.x; i < kSub * E; i += kThreads) s_sub[i] = 0;
   __syncthreads();
@@ -258,8 +265,10 @@ size_t route_ws_bytes(int n_flat, int E) {
 int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capacity,
                int32_t *counts, int32_t *offsets, int32_t *cum_inout, int64_t *pos,
                int32_t *src_row, int32_t *dst_row, int32_t *inv_pos, int64_t *idx_kept,
-               void *ws, size_t ws_bytes, hipStream_t stream) {
+               void *ws, size_t ws_bytes, hipStream_t stream, const PlanReq *plans = nullptr,
+               int n_plans = 0) {
   CCF_REQUIRE(gate_idx && pos, CCF_ERR_ARG, "route: null pointer");
+  CCF_REQUIRE(n_plans >= 0 && n_plans <= 2 && (n_plans == 0 || plans), CCF_ERR_ARG, "route: bad plan requests");
   CCF_REQUIRE(n_flat >= 0 && E > 0 && top_k >= 1, CCF_ERR_ARG, "route: bad size");
   CCF_REQUIRE(E <= kMaxExpert, CCF_ERR_SHAPE, "route: num_expert=%d exceeds %d", E, kMaxExpert);
   CCF_REQUIRE(ws && ws_bytes >= route_ws_bytes(n_flat, E), CCF_ERR_WORKSPACE,
@@ -273,9 +282,18 @@ int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capaci
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, chunk_cnt, nchunk, E, capacity,
                      counts, offsets, cum_inout);
   if (int rc = check_launch("scan_kernel")) return rc;
-  hipLaunchKernelGGL(pos_kernel, dim3(nchunk), dim3(kThreads), sizeof(int) * kSub * E, stream,
+  const PlanReq none{0, 0, 0, 0, 0, 0, nullptr, nullptr};
+  const size_t pos_lds = sizeof(int) * kSub * E;
+  if (pos_lds > 32768) {
+    // with the plan builder's static arrays the kernel passes 64 KB of LDS for many experts
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(pos_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(pos_lds));
+    if (e != hipSuccess) return fail(CCF_ERR_HIP, "route: LDS attribute: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(pos_kernel, dim3(nchunk + n_plans), dim3(kThreads), pos_lds, stream,
                      gate_idx, n_flat, E, nbits, top_k, capacity, chunk_cnt, offsets, pos, src_row,
-                     dst_row, inv_pos, idx_kept);
+                     dst_row, inv_pos, idx_kept, nchunk, n_plans > 0 ? plans[0] : none,
+                     n_plans > 1 ? plans[1] : none);
   return check_launch("pos_kernel");
 }
 
@@ -401,6 +419,17 @@ extern "C" int ccf_assign_pos(int32_t *cum_count, const int64_t *gate_idx, int n
   return route_impl(gate_idx, n_flat, num_expert, 1, -1, nullptr, offsets, cum_count, pos, nullptr,
                     nullptr, nullptr, nullptr, workspace, head, as_stream(stream));
 }
+
+namespace ccf {
+int route_with_plans(const int64_t *gate_idx, int n_flat, int num_expert, int top_k, int capacity,
+                     int32_t *counts, int32_t *offsets, int64_t *pos, int32_t *src_row, int32_t *dst_row,
+                     int32_t *inv_pos, int64_t *idx_kept, void *workspace, size_t workspace_bytes,
+                     hipStream_t stream, const PlanReq *plans, int n_plans) {
+  CCF_REQUIRE(counts && offsets, CCF_ERR_ARG, "route: null counts/offsets");
+  return route_impl(gate_idx, n_flat, num_expert, top_k, capacity, counts, offsets, nullptr, pos, src_row,
+                    dst_row, inv_pos, idx_kept, workspace, workspace_bytes, stream, plans, n_plans);
+}
+}  // namespace ccf
 
 extern "C" int ccf_route(const int64_t *gate_idx, int n_flat, int num_expert, int top_k,
                          int capacity, int32_t *counts, int32_t *offsets, int64_t *pos,
