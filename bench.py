@@ -24,15 +24,16 @@ sys.path.insert(0, ROOT)
 PEAK_FP16_TFLOPS = 2500.0          # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 
-# Bytes moved between L2 and the memory fabric per launch of the grouped GEMM, from two
-# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each
-# scaled by what the counter reads for a plain 256 MiB device copy in the same run (FETCH_SIZE
-# reads half the copied bytes: factor 2.0; WRITE_SIZE factor 1.0).  The summaries are in
-# profiles/grouped_gemm_<workload>_hbm_traffic.txt.  Counters cannot be read from inside a
-# normal run, so a workload without a profile reports null.
+# Bytes moved between L2 and the memory fabric per grouped GEMM, from two `rocprofv3 --pmc`
+# runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the
+# counter reads for a plain 256 MiB device copy in the same run (FETCH_SIZE reads half the
+# copied bytes: factor 2.0; WRITE_SIZE factor 1.0).  A grouped GEMM is three launches (the
+# persistent kernel, the parts of the split last round, their reduction): the figures are the
+# sums over the three.  The summaries are in profiles/grouped_gemm_<workload>_hbm_traffic.txt.
+# Counters cannot be read from inside a normal run, so a workload without a profile reports null.
 MEASURED_TRAFFIC_KIB = {
-    ("c3_mixtral", "ffn1"): {"FETCH_SIZE": 923101.2, "WRITE_SIZE": 229378.9},
-    ("c3_mixtral", "ffn2"): {"FETCH_SIZE": 1026486.6, "WRITE_SIZE": 65536.1},
+    ("c3_mixtral", "ffn1"): {"FETCH_SIZE": 931444.2, "WRITE_SIZE": 278531.2},
+    ("c3_mixtral", "ffn2"): {"FETCH_SIZE": 1045160.2, "WRITE_SIZE": 126981.0},
 }
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 
@@ -318,7 +319,8 @@ def main():
         line["ms_per_step_with_stage_events"] = wall_events / K * 1e3
         dom = "ffn1" if stage_ms["ffn1"] >= stage_ms["ffn2"] else "ffn2"
         ach = (flops / 2) / (stage_ms[dom] * 1e-3) / 1e12
-        line["roofline"] = {"kernel": f"grouped_gemm_persistent_kernel ({dom})", "bound": "mfma",
+        line["roofline"] = {"kernel": f"grouped GEMM of {dom}: grouped_gemm_persistent_kernel + "
+                                      "grouped_gemm_tail_kernel + splitk_reduce_kernel", "bound": "mfma",
                             "achieved": ach, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                             "frac": ach / PEAK_FP16_TFLOPS,
                             "traffic": measured_traffic(wl.name, dom), "traffic_unit": "bytes/launch",
