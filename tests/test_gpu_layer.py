@@ -263,3 +263,35 @@ def test_top1_output_written_by_ffn2_equals_the_staged_path(workloads):
     ops.ffn2(h, rt["dst_row"], rt["offsets"], n, w2, b2, y)
     staged = ops.combine(y, score.reshape(-1), 1, rt["inv_pos"])
     assert torch.equal(fused, staged)
+
+
+def _staged_forward(ops, args, E, k, capacity):
+    x, wg, bg, w1, b1, w2, b2 = args
+    idx, score = ops.gate_topk_softmax(x, wg, bg, k)
+    rt = ops.route(idx.reshape(-1), E, k, capacity)
+    n = x.shape[0] * k
+    h = ops.ffn1(x, rt["src_row"], rt["offsets"], n, w1, b1, gelu=True)
+    y = torch.zeros(n, x.shape[1], dtype=torch.float16, device="cuda")
+    ops.ffn2(h, rt["dst_row"], rt["offsets"], n, w2, b2, y)
+    return ops.combine(y, score.reshape(-1), k, rt["inv_pos"])
+
+
+@pytest.mark.parametrize("name,rows,variant", [("c3_mixtral", None, -1)] +
+                         [("c2_gshard", 1024, v) for v in range(7)])
+def test_fused_call_equals_stage_by_stage_calls(workloads, name, rows, variant):
+    """In the fused call the routing stage builds the tile plans of both GEMMs; stand-alone
+    GEMM calls build their own.  Same plans, same kernels, so the same bits: at full size on the
+    benchmark shape (last round of tiles split along K in both GEMMs) and, on a small batch, for
+    every GEMM variant (tile shapes and grids differ by variant)."""
+    from ccfuser_amd import ops
+    wl = workloads(name, rows) if rows else workloads(name)
+    t = wl.tensors
+    args = [t[n].cuda() for n in ("x", "wg", "bg", "w1", "b1", "w2", "b2")]
+    _say(f"fused against staged {name} T={wl.tokens} variant={variant}")
+    ops.set_option("gemm_variant", variant)
+    try:
+        fused = ops.moe_forward(*args, wl.top_k, wl.capacity)
+        staged = _staged_forward(ops, args, wl.num_expert, wl.top_k, wl.capacity)
+        assert torch.equal(fused, staged)
+    finally:
+        ops.set_option("gemm_variant", -1)
