@@ -675,6 +675,7 @@ int g_dgrad_transpose = 0;   // 1: input gradients always on a transposed copy o
 int g_split_tail = 1;        // 0: the last round of tiles is not cut along K
 constexpr int kSplitTailMinKT = 64;
 int g_split_tail_min_kt = kSplitTailMinKT;
+int g_split_max_parts = 8;
 
 struct Launch {
   int bm, bn, threads;
@@ -774,7 +775,7 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
   // worth its two small launches only where a tile is long: K of 4096 and more)
   g.split = g_split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && g.grid >= 8 && g.grid <= g.wgs &&
             g.grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= g_split_tail_min_kt;
-  g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, g.plan,
+  g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, g_split_max_parts, g.plan,
                   g.split ? g.tail : nullptr};
   return g;
 }
@@ -868,7 +869,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream,
-                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, plan, nullptr}, row_off, E);
+                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr}, row_off, E);
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
   p.A = A;
@@ -1010,6 +1011,11 @@ extern "C" int ccf_set_option(const char *name, int value) {
   if (!strcmp(name, "split_tail")) {         // 0 = off, 1 = default, n > 1: for K of n K tiles and more
     g_split_tail = value != 0;
     g_split_tail_min_kt = value > 1 ? value : kSplitTailMinKT;
+    return CCF_OK;
+  }
+  if (!strcmp(name, "split_parts")) {        // most parts a tile of the split last round is cut into
+    CCF_REQUIRE(value >= 2 && value <= 8, CCF_ERR_ARG, "set_option: split_parts %d outside 2..8", value);
+    g_split_max_parts = value;
     return CCF_OK;
   }
   if (!strcmp(name, "dgrad_transpose")) {

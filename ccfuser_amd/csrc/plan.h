@@ -64,6 +64,7 @@ struct PlanReq {
   int BM, max_tiles, max_rows, n_tiles_n;
   int spx;          // persistent workgroups per XCD when the last round may be split, else 0
   int k_tiles;      // K tiles of a tile (bounds the parts of a split)
+  int max_parts;    // most parts a tile is cut into
   int32_t *plan;
   int32_t *tail;    // split scratch (header and entries), or NULL
 };
@@ -145,7 +146,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     int S = 0;
     if (tail && spx > 0 && max_r > 0 && max_r * 2 <= spx) {
       S = spx / max_r;
-      S = S > 8 ? 8 : S;
+      S = S > rq.max_parts ? rq.max_parts : S;
       S = S > k_tiles / 4 ? k_tiles / 4 : S;           // at least four K tiles per part
       S = (S >= 2 && 8 * max_r * S <= kTailMaxParts) ? S : 0;
     }

@@ -53,14 +53,15 @@ int ccf_version(void);
 const char *ccf_last_error(void);
 
 /*
- * Tuning knobs (no counterpart in the reference).  "gemm_variant" selects the
- * grouped-GEMM main-loop variant used by the FFN entry points; -1 restores
- * the default.  "split_tail" (0 = off, 1 = default, n > 1 = for K of n*64 and more) cuts the
- * tiles of a launch's last, partly filled round along K.  "dgrad_transpose" (0/1) makes the backward's input-gradient GEMM run on a
- * transposed copy of the weight instead of reading the stored one.
- * "gate_waves" (4 or 16) caps the gate
- * kernel's wavefronts per workgroup.  Process-wide; not meant to be changed
- * while work is in flight.
+ * Tuning knobs (no counterpart in the reference).  Process-wide; not meant to
+ * be changed while work is in flight.
+ *   "gemm_variant"    grouped-GEMM main-loop variant of the FFN entry points; -1 restores the default
+ *   "split_tail"      0 = off, 1 = default, n > 1 = for K of n*64 and more: the tiles of a launch's
+ *                     last, partly filled round are cut along K and reduced by a second kernel
+ *   "split_parts"     2..8 (default 8): most parts such a tile is cut into
+ *   "dgrad_transpose" 0/1: the backward's input-gradient GEMM runs on a transposed copy of the
+ *                     weight instead of reading the stored one
+ *   "gate_waves"      4 or 16: cap on the gate kernel's wavefronts per workgroup
  */
 int ccf_set_option(const char *name, int value);
 
