@@ -296,9 +296,48 @@ def test_ffn_special_cases():
     assert O.max_abs_err(pre.cpu(), ref) <= MAX_ABS
 
 
+def test_split_k_tail_at_its_default_threshold():
+    """K = 4096 is where the split of the last round switches on by itself: 36 M tiles x 16 N
+    tiles = 2.25 rounds of 256 workgroups, in both GEMMs, whole outputs against fp32."""
+    from ccfuser_amd import ops
+    g = torch.Generator().manual_seed(22)
+    R, d, f, E = 8192, 4096, 4096, 6
+    x = torch.randn(R, d, generator=g).half()
+    w1 = (torch.randn(E, f, d, generator=g) * 0.02).half()
+    b1 = (torch.randn(E, f, generator=g) * 0.05).half()
+    w2 = (torch.randn(E, d, f, generator=g) * 0.02).half()
+    b2 = (torch.randn(E, d, generator=g) * 0.05).half()
+    idx = torch.randint(0, E, (R,), generator=g)
+    r = ops.route(dev(idx), E, 1, -1)
+    off, pos = r["offsets"].cpu(), r["pos"].cpu()
+    _say(f"split-K tail by default R={R} d={d} f={f} E={E} counts={r['counts'].tolist()}")
+    out = {}
+    for mode in (1, 0):
+        ops.set_option("split_tail", mode)
+        try:
+            h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True)
+            y = torch.zeros(R, d, dtype=torch.float16, device="cuda")
+            ops.ffn2(h, r["dst_row"], r["offsets"], R, dev(w2), dev(b2), y)
+            out[mode] = (h.cpu(), y.cpu())
+        finally:
+            ops.set_option("split_tail", 1)
+    buf = x[pos].float()
+    h_ref = torch.zeros(R, f)
+    y_ref = torch.zeros(R, d)
+    hq = out[1][0].float()
+    for e in range(E):
+        lo, hi = int(off[e]), int(off[e + 1])
+        h_ref[lo:hi] = O.gelu_exact(buf[lo:hi] @ w1[e].float().t() + b1[e].float())
+        y_ref[pos[lo:hi]] = hq[lo:hi] @ w2[e].float().t() + b2[e].float()
+    assert O.max_abs_err(out[1][0], h_ref) <= MAX_ABS and O.mean_rel_err(out[1][0], h_ref) <= MEAN_REL
+    assert O.max_abs_err(out[1][1], y_ref) <= MAX_ABS and O.mean_rel_err(out[1][1], y_ref) <= MEAN_REL
+    # the split did run: bits differ from the unsplit kernels
+    assert not torch.equal(out[1][0], out[0][0]) and not torch.equal(out[1][1], out[0][1])
+
+
 def test_split_k_tail_all_epilogues():
     """The last, partly filled round of tiles is cut along K and reduced by a separate kernel.
-    By default that happens for K >= 8192 only; here it is forced on a small K so that the
+    By default that happens for K >= 4096 only; here it is forced on a small K so that the
     reduction's three epilogues (plain with row index and scale, GELU, GELU keeping the
     pre-activation) are compared with the oracle and with the unsplit kernels."""
     from ccfuser_amd import ops
