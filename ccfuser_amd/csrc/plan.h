@@ -69,13 +69,18 @@ struct PlanReq {
   int32_t *tail;    // split scratch (header and entries), or NULL
 };
 
-// Built by ONE workgroup of any size that is a multiple of 64 (all of its threads call this).
-__device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__ offsets, int E) {
+// Built by `nparts` workgroups of any size that is a multiple of 64 (all threads of each call
+// this with the workgroup's `part`).  Every workgroup repeats the small scans and takes a share
+// of the experts and of the idle entries; which entries stay idle is known in closed form, so
+// no entry is written by two workgroups and their order does not matter.
+__device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__ offsets, int E,
+                                  int part = 0, int nparts = 1) {
   const int BM = rq.BM, max_tiles = rq.max_tiles, max_rows = rq.max_rows, n_tiles_n = rq.n_tiles_n;
   const int spx = rq.spx, k_tiles = rq.k_tiles;
   int32_t *__restrict__ plan = rq.plan;
   int32_t *__restrict__ tail = rq.tail;
   __shared__ int s_full[8];        // split last round: slots of XCD x from s_full[x] on go to the tail list
+  __shared__ int s_used[8];        // tiles of XCD x
   __shared__ int s_parts;          // parts per tail tile, 0 = no split
   __shared__ int s_off[1025];
   __shared__ int s_long[1025];     // exclusive scan of long M tiles per expert
@@ -111,10 +116,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   // the launcher checks that the worst-case tile count, and with it every count below, fits an int
   const int wgs = static_cast<int>(launched_wgs(max_tiles, n_tiles_n));
   int4v *entry = reinterpret_cast<int4v *>(plan);
-  for (int b = threadIdx.x; b < wgs; b += blockDim.x) entry[b] = int4v{-1, 0, 0, 0};
   int4v *tent = reinterpret_cast<int4v *>(tail + 64);
-  if (tail)
-    for (int b = threadIdx.x; b < kTailMaxParts; b += blockDim.x) tent[b] = int4v{-1, 0, 0, 0};
   __syncthreads();
   // Hardware hands consecutive workgroup ids to the 8 XCDs in turn, so XCD x
   // runs ids x, x+8, ... in order.  Each class is cut into eight equal
@@ -140,6 +142,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       ns_x = ns_x < 0 ? 0 : (ns_x > per_short ? per_short : ns_x);
       const int used = nl_x + ns_x;
       const int full = spx > 0 ? used / spx * spx : used;
+      s_used[x] = used;
       s_full[x] = full;
       max_r = (used - full) > max_r ? (used - full) : max_r;
     }
@@ -153,10 +156,21 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     s_parts = S;
     if (!S)
       for (int x = 0; x < 8; ++x) s_full[x] = INT_MAX;
-    if (tail) { tail[0] = S ? 8 * max_r : 0; tail[1] = S; }
+    if (tail && part == 0) { tail[0] = S ? 8 * max_r : 0; tail[1] = S; }
   }
   __syncthreads();
   const int S = s_parts;
+  // idle entries: slot j of XCD x holds a tile while j < used_x (and j < full_x when the last
+  // round is split off); tail entry x + 8 * (i * S + s) while i < used_x - full_x
+  for (int b = threadIdx.x + part * blockDim.x; b < wgs; b += blockDim.x * nparts) {
+    const int x = b & 7, j = b >> 3;
+    if (j >= s_used[x] || j >= s_full[x]) entry[b] = int4v{-1, 0, 0, 0};
+  }
+  if (tail && part == 0)
+    for (int b = threadIdx.x; b < kTailMaxParts; b += blockDim.x) {
+      const int x = b & 7;
+      if (!S || (b >> 3) / S >= s_used[x] - s_full[x]) tent[b] = int4v{-1, 0, 0, 0};
+    }
   // slot j of XCD x: into the plan, or cut into S parts on the tail list
   auto place = [&](int j, int x, int4v v) {
     const int b = j * 8 + x;
@@ -169,7 +183,8 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     }
   };
   // one wavefront per expert
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63, nwave = (blockDim.x >> 6) * nparts;
+  const int wave = (threadIdx.x >> 6) * nparts + part;          // interleaved over the workgroups
   for (int e = wave; e < E; e += nwave) {
     const int lo = s_off[e];
     int cnt = s_off[e + 1] - lo;

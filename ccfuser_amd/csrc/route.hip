@@ -141,11 +141,12 @@ pos_kernel(const int64_t *__restrict__ idx, int n, int E, int nbits, int top_k, 
            const int32_t *__restrict__ chunk_base, const int32_t *__restrict__ offsets,
            int64_t *__restrict__ pos, int32_t *__restrict__ src_row,
            int32_t *__restrict__ dst_row, int32_t *__restrict__ inv_pos,
-           int64_t *__restrict__ idx_kept, int nchunk, PlanReq plan0, PlanReq plan1) {
+           int64_t *__restrict__ idx_kept, int nchunk, int plan_wgs, PlanReq plan0, PlanReq plan1) {
   // Workgroups past the chunks build the tile plans of the GEMMs that follow: the offsets are
   // final since the scan, and the plans then cost no launch of their own.
   if (static_cast<int>(blockIdx.x) >= nchunk) {
-    build_plan(blockIdx.x == static_cast<unsigned>(nchunk) ? plan0 : plan1, offsets, E);
+    const int r = static_cast<int>(blockIdx.x) - nchunk;        // plan_wgs workgroups per plan
+    build_plan(r < plan_wgs ? plan0 : plan1, offsets, E, r % plan_wgs, plan_wgs);
     return;
   }
   extern __shared__ int s_sub[];                 // [kSub][E]
@@ -290,9 +291,12 @@ int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capaci
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(pos_lds));
     if (e != hipSuccess) return fail(CCF_ERR_HIP, "route: LDS attribute: %s", hipGetErrorString(e));
   }
-  hipLaunchKernelGGL(pos_kernel, dim3(nchunk + n_plans), dim3(kThreads), pos_lds, stream,
+  // a plan is built by enough workgroups of kThreads that every expert has a wavefront (at most 8)
+  int plan_wgs = (E + kThreads / 64 - 1) / (kThreads / 64);
+  plan_wgs = plan_wgs > 8 ? 8 : plan_wgs;
+  hipLaunchKernelGGL(pos_kernel, dim3(nchunk + n_plans * plan_wgs), dim3(kThreads), pos_lds, stream,
                      gate_idx, n_flat, E, nbits, top_k, capacity, chunk_cnt, offsets, pos, src_row,
-                     dst_row, inv_pos, idx_kept, nchunk, n_plans > 0 ? plans[0] : none,
+                     dst_row, inv_pos, idx_kept, nchunk, plan_wgs, n_plans > 0 ? plans[0] : none,
                      n_plans > 1 ? plans[1] : none);
   return check_launch("pos_kernel");
 }
