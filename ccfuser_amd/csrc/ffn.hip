@@ -48,7 +48,7 @@ struct GroupedArgs {
   // of BK, at least four K tiles) and rows e*seg_rows .. of C.  NULL otherwise.
   const int32_t *k_seg;
   int lda, ldb, seg_rows;
-  // split-K tail (see tail_kernel): header {tiles, parts per tile}, entries, fp32 partial tiles
+  // split last round (layout in plan.h): header and part entries, fp32 partial tiles
   const int32_t *tail;
   float *partial;
 };

@@ -128,7 +128,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   const int total_short = s_short[E] * n_tiles_n;
   const int per_long = (total_long + 7) / 8;
   const int per_short = (total_short + 7) / 8;
-  // The split last round (see "split-K tail" below).  XCD x holds used_x tiles; with spx
+  // The split last round (run by grouped_gemm_tail_kernel and splitk_reduce_kernel in ffn.hip).  XCD x holds used_x tiles; with spx
   // persistent workgroups per XCD the last used_x % spx of them form a partly filled round.
   // When that round is at most half full on every XCD, its tiles leave the plan: tile i of
   // XCD x's last round, part s of S, becomes tail entry x + 8 * (i * S + s), the workgroup id
