@@ -116,7 +116,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   // the launcher checks that the worst-case tile count, and with it every count below, fits an int
   const int wgs = static_cast<int>(launched_wgs(max_tiles, n_tiles_n));
   int4v *entry = reinterpret_cast<int4v *>(plan);
-  int4v *tent = reinterpret_cast<int4v *>(tail + 64);
+  int4v *tent = tail ? reinterpret_cast<int4v *>(tail + 64) : nullptr;
   __syncthreads();
   // Hardware hands consecutive workgroup ids to the 8 XCDs in turn, so XCD x
   // runs ids x, x+8, ... in order.  Each class is cut into eight equal
@@ -128,8 +128,9 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   const int total_short = s_short[E] * n_tiles_n;
   const int per_long = (total_long + 7) / 8;
   const int per_short = (total_short + 7) / 8;
-  // The split last round (run by grouped_gemm_tail_kernel and splitk_reduce_kernel in ffn.hip).  XCD x holds used_x tiles; with spx
-  // persistent workgroups per XCD the last used_x % spx of them form a partly filled round.
+  // The split last round (run by grouped_gemm_tail_kernel and splitk_reduce_kernel in ffn.hip).
+  // XCD x holds used_x tiles; with spx persistent workgroups per XCD the last used_x % spx of
+  // them form a partly filled round.
   // When that round is at most half full on every XCD, its tiles leave the plan: tile i of
   // XCD x's last round, part s of S, becomes tail entry x + 8 * (i * S + s), the workgroup id
   // that the hardware places on the same XCD, so the patch of neighbouring tiles keeps sharing
