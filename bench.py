@@ -32,8 +32,8 @@ PEAK_HBM_GBS = 8000.0
 # sums over the three.  The summaries are in profiles/grouped_gemm_<workload>_hbm_traffic.txt.
 # Counters cannot be read from inside a normal run, so a workload without a profile reports null.
 MEASURED_TRAFFIC_KIB = {
-    ("c3_mixtral", "ffn1"): {"FETCH_SIZE": 931444.2, "WRITE_SIZE": 278531.2},
-    ("c3_mixtral", "ffn2"): {"FETCH_SIZE": 1045160.2, "WRITE_SIZE": 126981.0},
+    ("c3_mixtral", "ffn1"): {"FETCH_SIZE": 924215.3, "WRITE_SIZE": 278531.7},
+    ("c3_mixtral", "ffn2"): {"FETCH_SIZE": 1045322.1, "WRITE_SIZE": 126976.1},
 }
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 
