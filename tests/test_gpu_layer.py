@@ -295,3 +295,23 @@ def test_fused_call_equals_stage_by_stage_calls(workloads, name, rows, variant):
         assert torch.equal(fused, staged)
     finally:
         ops.set_option("gemm_variant", -1)
+
+
+@pytest.mark.parametrize("T,d,f,E,k", [(2048, 64, 128, 600, 2), (4096, 128, 64, 1024, 1), (300, 64, 64, 37, 4)])
+def test_fused_layer_with_many_experts(T, d, f, E, k):
+    """Most experts get a handful of rows or none; the routing launch builds the tile plans with
+    eight workgroups per plan and needs more than 64 KB of LDS past 512 experts."""
+    from ccfuser_amd import ops
+    g = torch.Generator().manual_seed(E)
+    r = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).half()
+    x, wg, bg = r(T, d), r(E, d, sc=0.3), r(E, sc=0.3)
+    w1, b1, w2, b2 = r(E, f, d, sc=0.1), r(E, f, sc=0.1), r(E, d, f, sc=0.1), r(E, d, sc=0.1)
+    _say(f"many experts T={T} d={d} f={f} E={E} k={k}")
+    args = [a.cuda() for a in (x, wg, bg, w1, b1, w2, b2)]
+    fused, rt = ops.moe_forward(*args, k, -1, return_routing=True)
+    ref = O.moe_layer_forward(x, wg, bg, w1, b1, w2, b2, k)
+    assert torch.equal(rt["idx"].cpu(), ref["idx"])
+    assert torch.equal(rt["offsets"].cpu().long(), ref["offsets"].long())
+    assert O.max_abs_err(fused.cpu(), ref["out"]) <= MAX_ABS
+    assert O.mean_rel_err(fused.cpu(), ref["out"]) <= MEAN_REL
+    assert torch.equal(fused, _staged_forward(ops, args, E, k, -1))
