@@ -314,9 +314,9 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
   if (tokens == 0) return CCF_OK;
   // Enough wavefronts to hide HBM latency: fewer tokens per wavefront when the batch is small.
   const int tt = tokens >= 32768 ? 4 : (tokens >= 8192 ? 2 : 1);
-  const int group = tot_expert < kGateEG ? tot_expert : kGateEG;
   const size_t esz = dtype == CCF_F16 ? 2 : 4;
-  const size_t w_bytes = static_cast<size_t>(group) * d_model * esz;
+  // the kernel always stages kGateEG weight rows (rows past the last expert repeat it)
+  const size_t w_bytes = static_cast<size_t>(kGateEG) * d_model * esz;
   const bool w_lds = w_bytes <= 65536;             // one expert group of weights fits next to the logits
   // Wavefronts per workgroup: 16 (one workgroup per CU stages the weights once for 16
   // wavefronts) when the weights sit in LDS, else 4 (two workgroups per CU).
