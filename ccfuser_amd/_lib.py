@@ -29,6 +29,8 @@ SIGNATURES = {
     "ccf_expert_count": (_i, [_p, _i, _p, _i, _p]),
     "ccf_assign_pos": (_i, [_p, _p, _i, _i, _p, _p, _sz, _p]),
     "ccf_route": (_i, [_p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "ccf_route_static": (_i, [_p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "ccf_route_static_max_entries": (_i, []),
     "ccf_plan_blocks": (_i, [_p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p]),
     "ccf_segments_to_rows": (_i, [_p, _p, _p, _i, _i, _i, _p, _p, _p, _p]),
     "ccf_local_scatter": (_i, [_p, _p, _p, _i, _i, _p]),

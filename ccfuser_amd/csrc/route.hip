@@ -18,6 +18,15 @@
 #include "ccf_common.h"
 #include "plan.h"
 
+#include <mutex>
+
+// Scratch of ccf_route_static: the per-chunk count table (the workspace of ccf_route) as a
+// device array that lives in the library image, so that the call allocates nothing.  Every
+// GPU the library runs on holds its own copy (1 MiB) until the process ends.  In host code the
+// name is only a handle for hipGetSymbolAddress: kernels are given the address it returns.
+constexpr int kStaticScratchInts = 1 << 18;
+static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
+
 namespace ccf {
 namespace {
 
@@ -444,6 +453,53 @@ extern "C" int ccf_route(const int64_t *gate_idx, int n_flat, int num_expert, in
   return route_impl(gate_idx, n_flat, num_expert, top_k, capacity, counts, offsets, nullptr, pos,
                     src_row, dst_row, inv_pos, idx_kept, workspace, workspace_bytes,
                     as_stream(stream));
+}
+
+namespace ccf {
+namespace {
+constexpr int kMaxDevices = 64;
+int32_t *g_scratch_ptr[kMaxDevices] = {nullptr};   // device address of `scratch`, per device
+std::mutex g_scratch_mu;
+
+// Device address of this device's copy of `scratch`, looked up once per device.
+int static_scratch(int32_t **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(CCF_ERR_HIP, "route_static: hipGetDevice: %s", hipGetErrorString(e));
+  CCF_REQUIRE(dev >= 0 && dev < kMaxDevices, CCF_ERR_UNSUPPORTED, "route_static: device %d outside 0..%d", dev,
+              kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(CCF_ERR_HIP, "route_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<int32_t *>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return CCF_OK;
+}
+}  // namespace
+}  // namespace ccf
+
+extern "C" int ccf_route_static_max_entries(void) { return kStaticScratchInts; }
+
+extern "C" int ccf_route_static(const int64_t *gate_idx, int n_flat, int num_expert, int top_k,
+                                int capacity, int32_t *counts, int32_t *offsets, int64_t *pos,
+                                int32_t *src_row, int32_t *dst_row, int32_t *inv_pos,
+                                int64_t *idx_kept, ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(counts && offsets, CCF_ERR_ARG, "route_static: null counts/offsets");
+  CCF_REQUIRE(n_flat >= 0 && num_expert > 0 && num_expert <= kMaxExpert, CCF_ERR_ARG, "route_static: bad size");
+  const long long nchunk = n_flat > 0 ? (static_cast<long long>(n_flat) + kChunk - 1) / kChunk : 1;
+  CCF_REQUIRE(nchunk * num_expert <= kStaticScratchInts, CCF_ERR_SHAPE,
+              "route_static: ceil(n_flat / %d) * num_expert = %lld exceeds the built-in scratch of %d entries; "
+              "use ccf_route with a workspace", kChunk, nchunk * num_expert, kStaticScratchInts);
+  int32_t *ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // hist_kernel writes every entry of the table before scan_kernel reads it: nothing to clear
+  return route_impl(gate_idx, n_flat, num_expert, top_k, capacity, counts, offsets, nullptr, pos, src_row,
+                    dst_row, inv_pos, idx_kept, ws, sizeof(int32_t) * kStaticScratchInts, as_stream(stream));
 }
 
 extern "C" int ccf_segments_to_rows(const int32_t *seg_start, const int32_t *seg_len,

@@ -127,6 +127,32 @@ def route(gate_idx: torch.Tensor, num_expert: int, top_k: int, capacity: int = -
     return out
 
 
+def route_static(gate_idx: torch.Tensor, num_expert: int, top_k: int, capacity: int = -1,
+                 out: Optional[Dict[str, torch.Tensor]] = None) -> Dict[str, torch.Tensor]:
+    """``route`` through the entry point that allocates nothing: its scratch is a device
+    array inside the library.  ``out`` takes preallocated result tensors (the keys ``route``
+    returns); without it they are allocated here, before the call.  Raises ``CcfError`` when
+    ``ceil(n / 1024) * num_expert`` exceeds the built-in scratch."""
+    _check(gate_idx, "gate_idx", dtype=torch.int64)
+    n = gate_idx.numel()
+    dev = gate_idx.device
+    if out is None:
+        out = {
+            "counts": torch.empty(num_expert, dtype=torch.int32, device=dev),
+            "offsets": torch.empty(num_expert + 1, dtype=torch.int32, device=dev),
+            "pos": torch.empty(n, dtype=torch.int64, device=dev),
+            "src_row": torch.empty(n, dtype=torch.int32, device=dev),
+            "dst_row": torch.empty(n, dtype=torch.int32, device=dev),
+            "inv_pos": torch.empty(n, dtype=torch.int32, device=dev),
+            "idx_kept": torch.empty(n, dtype=torch.int64, device=dev),
+        }
+    with torch.cuda.device(dev):
+        _lib.call("ccf_route_static", _ptr(gate_idx), n, int(num_expert), int(top_k), int(capacity),
+                  _ptr(out["counts"]), _ptr(out["offsets"]), _ptr(out["pos"]), _ptr(out["src_row"]),
+                  _ptr(out["dst_row"]), _ptr(out["inv_pos"]), _ptr(out["idx_kept"]), _stream(gate_idx))
+    return out
+
+
 def plan_blocks(counts: torch.Tensor, max_rows: int, block_size: int = 64, rank: int = 0) -> Dict[str, torch.Tensor]:
     """The reference's block arrays (transformer.py:242-250) from per-expert counts,
     on the device and without a host synchronisation.

@@ -133,6 +133,26 @@ int ccf_route(const int64_t *gate_idx, int n_flat, int num_expert, int top_k,
               ccf_stream_t stream);
 
 /*
+ * ccf_route without a workspace and without any allocation: the per-chunk count
+ * table that ccf_route keeps in its workspace lives in a 1 MiB device array
+ * inside the library image instead.  It has no counterpart in the reference and is for
+ * callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  Same arguments and
+ * results as ccf_route.  Limit: ceil(n_flat / 1024) * num_expert must not exceed
+ * ccf_route_static_max_entries() (262144), e.g. 1M indices for 256 experts;
+ * larger inputs return CCF_ERR_SHAPE.  All calls on one GPU share that GPU's
+ * array: calls that overlap in time on one GPU (different streams or threads)
+ * race and must be serialised by the caller.
+ */
+int ccf_route_static(const int64_t *gate_idx, int n_flat, int num_expert, int top_k,
+                     int capacity, int32_t *counts, int32_t *offsets, int64_t *pos,
+                     int32_t *src_row, int32_t *dst_row, int32_t *inv_pos,
+                     int64_t *idx_kept, ccf_stream_t stream);
+
+/* Entries of the built-in scratch of ccf_route_static (no counterpart in the reference). */
+int ccf_route_static_max_entries(void);
+
+/*
  * Block plan in the reference's wire format, built on the device from the
  * per-expert counts: what AsyncExpertAssignment.divide_into_block computes in
  * Python loops and ships with seven blocking copies
