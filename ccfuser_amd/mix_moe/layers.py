@@ -20,13 +20,14 @@ def _local_scatter(inp, pos):
 
 
 def _local_gather(inp, pos, out_batch_size, maybe_overlap=True):
-    """Rows back to their slots (reference layers.py:24-31).  With
-    ``maybe_overlap`` the rows are accumulated (several may share a slot),
-    otherwise each slot is written once by the HIP row kernel."""
+    """Rows back to their slots (reference layers.py:24-31) by the HIP row kernel; every
+    slot is written at most once.  The reference's accumulating form
+    (``maybe_overlap=True``, an ``index_add_``) is never used on this path (its one call,
+    layers.py:453, passes ``False``) and has no kernel here: asking for it raises instead
+    of falling back to a torch op."""
     if maybe_overlap:
-        buf = torch.zeros(out_batch_size, inp.shape[-1], dtype=inp.dtype, device=inp.device)
-        buf.index_add_(0, pos, inp)
-        return buf
+        raise NotImplementedError("_local_gather(maybe_overlap=True) has no HIP kernel: rows that share a slot "
+                                  "are summed by ops.combine; pass maybe_overlap=False for a pure row move")
     return ops.local_gather(inp.contiguous(), pos.to(torch.int32), out_batch_size)
 
 
