@@ -104,7 +104,8 @@ SegWs carve_seg(void *ws, int total_rows, int d, int f, int E) {
 }
 
 // Optional per-stage timing: events recorded on the layer's stream before the
-// gate and after each of the five stages of the next ccf_moe_forward calls.
+// gate and after each of the five stages of the next ccf_moe_forward calls
+// (ccf_moe_ffn_segments records the same six; its gate and combine stages are empty).
 thread_local hipEvent_t g_stage_events[6];
 thread_local int g_stage_event_count = 0;
 
@@ -170,22 +171,23 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
   // the tile plans of both GEMMs are built by two more workgroups of the routing stage's last
   // launch (they need the offsets only), which saves the GEMMs a small launch each
   PlanReq plans[2];
-  const bool planned = forward_plan_request(1, n, num_expert, d_model, d_ffn, w.ffn_ws, &plans[0]) &&
-                       forward_plan_request(2, n, num_expert, d_model, d_ffn, w.ffn_ws, &plans[1]);
+  const GemmOptions opt = forward_options();        // one snapshot for the plans and the GEMMs that consume them
+  const bool planned = forward_plan_request(1, n, num_expert, d_model, d_ffn, w.ffn_ws, opt, &plans[0]) &&
+                       forward_plan_request(2, n, num_expert, d_model, d_ffn, w.ffn_ws, opt, &plans[1]);
   if ((rc = route_with_plans(w.idx, n, num_expert, top_k, capacity, w.counts, w.offsets, w.pos, w.src_row,
                              w.dst_row, w.inv_pos, w.idx_kept, w.route_ws, w.route_bytes, st, plans,
                              planned ? 2 : 0)))
     return rc;
   mark_stage(2, st);
   if ((rc = ffn1_forward(x, w.src_row, nullptr, w.offsets, n, num_expert, d_model, d_ffn, w1, b1, 1, w.h,
-                         w.ffn_ws, w.ffn_bytes, st, planned)))
+                         w.ffn_ws, w.ffn_bytes, st, planned ? &opt : nullptr)))
     return rc;
   mark_stage(3, st);
   // top-1 without a capacity limit: every token has one slot, its score is exactly 1 (the softmax of
   // one logit) and its flat row is its token row, so FFN2 writes the layer output itself
   const bool direct = top_k == 1 && capacity < 0;
   if ((rc = ffn2_forward(w.h, nullptr, w.dst_row, w.offsets, n, num_expert, d_model, d_ffn, w2, b2,
-                         nullptr, direct ? out : w.y_flat, w.ffn_ws, w.ffn_bytes, st, planned)))
+                         nullptr, direct ? out : w.y_flat, w.ffn_ws, w.ffn_bytes, st, planned ? &opt : nullptr)))
     return rc;
   mark_stage(4, st);
   if (!direct) {
@@ -226,13 +228,21 @@ extern "C" int ccf_moe_ffn_segments(const void *x, const int32_t *seg_start, con
               "moe_ffn_segments: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   if (total_rows == 0 || n_seg == 0) return CCF_OK;
   SegWs w = carve_seg(workspace, total_rows, d_model, d_ffn, num_expert);
+  hipStream_t st = as_stream(stream);
   int rc;
+  mark_stage(0, st);
+  mark_stage(1, st);                                  // no gate in this call
   if ((rc = ccf_segments_to_rows(seg_start, seg_len, seg_expert, n_seg, num_expert, total_rows,
                                  w.counts, w.offsets, w.rows, stream)))
     return rc;
+  mark_stage(2, st);
   if ((rc = ccf_ffn1_forward(x, w.rows, nullptr, w.offsets, total_rows, num_expert, d_model, d_ffn, w1, b1, 1,
                              w.h, w.ffn_ws, w.ffn_bytes, stream)))
     return rc;
-  return ccf_ffn2_forward(w.h, nullptr, w.rows, w.offsets, total_rows, num_expert, d_model, d_ffn, w2, b2,
-                          nullptr, y, w.ffn_ws, w.ffn_bytes, stream);
+  mark_stage(3, st);
+  rc = ccf_ffn2_forward(w.h, nullptr, w.rows, w.offsets, total_rows, num_expert, d_model, d_ffn, w2, b2,
+                        nullptr, y, w.ffn_ws, w.ffn_bytes, stream);
+  mark_stage(4, st);
+  mark_stage(5, st);                                  // no combine either
+  return rc;
 }

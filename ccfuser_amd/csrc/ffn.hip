@@ -677,6 +677,11 @@ constexpr int kSplitTailMinKT = 64;
 int g_split_tail_min_kt = kSplitTailMinKT;
 int g_split_max_parts = 8;
 
+// The tuning knobs a grouped GEMM's plan and launches depend on, read once per call: the plan
+// and the kernels that consume it must agree even if another thread calls ccf_set_option
+// between the routing stage (which builds the plans of the layer's forward call) and the GEMMs.
+GemmOptions current_options() { return GemmOptions{g_variant, g_split_tail, g_split_tail_min_kt, g_split_max_parts}; }
+
 struct Launch {
   int bm, bn, threads;
   void (*plain)(GroupedArgs);
@@ -751,7 +756,8 @@ struct GemmSetup {
   PlanReq req;
 };
 
-GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void *workspace, int region) {
+GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void *workspace, int region,
+                     const GemmOptions &opt) {
   GemmSetup g;
   char *ws = static_cast<char *>(workspace);
   g.partial = reinterpret_cast<float *>(ws + kTailHead);
@@ -763,7 +769,7 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
     g.plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.tail) + kTailHead);
   }
   const bool gelu = epi != kEpiPlain;
-  g.v = &kVariants[b_kn ? kKnVariant : (epi >= kEpiGeluKeep ? kTrainVariant : g_variant)];
+  g.v = &kVariants[b_kn ? kKnVariant : (epi >= kEpiGeluKeep ? kTrainVariant : opt.variant)];
   const Launch &v = *g.v;
   // which of the entry's two kernels: the K-N and training entries hold the GELU-gradient form in the second slot
   g.second = b_kn ? epi == kEpiGeluGrad : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu);
@@ -773,9 +779,9 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
   g.grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
   // the last, partly filled round is cut along K and spread over all workgroups (forward forms;
   // worth its two small launches only where a tile is long: K of 4096 and more)
-  g.split = g_split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && g.grid >= 8 && g.grid <= g.wgs &&
-            g.grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= g_split_tail_min_kt;
-  g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, g_split_max_parts, g.plan,
+  g.split = opt.split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && g.grid >= 8 && g.grid <= g.wgs &&
+            g.grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= opt.split_tail_min_kt;
+  g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, opt.split_max_parts, g.plan,
                   g.split ? g.tail : nullptr};
   return g;
 }
@@ -786,7 +792,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
                  int N, int K, const half_t *B, const half_t *bias, int epi, half_t *C,
                  const int32_t *c_rows, const half_t *row_scale, void *workspace, hipStream_t stream,
                  const char *what, bool b_kn = false, half_t *C2 = nullptr, int region = 0,
-                 bool plan_ready = false) {
+                 bool plan_ready = false, const GemmOptions *opt = nullptr) {
   CCF_REQUIRE(A && offsets && B && C && workspace, CCF_ERR_ARG, "%s: null pointer", what);
   const bool gelu = epi != kEpiPlain;
   CCF_REQUIRE(epi >= kEpiPlain && epi <= kEpiGeluGrad && (epi < kEpiGeluKeep || (C2 && aligned16(C2))), CCF_ERR_ARG,
@@ -803,7 +809,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
               "%s: operands must be 16-byte aligned", what);
   CCF_REQUIRE(!(gelu && row_scale), CCF_ERR_ARG, "%s: the GELU epilogue takes no row scale", what);
   if (max_rows == 0) return CCF_OK;
-  const GemmSetup gs = setup_gemm(max_rows, E, N, K, epi, b_kn, workspace, region);
+  const GemmSetup gs = setup_gemm(max_rows, E, N, K, epi, b_kn, workspace, region, opt ? *opt : current_options());
   const Launch &v = *gs.v;
   const bool second = gs.second, split = gs.split;
   const int grid = gs.grid;
@@ -1040,11 +1046,14 @@ namespace ccf {
 // Plan requests of the layer's two forward GEMMs (which = 1: FFN1 with GELU, 2: FFN2), for a
 // caller that builds the plans itself (the routing stage does) and then passes plan_ready.
 // False when the sizes are not ones the GEMM accepts: the caller then leaves the plan to it.
-bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, PlanReq *out) {
+GemmOptions forward_options() { return current_options(); }
+
+bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, const GemmOptions &opt,
+                          PlanReq *out) {
   if (!workspace || max_rows <= 0 || E <= 0 || E > 1024 || d <= 0 || f <= 0 || d % 64 || f % 64) return false;
   const int N = which == 1 ? f : d, K = which == 1 ? d : f;
   const GemmSetup gs = setup_gemm(max_rows, E, N, K, which == 1 ? kEpiGelu : kEpiPlain, false, workspace,
-                                  which == 1 ? 0 : 1);
+                                  which == 1 ? 0 : 1, opt);
   if (gs.wgs >= (1ll << 31)) return false;
   *out = gs.req;
   return true;
@@ -1053,27 +1062,29 @@ bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *wo
 int ffn1_forward(const void *x, const int32_t *src_row, const int32_t *dst_row, const int32_t *offsets,
                  int max_rows, int num_expert, int d_model, int d_ffn, const void *w1, const void *b1,
                  int apply_gelu, void *h, void *workspace, size_t workspace_bytes, hipStream_t stream,
-                 bool plan_ready) {
+                 const GemmOptions *planned) {
+  const bool plan_ready = planned != nullptr;
   const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
   CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
               "ffn1: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   return grouped_gemm(static_cast<const half_t *>(x), src_row, offsets, max_rows, num_expert, d_ffn,
                       d_model, static_cast<const half_t *>(w1), static_cast<const half_t *>(b1),
                       apply_gelu != 0 ? kEpiGelu : kEpiPlain, static_cast<half_t *>(h), dst_row, nullptr,
-                      workspace, stream, "ffn1", false, nullptr, 0, plan_ready && apply_gelu != 0);
+                      workspace, stream, "ffn1", false, nullptr, 0, plan_ready && apply_gelu != 0, planned);
 }
 
 int ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row, const int32_t *offsets,
                  int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
                  const void *row_scale, void *y, void *workspace, size_t workspace_bytes,
-                 hipStream_t stream, bool plan_ready) {
+                 hipStream_t stream, const GemmOptions *planned) {
+  const bool plan_ready = planned != nullptr;
   const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
   CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
               "ffn2: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   return grouped_gemm(static_cast<const half_t *>(h), src_row, offsets, max_rows, num_expert, d_model,
                       d_ffn, static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), kEpiPlain,
                       static_cast<half_t *>(y), dst_row, static_cast<const half_t *>(row_scale),
-                      workspace, stream, "ffn2", false, nullptr, 1, plan_ready);
+                      workspace, stream, "ffn2", false, nullptr, 1, plan_ready, planned);
 }
 
 }  // namespace ccf
@@ -1083,7 +1094,7 @@ extern "C" int ccf_ffn1_forward(const void *x, const int32_t *src_row, const int
                                 int d_ffn, const void *w1, const void *b1, int apply_gelu, void *h,
                                 void *workspace, size_t workspace_bytes, ccf_stream_t stream) {
   return ccf::ffn1_forward(x, src_row, dst_row, offsets, max_rows, num_expert, d_model, d_ffn, w1, b1,
-                           apply_gelu, h, workspace, workspace_bytes, ccf::as_stream(stream), false);
+                           apply_gelu, h, workspace, workspace_bytes, ccf::as_stream(stream), nullptr);
 }
 
 extern "C" int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row,
@@ -1092,7 +1103,7 @@ extern "C" int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int
                                 void *y, void *workspace, size_t workspace_bytes,
                                 ccf_stream_t stream) {
   return ccf::ffn2_forward(h, src_row, dst_row, offsets, max_rows, num_expert, d_model, d_ffn, w2, b2,
-                           row_scale, y, workspace, workspace_bytes, ccf::as_stream(stream), false);
+                           row_scale, y, workspace, workspace_bytes, ccf::as_stream(stream), nullptr);
 }
 
 extern "C" size_t ccf_ffn_backward_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn) {

@@ -227,15 +227,21 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
 
 // ---- the layer's forward call: plans built by the routing stage ------------------
 // ffn.hip
-bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, PlanReq *out);
+// Snapshot of the tuning knobs (ccf_set_option) that a grouped GEMM's plan and launches depend on.
+struct GemmOptions {
+  int variant, split_tail, split_tail_min_kt, split_max_parts;
+};
+GemmOptions forward_options();
+bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, const GemmOptions &opt,
+                          PlanReq *out);
 int ffn1_forward(const void *x, const int32_t *src_row, const int32_t *dst_row, const int32_t *offsets,
                  int max_rows, int num_expert, int d_model, int d_ffn, const void *w1, const void *b1,
                  int apply_gelu, void *h, void *workspace, size_t workspace_bytes, hipStream_t stream,
-                 bool plan_ready);
+                 const GemmOptions *planned);   // planned: the options the plan in the workspace was built under, or NULL
 int ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row, const int32_t *offsets,
                  int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
                  const void *row_scale, void *y, void *workspace, size_t workspace_bytes,
-                 hipStream_t stream, bool plan_ready);
+                 hipStream_t stream, const GemmOptions *planned);
 // route.hip: ccf_route(), whose last launch also builds n_plans (0..2) tile plans from the offsets
 int route_with_plans(const int64_t *gate_idx, int n_flat, int num_expert, int top_k, int capacity,
                      int32_t *counts, int32_t *offsets, int64_t *pos, int32_t *src_row, int32_t *dst_row,

@@ -280,7 +280,9 @@ int ccf_moe_forward(const void *x, const void *wg, const void *bg,
  * Profiling hook (no counterpart in the reference).  Gives up to six hipEvent_t
  * handles; every later ccf_moe_forward on this thread records them on its
  * stream: [0] before the gate, then after the gate, the count/scan/pos, FFN1,
- * FFN2 and the combine.  count = 0 switches the recording off.
+ * FFN2 and the combine.  ccf_moe_ffn_segments records the same six, with the
+ * regrouping of the segments as its count/scan/pos stage and nothing between
+ * [0] and [1] or [4] and [5].  count = 0 switches the recording off.
  */
 int ccf_moe_forward_set_events(void *const *events, int count);
 
