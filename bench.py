@@ -24,25 +24,70 @@ sys.path.insert(0, ROOT)
 PEAK_FP16_TFLOPS = 2500.0          # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 
-# Bytes moved between L2 and the memory fabric per grouped GEMM, from two `rocprofv3 --pmc`
+# Bytes moved between L2 and the memory fabric per grouped GEMM come from two `rocprofv3 --pmc`
 # runs of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the
-# counter reads for a plain 256 MiB device copy in the same run (FETCH_SIZE reads half the
-# copied bytes: factor 2.0; WRITE_SIZE factor 1.0).  A grouped GEMM is three launches (the
-# persistent kernel, the parts of the split last round, their reduction): the figures are the
-# sums over the three.  The summaries are in profiles/grouped_gemm_<workload>_hbm_traffic.txt.
-# Counters cannot be read from inside a normal run, so a workload without a profile reports null.
-MEASURED_TRAFFIC_KIB = {
-    ("c3_mixtral", "ffn1"): {"FETCH_SIZE": 924215.3, "WRITE_SIZE": 278531.7},
-    ("c3_mixtral", "ffn2"): {"FETCH_SIZE": 1045322.1, "WRITE_SIZE": 126976.1},
-}
-FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+# counter reads for a plain 256 MiB device copy in the same run.  Counters cannot be read from
+# inside a normal run, so the figures are parsed from the committed summary
+# profiles/grouped_gemm_<workload>_hbm_traffic.txt (its last line, "TRAFFIC ..."), which also
+# records a hash of the kernel sources it was measured on: when the sources have changed since,
+# the line says so ("traffic_stale": true).  A workload without a summary reports null.
+KERNEL_SOURCES = ("ccfuser_amd/csrc/ffn.hip", "ccfuser_amd/csrc/gemm_tile.h", "ccfuser_amd/csrc/plan.h")
+
+
+def kernel_sources_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def measured_traffic(workload, stage):
-    m = MEASURED_TRAFFIC_KIB.get((workload, stage))
-    if m is None:
-        return None
-    return (m["FETCH_SIZE"] * FETCH_SCALE + m["WRITE_SIZE"] * WRITE_SCALE) * 1024.0
+    """(bytes per launch, stale flag, file) from the profile summary, or (None, None, None)."""
+    rel = f"profiles/grouped_gemm_{workload}_hbm_traffic.txt"
+    path = os.path.join(ROOT, rel)
+    if not os.path.exists(path):
+        return None, None, None
+    rec = None
+    for ln in open(path):
+        if ln.startswith("TRAFFIC "):
+            rec = dict(kv.split("=", 1) for kv in ln.split()[1:])
+    if rec is None or f"{stage}_fetch_kib" not in rec:
+        return None, None, rel
+    nbytes = (float(rec[f"{stage}_fetch_kib"]) * float(rec["fetch_scale"]) +
+              float(rec[f"{stage}_write_kib"]) * float(rec["write_scale"])) * 1024.0
+    return nbytes, rec.get("sources") != kernel_sources_hash(), rel
+
+
+def dense_hgemm_ceiling(rows, d, f, steps=30, warmup=15):
+    """What the vendor's dense fp16 GEMM (hipBLASLt through torch.matmul) sustains on this box,
+    in this process, on the two GEMM shapes of the workload with random operands: rows x d x f
+    (FFN1's) and rows x f x d (FFN2's), weights stored [N, K] as the layer stores them.  Reported
+    beside the nominal peak: a measured ceiling for a dense, unragged GEMM of the same size."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(7)
+    out = {}
+    for name, (K, N) in (("ffn1_shape", (d, f)), ("ffn2_shape", (f, d))):
+        a = torch.randn(rows, K, device="cuda", generator=g).half()
+        w = (torch.randn(N, K, device="cuda", generator=g) * 0.02).half()
+        for _ in range(warmup):
+            torch.matmul(a, w.t())
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            torch.matmul(a, w.t())
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        tf = 2.0 * rows * K * N / (ms * 1e-3) / 1e12
+        out[name] = {"m": rows, "n": N, "k": K, "ms": ms, "tflops": tf, "frac_of_peak": tf / PEAK_FP16_TFLOPS}
+        del a, w
+    mean = sum(v["tflops"] for v in out.values()) / 2
+    out["tflops"] = mean
+    out["frac_of_peak"] = mean / PEAK_FP16_TFLOPS
+    out["what"] = f"torch.matmul (hipBLASLt) fp16, random operands, {warmup} warm-up + {steps} timed calls per shape"
+    return out
 
 
 class HipEvents:
@@ -80,18 +125,24 @@ def cpu_baseline(wl, max_seconds=30.0):
     import torch
     from oracle import moe_oracle as O
     t = wl.tensors
-    names = ("x", "wg", "bg", "w1", "b1", "w2", "b2")
-    args = [t[n].float() for n in names]
+    if "seg_start" in t:
+        # the expert-parallel share has no gate: the expert FFN over the inbound segments
+        f32 = [t[n].float() for n in ("x", "w1", "b1", "w2", "b2")]
+        segs = [t[n] for n in ("seg_start", "seg_len", "seg_expert")]
+        run = lambda: O.ffn_segments(f32[0], *segs, *f32[1:])
+    else:
+        args = [t[n].float() for n in ("x", "wg", "bg", "w1", "b1", "w2", "b2")]
+        run = lambda: O.reference_layer_torch(*args, wl.top_k, capacity=wl.capacity)
     threads = torch.get_num_threads()
     with torch.no_grad():
         t0 = time.perf_counter()
-        O.reference_layer_torch(*args, wl.top_k, capacity=wl.capacity)
+        run()
         first = time.perf_counter() - t0
         times = []
         spent = first
         while len(times) < 3 and (not times or spent + times[-1] < max_seconds):
             t0 = time.perf_counter()
-            O.reference_layer_torch(*args, wl.top_k, capacity=wl.capacity)
+            run()
             times.append(time.perf_counter() - t0)
             spent += times[-1]
     med = sorted(times)[len(times) // 2]
@@ -196,6 +247,8 @@ def main():
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="ccf_set_option before the run (tuning knobs), may repeat")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dense-ceiling", action="store_true",
+                    help="skip the vendor dense-GEMM measurement on the workload's GEMM shapes")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (a known HBM traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -237,21 +290,18 @@ def main():
     if a.backward:
         return bench_backward(a, wl, ops)
 
-    if a.workload == "c4_ep_share":
+    segments = a.workload == "c4_ep_share"
+    if segments:
         names = ("x", "seg_start", "seg_len", "seg_expert", "w1", "b1", "w2", "b2")
         g = [t[n].cuda() for n in names]
         y = torch.zeros(T, d, dtype=torch.float16, device="cuda")
-        run = lambda: ops.moe_ffn_segments(*g, y=y)
-        routed = T
-        stage_ms = None
-        for _ in range(W):
-            run()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(K):
-            run()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
+        n_seg = g[1].numel()
+        ws = torch.empty(lib.ccf_segments_workspace_bytes(T, n_seg, E, d, f), dtype=torch.uint8, device="cuda")
+        x_, s0, s1, s2, w1_, b1_, w2_, b2_ = [v.data_ptr() for v in g]
+
+        def run():
+            _lib.call("ccf_moe_ffn_segments", x_, s0, s1, s2, n_seg, T, d, f, E, w1_, b1_, w2_, b2_,
+                      y.data_ptr(), ws.data_ptr(), ws.numel(), stream)
     else:
         names = ("x", "wg", "bg", "w1", "b1", "w2", "b2")
         g = [t[n].cuda() for n in names]
@@ -264,36 +314,36 @@ def main():
             _lib.call("ccf_moe_forward", *ptrs, T, d, f, E, k, wl.capacity, out.data_ptr(), None,
                       None, None, None, offsets.data_ptr(), ws.data_ptr(), ws.numel(), stream)
 
-        events = [[ev.create() for _ in range(6)] for _ in range(K)]
-        arrs = [(ctypes.c_void_p * 6)(*row) for row in events]
-        for _ in range(W):
-            run()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
+    events = [[ev.create() for _ in range(6)] for _ in range(K)]
+    arrs = [(ctypes.c_void_p * 6)(*row) for row in events]
+    for _ in range(W):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        if a.stage_events == "timed":
+            _lib.call("ccf_moe_forward_set_events", arrs[i], 6)
+        run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    if a.stage_events == "after":
+        # the same K steps once more, now with an event recorded between the stages
+        t1 = time.perf_counter()
         for i in range(K):
-            if a.stage_events == "timed":
-                _lib.call("ccf_moe_forward_set_events", arrs[i], 6)
+            _lib.call("ccf_moe_forward_set_events", arrs[i], 6)
             run()
         torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        if a.stage_events == "after":
-            # the same K steps once more, now with an event recorded between the stages
-            t1 = time.perf_counter()
-            for i in range(K):
-                _lib.call("ccf_moe_forward_set_events", arrs[i], 6)
-                run()
-            torch.cuda.synchronize()
-            wall_events = time.perf_counter() - t1
-        else:
-            wall_events = wall
-        _lib.call("ccf_moe_forward_set_events", None, 0)
-        routed = int(offsets[-1].item())
-        stage_names = ("gate", "route", "ffn1", "ffn2", "combine")
-        stage_ms = {n: sum(ev.elapsed_ms(events[i][s], events[i][s + 1]) for i in range(K)) / K
-                    for s, n in enumerate(stage_names)}
-        for row in events:
-            for e in row:
-                ev.destroy(e)
+        wall_events = time.perf_counter() - t1
+    else:
+        wall_events = wall
+    _lib.call("ccf_moe_forward_set_events", None, 0)
+    routed = T if segments else int(offsets[-1].item())
+    stage_names = ("gate", "route", "ffn1", "ffn2", "combine")
+    stage_ms = {n: sum(ev.elapsed_ms(events[i][s], events[i][s + 1]) for i in range(K)) / K
+                for s, n in enumerate(stage_names)}
+    for row in events:
+        for e in row:
+            ev.destroy(e)
 
     if a.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
@@ -314,19 +364,24 @@ def main():
                    "capacity": wl.capacity, "seed": wl.seed},
         "gemm_tflops": tflops, "frac_fp16_mfma_peak": tflops / PEAK_FP16_TFLOPS,
     }
-    if stage_ms is not None:
-        line["stages_ms"] = stage_ms
-        line["ms_per_step_with_stage_events"] = wall_events / K * 1e3
-        dom = "ffn1" if stage_ms["ffn1"] >= stage_ms["ffn2"] else "ffn2"
-        ach = (flops / 2) / (stage_ms[dom] * 1e-3) / 1e12
-        line["roofline"] = {"kernel": f"grouped GEMM of {dom}: grouped_gemm_persistent_kernel + "
-                                      "grouped_gemm_tail_kernel + splitk_reduce_kernel", "bound": "mfma",
-                            "achieved": ach, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                            "frac": ach / PEAK_FP16_TFLOPS,
-                            "traffic": measured_traffic(wl.name, dom), "traffic_unit": "bytes/launch",
-                            "flop_per_launch": flops / 2, "avg_launch_ms": stage_ms[dom]}
+    line["stages_ms"] = stage_ms
+    line["ms_per_step_with_stage_events"] = wall_events / K * 1e3
+    dom = "ffn1" if stage_ms["ffn1"] >= stage_ms["ffn2"] else "ffn2"
+    ach = (flops / 2) / (stage_ms[dom] * 1e-3) / 1e12
+    traffic, stale, traffic_file = measured_traffic(wl.name, dom)
+    line["roofline"] = {"kernel": f"grouped GEMM of {dom} (all launches between the stage's two events)",
+                        "bound": "mfma", "achieved": ach, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                        "frac": ach / PEAK_FP16_TFLOPS,
+                        "traffic": traffic, "traffic_unit": "bytes/launch", "traffic_source": traffic_file,
+                        "traffic_stale": stale,
+                        "flop_per_launch": flops / 2, "avg_launch_ms": stage_ms[dom]}
+    if not segments:
         hbm_bytes = T * d * 2 + E * d * 2 + T * k * 10
         line["gate_gbs"] = hbm_bytes / (stage_ms["gate"] * 1e-3) / 1e9
+    if not a.no_dense_ceiling:
+        ceil = dense_hgemm_ceiling(routed, d, f)
+        line["dense_hgemm_ceiling"] = ceil
+        line["roofline"]["frac_of_dense_hgemm_ceiling"] = ach / ceil[f"{dom}_shape"]["tflops"]
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(line))

@@ -148,6 +148,73 @@ def test_extension_class_with_reference_block_arrays(workloads):
     assert O.max_abs_err(y2.cpu(), y_ref) <= MAX_ABS
 
 
+def test_extension_class_backward_with_reference_block_arrays(workloads):
+    """mix_moe_cuda.MixMOE.first_gemm_backward / second_gemm_backward called the way
+    MixMOELinear1/2.backward call them (linear.py:103, 162; pybind.cpp:56-57): stored
+    [E, out, in] weights, gradients and saved inputs in the padded 64-row block layout,
+    the block arrays and the CSR arrays.  Against the oracle's closed-form backward."""
+    from ccfuser_amd import mix_moe_hip
+    from ccfuser_amd.mix_moe.transformer import plan_blocks
+    wl = workloads("c2_gshard", 512)
+    t = wl.tensors
+    E, d, f, k = wl.num_expert, wl.d_model, wl.d_ffn, wl.top_k
+    idx, score, _ = O.naive_gate(t["x"], t["wg"], t["bg"], k)
+    pos_ref, off_ref = O.assign_pos(idx, E)
+    R, n_flat = pos_ref.numel(), wl.tokens * k
+    plan = plan_blocks(O.expert_count(idx, E).numpy())
+    dev_i32 = lambda l: torch.tensor(l, dtype=torch.int32, device="cuda")
+    blocks = (dev_i32(plan["expert_ids"]), dev_i32(plan["ranks"]), dev_i32(plan["lens"]),
+              dev_i32(plan["start_addrs"]), plan["total_block_num"], plan["remote_block_num"])
+    csr = (dev_i32(plan["expert_block_ids"]), dev_i32(plan["expert_block_id_idxs"]))
+    nb, bs = plan["total_block_num"], 64
+    # expert-order row of every padded row (-1 = padding of a short block)
+    sorted_of_padded = torch.full((nb * bs,), -1, dtype=torch.long)
+    for b in range(nb):
+        n, st = plan["lens"][b], plan["start_addrs"][b]
+        sorted_of_padded[b * bs: b * bs + n] = torch.arange(st, st + n)
+    valid = sorted_of_padded >= 0
+
+    def to_padded(rows_sorted):
+        out = torch.zeros(nb * bs, rows_sorted.shape[1], dtype=rows_sorted.dtype)
+        out[valid] = rows_sorted[sorted_of_padded[valid]]
+        return out
+
+    g = torch.Generator().manual_seed(5)
+    m = mix_moe_hip.MixMOE(1, wl.tokens, E, k, d, f, bs)
+    x, pos = t["x"].cuda(), pos_ref.cuda()
+    w1, w2 = t["w1"].cuda(), t["w2"].cuda()                      # stored layout, as linear.py:103, 162 pass it
+    merged, _ = m.first_gemm_forward(x, pos, *blocks, w1.transpose(-2, -1).contiguous(), t["b1"].cuda())
+    # ---- first_gemm_backward
+    g_h = torch.randn(R, f, generator=g).half()
+    _say(f"first_gemm_backward blocks={nb} rows={R}")
+    grad_in, g_w1, g_b1 = m.first_gemm_backward(to_padded(g_h).cuda(), w1, t["b1"].cuda(), merged, *csr, pos,
+                                                *blocks)
+    ref_in, ref_w1, ref_b1 = O.ffn1_backward(g_h, t["x"], pos_ref, k, off_ref, t["w1"])
+    assert tuple(grad_in.shape) == (n_flat // k, d)
+    for got, ref, what in ((grad_in, ref_in, "grad_in"), (g_w1, ref_w1, "grad_w1"), (g_b1, ref_b1, "grad_b1")):
+        got, ref = got.float().cpu(), ref.float()
+        assert O.max_abs_err(got, ref) <= MAX_ABS * max(1.0, float(ref.abs().max())), what
+        assert O.mean_rel_err(got, ref) <= MEAN_REL, what
+    # ---- second_gemm_backward
+    act = torch.randn(R, f, generator=g).half()
+    g_y = torch.randn(n_flat, d, generator=g).half()
+    _say("second_gemm_backward")
+    g_buf, g_w2, g_b2 = m.second_gemm_backward(g_y.cuda(), to_padded(act).cuda(), *csr, w2, t["b2"].cuda(), pos,
+                                               *blocks)
+    ref_act, ref_w2, ref_b2 = O.ffn2_backward(g_y, act, pos_ref, off_ref, t["w2"])
+    assert tuple(g_buf.shape) == (nb * bs, f)
+    g_buf = g_buf.cpu()
+    assert not g_buf[~valid].any(), "padding rows of grad_inp_buf must be zero"
+    for got, ref, what in ((g_buf[valid], ref_act[sorted_of_padded[valid]], "grad_inp_buf"),
+                           (g_w2, ref_w2, "grad_w2"), (g_b2, ref_b2, "grad_b2")):
+        got, ref = got.float().cpu(), ref.float()
+        assert O.max_abs_err(got, ref) <= MAX_ABS * max(1.0, float(ref.abs().max())), what
+        assert O.mean_rel_err(got, ref) <= MEAN_REL, what
+    with pytest.raises(ValueError):                              # the backward takes the stored layout only
+        m.second_gemm_backward(g_y.cuda(), to_padded(act).cuda(), *csr, w2.transpose(-2, -1).contiguous(),
+                               t["b2"].cuda(), pos, *blocks)
+
+
 def test_ep_share_segments(workloads):
     """One GPU's expert-parallel share at reduced rows: (start, len, expert) triples."""
     from ccfuser_amd import ops
@@ -178,35 +245,109 @@ def test_error_paths_raise():
         ops.gate_topk_softmax(x.half(), torch.randn(4, 64, device="cuda").half(), None, 9)
 
 
-@pytest.mark.parametrize("name", ["c3_mixtral", "c5_skewed"])
-def test_full_size_properties(workloads, name):
-    """At BASELINE sizes the oracle's FFN is too slow for a unit test, so check what
-    does not depend on size: routing bit-exact against the oracle (integer work is
-    cheap), every output row finite, top-1 rows equal their expert's dense MLP on a
-    sample, and scaling the gate scores scales the output (linearity of the combine)."""
+def _dense_token(t, tok, experts, scores):
+    """The layer's output row of one token by the dense per-token formula in fp32; a
+    dropped slot (expert -1) contributes zero."""
+    acc = torch.zeros(t["x"].shape[1])
+    for e, sc in zip(experts, scores):
+        if e < 0:
+            continue
+        h = O.gelu_exact(t["w1"][e].float() @ t["x"][tok].float() + t["b1"][e].float())
+        acc += float(sc) * (t["w2"][e].float() @ h + t["b2"][e].float())
+    return acc
+
+
+def _full_size_check(wl, t, n_sample=48, must_drop=False):
+    """Size-independent checks of the fused call at full size: routing bit-exact against the
+    oracle (integer work is cheap on the CPU), every output finite, sampled tokens against the
+    dense per-token formula, and exact linearity in the second layer's parameters."""
     from ccfuser_amd import ops
-    wl = workloads(name)
-    t = wl.tensors
-    _say(f"full size {name}")
+    E, k = wl.num_expert, wl.top_k
     args = [t[n].cuda() for n in ("x", "wg", "bg", "w1", "b1", "w2", "b2")]
-    out, r = ops.moe_forward(*args, wl.top_k, wl.capacity, return_routing=True)
+    out, r = ops.moe_forward(*args, k, wl.capacity, return_routing=True)
     torch.cuda.synchronize()
-    idx_ref, score_ref, _ = O.naive_gate(t["x"], t["wg"], t["bg"], wl.top_k)
-    assert torch.equal(r["idx"].cpu(), idx_ref)
-    pos_ref, off_ref = O.assign_pos(idx_ref, wl.num_expert)
+    idx_ref, score_ref, _ = O.naive_gate(t["x"], t["wg"], t["bg"], k)
+    kept_ref = O.limit_by_capacity(idx_ref, E, wl.capacity)
+    dropped = int((kept_ref < 0).sum())
+    _say(f"  routed {int((kept_ref >= 0).sum())} rows, {dropped} slots dropped by capacity {wl.capacity}")
+    assert not must_drop or dropped > 0
+    assert torch.equal(r["idx"].cpu(), kept_ref)
+    pos_ref, off_ref = O.assign_pos(kept_ref, E)
+    R = int(off_ref[-1])
     assert torch.equal(r["offsets"].cpu(), off_ref)
-    assert torch.equal(r["pos"].cpu(), pos_ref)
+    assert torch.equal(r["counts"].cpu().long(), O.expert_count(kept_ref, E).long())
+    assert torch.equal(r["pos"].cpu()[:R], pos_ref)
     assert torch.isfinite(out.float()).all()
-    # sampled rows against the dense per-token formula in fp32
     g = torch.Generator().manual_seed(0)
-    sample = torch.randperm(wl.tokens, generator=g)[:48]
-    for tok in sample.tolist():
-        acc = torch.zeros(wl.d_model)
-        for s in range(wl.top_k):
-            e = int(idx_ref[tok, s])
-            h = O.gelu_exact(t["w1"][e].float() @ t["x"][tok].float() + t["b1"][e].float())
-            acc += float(score_ref[tok, s]) * (t["w2"][e].float() @ h + t["b2"][e].float())
-        assert (out[tok].cpu().float() - acc).abs().max() <= MAX_ABS
+    sample = torch.randperm(wl.tokens, generator=g)[:n_sample].tolist()
+    if dropped:                                       # make sure tokens that lost a slot are among the sample
+        lost = torch.nonzero((kept_ref < 0).any(-1)).view(-1)
+        sample += lost[torch.randperm(lost.numel(), generator=g)[:8]].tolist()
+    for tok in sample:
+        ref_row = _dense_token(t, tok, kept_ref[tok].tolist(), score_ref[tok].tolist())
+        assert (out[tok].cpu().float() - ref_row).abs().max() <= MAX_ABS, tok
+    # Linearity: the output is linear in (w2, b2), and doubling is exact in fp16 and in the
+    # fp32 accumulators, so doubling both doubles every output bit for bit, except where an
+    # expert output falls into fp16's subnormal range (below 2^-14 the rounding step is
+    # absolute, so rounding does not commute with doubling there): such an element may move the
+    # token's sum by one rounding step.
+    out2 = ops.moe_forward(args[0], args[1], args[2], args[3], args[4], args[5] * 2, args[6] * 2, k, wl.capacity)
+    want = out.float() * 2
+    diff = (out2.float() - want).abs()
+    assert bool((diff <= want.abs() * 2.0 ** -10 + 2.0 ** -22).all()), "doubling w2 and b2 did not double the output"
+    mism = float((diff > 0).float().mean())
+    _say(f"  linearity: {mism:.2e} of the elements off by one rounding step")
+    assert mism < 1e-2
+
+
+@pytest.mark.parametrize("name", ["c2_gshard", "c3_mixtral", "c5_skewed"])
+def test_full_size_properties(workloads, name):
+    """At BASELINE sizes the oracle's FFN is too slow for a unit test, so check what does not
+    depend on size (see _full_size_check)."""
+    wl = workloads(name)
+    _say(f"full size {name}")
+    _full_size_check(wl, wl.tensors)
+
+
+def test_full_size_gshard_shape_with_binding_capacity(workloads):
+    """The capacity-limited workload's own seed routes almost uniformly, so its capacity of
+    2560 rows per expert drops nothing.  Same shapes and tensors with a gate bias that sends
+    most tokens to experts 2 and 5: both overflow, their late slots are dropped (expert -1,
+    score kept, zero contribution) and every other check of the full-size test must hold."""
+    wl = workloads("c2_gshard")
+    t = dict(wl.tensors)
+    bg = t["bg"].clone().float()
+    bg[2] += 0.6
+    bg[5] += 0.5
+    t["bg"] = bg.half()
+    _say("full size c2_gshard shapes, biased gate")
+    _full_size_check(wl, t, must_drop=True)
+
+
+def test_full_size_ep_share_segments(workloads):
+    """One GPU's expert-parallel share at its full 16384 inbound rows (K = 8192 in the second
+    GEMM, so the last round of tiles is cut along K): sampled rows against the dense formula,
+    rows outside every segment untouched, a second call bit-identical."""
+    from ccfuser_amd import ops
+    wl = workloads("c4_ep_share")
+    t = wl.tensors
+    names = ("x", "seg_start", "seg_len", "seg_expert", "w1", "b1", "w2", "b2")
+    _say(f"full size c4_ep_share rows={wl.tokens} n_seg={t['seg_start'].numel()}")
+    args = [t[n].cuda() for n in names]
+    y = ops.moe_ffn_segments(*args)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    expert_of_row = torch.full((wl.tokens,), -1, dtype=torch.long)
+    for st, ln, e in zip(t["seg_start"].tolist(), t["seg_len"].tolist(), t["seg_expert"].tolist()):
+        expert_of_row[st:st + ln] = e
+    assert (expert_of_row >= 0).all()                     # the segments tile the inbound buffer
+    g = torch.Generator().manual_seed(1)
+    rows = torch.randperm(wl.tokens, generator=g)[:48].tolist()
+    rows += [0, wl.tokens - 1] + t["seg_start"].tolist()[:8]      # buffer ends and segment heads
+    for r_ in rows:
+        ref_row = _dense_token(t, r_, [int(expert_of_row[r_])], [1.0])
+        assert (y[r_].cpu().float() - ref_row).abs().max() <= MAX_ABS, r_
+    assert torch.equal(y, ops.moe_ffn_segments(*args))
 
 
 def test_forward_replays_from_a_hip_graph(workloads):
