@@ -51,6 +51,8 @@ struct GroupedArgs {
   // split last round (layout in plan.h): header and part entries, fp32 partial tiles
   const int32_t *tail;
   float *partial;
+  // skinny list (layout in plan.h) of this GEMM, or NULL
+  const int32_t *skinny;
 };
 
 // erf-form GELU, v * Phi(v) with Phi(v) = 0.5 + 0.5*erf(v/sqrt2) = 0.5 + u*Q(u^2), u = v
@@ -385,6 +387,166 @@ grouped_gemm_kernel(GroupedArgs p) {
   }
 }
 
+// ---- skinny tiles -----------------------------------------------------------------
+// The rows an expert has beyond its full 256-row tiles, when the plan says so (plan.h tells which
+// rows and when), as 64 x 256 tiles over the skinny list.  Such a tile does little arithmetic
+// per byte of weights it streams, so this loop is built for memory latency, not for the MFMA
+// pipe: four whole-K-tile stages of 40 KB (the persistent kernel's 160 KB of LDS: three K tiles
+// in flight while one is read), the same direct-to-LDS loads and XOR swizzle as the main loop,
+// four wavefronts side by side along N (64 x 64 each), fragment reads and MFMAs back to back.
+// It runs in the few workgroups per XCD of the persistent kernel that the plan sets aside:
+// worker `worker` of `ns` on XCD `xcd` takes entries worker, worker + ns, ... of that XCD's
+// share of the list.  Accumulation runs over K in the same 32-wide steps and the same order as
+// in the main loop, so a skinny tile gives the bits a 256-row tile would give.
+struct SkinnyCfg {
+  static constexpr int BM = kSkinnyRows, BN = 256, BK = 64;
+  static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES, STAGES = 4;
+  static constexpr int A_DMA = BM / 8 / 4, B_DMA = BN / 8 / 4;     // tile loads per wavefront: 8 rows of 128 bytes each
+  static constexpr int TM = BM / 16, TN = 4;                       // 16 x 16 blocks per wavefront (64 x 64)
+  static constexpr int LOADS = A_DMA + B_DMA;
+};
+
+// acc += w (16 weight rows) x t (16 token rows), K = 32, on ordinary registers
+__device__ __forceinline__ void mfma16_v(float4v &acc, const half8 &w, const half8 &t) {
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(t));
+}
+
+template <int kEpi>
+__device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, int ns, int xcd, lds_char *lds,
+                                            uint32_t lds_base) {
+  using C = SkinnyCfg;
+  static_assert(C::STAGES * C::STAGE_BYTES <= 5 * 32768, "the stages share the ring's LDS");
+  const int T = p.skinny[0], per_x = p.skinny[2];
+  const int4v *list = reinterpret_cast<const int4v *>(p.skinny + 4);
+  const int tid = fresh_tid(), lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // = the wavefront's 64 columns
+  const int KT = p.K / C::BK;
+  // this lane's fragment chunk of row block 0, per K half (16x16x32 operand: row lane%16, K chunk lane/16)
+  uint32_t a_off[2], b_off[2];
+  {
+    const int ra = lane & 15, rb = wave * 64 + (lane & 15);
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      const int c = sub * 4 + (lane >> 4);
+      a_off[sub] = (ra * 8 + (c ^ swz<8>(ra))) * 16;
+      b_off[sub] = C::A_BYTES + (rb * 8 + (c ^ swz<8>(rb))) * 16;
+    }
+  }
+  for (int i = worker; i < per_x; i += ns) {
+    const int w = xcd * per_x + i;
+    if (w >= T) break;
+    const int4v ent = list[w];
+    const int e = ent[0], row0 = ent[1], rows = ent[2], n0 = ent[3] * C::BN;
+    int live_m = (rows + 15) / 16;                                 // 16-row blocks with real rows
+    live_m = __builtin_amdgcn_readfirstlane(live_m > C::TM ? C::TM : live_m);
+    // global source of every tile load of this lane
+    const half_t *a_src[C::A_DMA], *b_src[C::B_DMA];
+    const half_t *Be = p.B + static_cast<size_t>(e) * p.N * p.K;
+#pragma unroll
+    for (int j = 0; j < C::A_DMA; ++j) {
+      const int r = (j * 4 + wave) * 8 + (lane >> 3);
+      int g = row0 + (r < rows ? r : rows - 1);                    // padded tile rows re-read the last real row
+      if (p.a_rows) g = p.a_rows[g];
+      a_src[j] = p.A + static_cast<size_t>(g) * p.K + ((lane & 7) ^ swz<8>(r)) * 8;
+    }
+#pragma unroll
+    for (int j = 0; j < C::B_DMA; ++j) {
+      const int r = (j * 4 + wave) * 8 + (lane >> 3);
+      const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
+      b_src[j] = Be + static_cast<size_t>(n) * p.K + ((lane & 7) ^ swz<8>(r)) * 8;
+    }
+    auto issue = [&](int kt, int stage) {                          // K tile kt into a stage
+      const int k_elem = (kt < KT ? kt : KT - 1) * C::BK;          // past the end: the last tile again, into a stage nobody reads
+      lds_char *base = lds + stage * C::STAGE_BYTES;
+#pragma unroll
+      for (int j = 0; j < C::A_DMA; ++j) lds_dma16(a_src[j] + k_elem, base + (j * 4 + wave) * 1024);
+#pragma unroll
+      for (int j = 0; j < C::B_DMA; ++j) lds_dma16(b_src[j] + k_elem, base + C::A_BYTES + (j * 4 + wave) * 1024);
+    };
+    float4v acc[C::TM][C::TN];
+#pragma unroll
+    for (int tm = 0; tm < C::TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < C::TN; ++tn) acc[tm][tn] = float4v{0, 0, 0, 0};
+    wait_vmcnt<0>();                                               // the previous tile's stores: the waits below count loads only
+    block_barrier();                                               // and its last LDS reads are done
+    issue(0, 0);
+    issue(1, 1);
+    issue(2, 2);
+    int stage = 0;
+    for (int kt = 0; kt < KT; ++kt) {
+      // K tile kt has landed for this wavefront (the loads of the two tiles behind it may be in flight), then for all
+      wait_vmcnt<2 * C::LOADS>();
+      block_barrier();
+      // behind the barrier everyone is done with K tile kt-1, whose stage takes K tile kt+3
+      issue(kt + 3, stage >= 1 ? stage - 1 : C::STAGES - 1);
+      const uint32_t sb = lds_base + stage * C::STAGE_BYTES;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        half8 a[C::TM], b[C::TN];
+        static_for<0, C::TN>([&](auto J) { b[J.value] = lds_read_b128<J.value * 2048>(sb + b_off[sub]); });
+        static_for<0, C::TM>([&](auto I) { a[I.value] = lds_read_b128<I.value * 2048>(sb + a_off[sub]); });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int q = 0; q < C::TM; ++q) asm volatile("" : "+v"(a[q]));
+#pragma unroll
+        for (int q = 0; q < C::TN; ++q) asm volatile("" : "+v"(b[q]));
+        static_for<0, C::TM>([&](auto I) {
+          constexpr int tm = I.value;
+          if (tm < live_m) {                                       // uniform
+#pragma unroll
+            for (int tn = 0; tn < C::TN; ++tn) mfma16_v(acc[tm][tn], b[tn], a[tm]);
+          }
+        });
+      }
+      stage = stage == C::STAGES - 1 ? 0 : stage + 1;
+    }
+    wait_vmcnt<0>();                                               // the redundant loads past the end
+    // the MFMAs are opaque to the compiler: keep the distance it would keep before their results are read
+    asm volatile("s_nop 15\n s_nop 15" ::: "memory");
+#pragma unroll
+    for (int tm = 0; tm < C::TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < C::TN; ++tn) asm volatile("" : "+v"(acc[tm][tn]));
+    // epilogue: bias, GELU or row scale, fp16 through the row index; 8-byte stores
+    const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
+    const int colb = n0 + wave * 64 + 4 * (lane >> 4);             // column of block tn = colb + 16 tn
+#pragma unroll
+    for (int tm = 0; tm < C::TM; ++tm) {
+      if (tm >= live_m) break;                                     // uniform
+      const int r = tm * 16 + (lane & 15);
+      const bool real = r < rows;
+      const int j = row0 + (real ? r : rows - 1);
+      const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
+      const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
+      half_t *dst = p.C + crow * p.N;
+      half_t *row2 = kEpi == kEpiGeluKeep ? p.C2 + static_cast<size_t>(j) * p.N : nullptr;
+#pragma unroll
+      for (int tn = 0; tn < C::TN; ++tn) {
+        const int col = colb + 16 * tn;
+        if (!real || col >= p.N) continue;
+        half4 bv = {0, 0, 0, 0};
+        if (p.bias) bv = *reinterpret_cast<const half4 *>(bias_e + col);
+        half4 o, pre;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          float x = acc[tm][tn][c] + static_cast<float>(bv[c]);
+          if (kEpi == kEpiPlain) {
+            x *= sc;
+          } else {
+            pre[c] = static_cast<half_t>(x);
+            x = gelu_erf(x);
+          }
+          o[c] = static_cast<half_t>(x);
+        }
+        *reinterpret_cast<half4 *>(dst + col) = o;
+        if (kEpi == kEpiGeluKeep) *reinterpret_cast<half4 *>(row2 + col) = pre;
+      }
+    }
+  }
+  wait_vmcnt<0>();
+}
+
 // ---- persistent form -------------------------------------------------------------
 // One workgroup per CU walks the plan entries of its XCD (entry b belongs to XCD
 // b % 8; the workgroup with blockIdx b takes slots b/8, b/8 + gridDim/8, ...).
@@ -410,8 +572,20 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   const int bmul = kKN ? p.N : 1;                     // elements between K rows of a [K][N] B
   constexpr int TM = R::TM, TN = R::TN;
   const int4v *plan = reinterpret_cast<const int4v *>(p.plan);
-  const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
+  const int xcd = blockIdx.x & 7;
+  int stride = gridDim.x >> 3;
   int slot_j = blockIdx.x >> 3;
+  if constexpr (!kSeg && !kKN && kEpi <= kEpiGeluKeep) {
+    // the last ns workgroups of each XCD do the skinny tiles (if the plan has any), the others the 256-row tiles
+    if (p.skinny) {
+      const int ns = __builtin_amdgcn_readfirstlane(p.skinny[1]);
+      stride -= ns;
+      if (slot_j >= stride) {
+        skinny_role<kEpi>(p, slot_j - stride, ns, xcd, R::lds(), R::lds_addr());
+        return;
+      }
+    }
+  }
   if (slot_j >= slots_per_xcd) return;
   int4v ent = plan[slot_j * 8 + xcd];
   if (ent[0] < 0) return;                             // the used slots of an XCD are a prefix
@@ -676,11 +850,14 @@ int g_split_tail = 1;        // 0: the last round of tiles is not cut along K
 constexpr int kSplitTailMinKT = 64;
 int g_split_tail_min_kt = kSplitTailMinKT;
 int g_split_max_parts = 8;
+int g_skinny_pct = 70;       // a K step of a skinny tile in percent of a 256-row tile's (plan model); 0: no skinny tiles
 
 // The tuning knobs a grouped GEMM's plan and launches depend on, read once per call: the plan
 // and the kernels that consume it must agree even if another thread calls ccf_set_option
 // between the routing stage (which builds the plans of the layer's forward call) and the GEMMs.
-GemmOptions current_options() { return GemmOptions{g_variant, g_split_tail, g_split_tail_min_kt, g_split_max_parts}; }
+GemmOptions current_options() {
+  return GemmOptions{g_variant, g_split_tail, g_split_tail_min_kt, g_split_max_parts, g_skinny_pct};
+}
 
 struct Launch {
   int bm, bn, threads;
@@ -735,9 +912,14 @@ constexpr int kMinBN = 128;
 // Workspace of one grouped GEMM: the split-K tail area, then the tile plan.  A second plan
 // (region 1: header and entries of its own, then the plan; the partial tiles are shared) follows
 // in the forward workspace, so that the plans of both GEMMs of a layer can exist at once.
-size_t plan_only_bytes(int max_rows, int E, int n_max) {
+size_t plan_core_bytes(int max_rows, int E, int n_max) {
   return round_up(sizeof(int32_t) * plan_ints(launched_wgs(max_tiles_for(max_rows, E, kMinBM),
                                                            (n_max + kMinBN - 1) / kMinBN)), 256);
+}
+// the tile plan, then the skinny list
+size_t plan_only_bytes(int max_rows, int E, int n_max) {
+  return plan_core_bytes(max_rows, E, n_max) +
+         round_up(sizeof(int32_t) * skinny_ints(max_rows, E, (n_max + kMinBN - 1) / kMinBN), 256);
 }
 size_t plan_bytes(int max_rows, int E, int n_max) { return kTailBytes + plan_only_bytes(max_rows, E, n_max); }
 size_t forward_ws_bytes(int max_rows, int E, int n_max) {
@@ -746,9 +928,14 @@ size_t forward_ws_bytes(int max_rows, int E, int n_max) {
 
 // Everything the launches of one grouped GEMM derive from its sizes, and the request that
 // builds its plan.
+// Epilogue of a 256-row tile in K steps of the main loop (for the plan's cost model): the GELU
+// epilogue is ~13 us, the plain one ~7 us, a K step ~1.45 us.
+constexpr int kEpiCostGelu = 9, kEpiCostPlain = 5;
+
 struct GemmSetup {
   const Launch *v;
-  bool second, split;
+  bool second, split, skinny;
+  int32_t *skinny_list;
   int grid;
   long long wgs;
   int32_t *tail, *plan;
@@ -781,8 +968,13 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
   // worth its two small launches only where a tile is long: K of 4096 and more)
   g.split = opt.split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && g.grid >= 8 && g.grid <= g.wgs &&
             g.grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= opt.split_tail_min_kt;
+  // remainder rows as skinny tiles: forward epilogues of the persistent 256 x 256 kernel with the [N][K] weight
+  g.skinny = opt.skinny_pct != 0 && !b_kn && epi <= kEpiGeluKeep && g.grid >= 64 && g.grid <= g.wgs &&
+             v.bm == Cfg5::BM && v.bn == Cfg5::BN && v.persistent_plain;
+  g.skinny_list = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.plan) + plan_core_bytes(max_rows, E, N > K ? N : K));
   g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, opt.split_max_parts, g.plan,
-                  g.split ? g.tail : nullptr};
+                  g.split ? g.tail : nullptr, g.skinny ? g.skinny_list : nullptr, g.grid,
+                  gelu ? kEpiCostGelu : kEpiCostPlain, opt.skinny_pct};
   return g;
 }
 
@@ -838,6 +1030,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.seg_rows = 0;
   p.tail = tail;
   p.partial = partial;
+  p.skinny = gs.skinny ? gs.skinny_list : nullptr;
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;                // wgs is a multiple of 8
     hipLaunchKernelGGL(second ? v.persistent_gelu : v.persistent_plain, dim3(static_cast<unsigned>(g)),
@@ -875,7 +1068,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream,
-                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr}, row_off, E);
+                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0}, row_off, E);
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
   p.A = A;
@@ -895,6 +1088,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.seg_rows = M;
   p.tail = nullptr;
   p.partial = nullptr;
+  p.skinny = nullptr;
   const int grid = persistent_grid();
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;
@@ -1022,6 +1216,13 @@ extern "C" int ccf_set_option(const char *name, int value) {
   if (!strcmp(name, "split_parts")) {        // most parts a tile of the split last round is cut into
     CCF_REQUIRE(value >= 2 && value <= 8, CCF_ERR_ARG, "set_option: split_parts %d outside 2..8", value);
     g_split_max_parts = value;
+    return CCF_OK;
+  }
+  if (!strcmp(name, "skinny")) {             // 0: off; 1: default; n > 1: cost of a skinny K step in percent (plan model);
+                                             // -n: always, with n workgroups per XCD
+    CCF_REQUIRE(value >= -kSkinnyMaxWgs && value <= 400, CCF_ERR_ARG, "set_option: skinny %d outside %d..400", value,
+                -kSkinnyMaxWgs);
+    g_skinny_pct = value == 1 ? 70 : value;
     return CCF_OK;
   }
   if (!strcmp(name, "dgrad_transpose")) {

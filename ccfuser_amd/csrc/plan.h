@@ -33,6 +33,48 @@ constexpr int kTailMaxTiles = kTailMaxParts / 2;     // tile slots: every tile h
 constexpr size_t kTailHead = 256 + 16 * kTailMaxParts;
 constexpr size_t kTailBytes = kTailHead + static_cast<size_t>(kTailMaxParts) * 256 * 256 * 4;
 
+// ---- skinny tiles --------------------------------------------------------------
+// An expert's rows rarely fill its last 256-row M tile, and a tile with a few dozen real rows
+// costs a CU as much as a full one: its K steps are paced by the tile loads, not by the MFMAs
+// it skips.  With a skinny list in the plan request, a remainder of at most kSkinnyRows rows
+// (rows % BM, or all rows of an expert smaller than that) may leave the plan of 256-row tiles
+// and become one entry per N tile of a second list.  A few workgroups per XCD of the persistent
+// kernel (ffn.hip) then do nothing but those entries, as 64 x 256 tiles that stream their
+// weight panel through a deep LDS pipeline: little arithmetic, mostly memory latency, so they
+// run beside the compute-bound 256-row tiles on bandwidth those leave idle.  Whether that pays
+// depends on the tile counts (a CU taken from the 256-row tiles costs them 1/32 of their
+// rate; whole rounds of tiles matter more than tiles), so build_plan prices both ways with a
+// small model and picks: ns = workgroups per XCD given to skinny tiles, 0 = none (every row
+// stays in 256-row tiles).  Layout of the list (int32):
+//   [0] tiles T   [1] ns   [2] tiles per XCD (XCD x owns entries [x * [2], (x + 1) * [2]))   [3] unused
+//   [4 + 4 i ...] entry i < T: {expert, first sorted row, rows (1..kSkinnyRows), N tile}
+constexpr int kSkinnyRows = 64;
+constexpr int kSkinnyMaxWgs = 4;                     // per XCD
+__host__ __device__ inline size_t skinny_ints(int max_rows, int E, int n_tiles_n) {
+  const int most = E < max_rows ? E : max_rows;      // at most one skinny M tile per expert
+  return 4 + 4 * static_cast<size_t>(most > 0 ? most : 0) * n_tiles_n;
+}
+
+// Time, in K steps of a 256-row tile, that F tiles of k_tiles K steps and an epilogue worth
+// `epi` K steps take on spx workgroups: whole rounds, then the last, partly filled round, which
+// is cut along K when the request allows it (same rule as the split below).
+__device__ inline int rounds_cost(int F, int spx, int k_tiles, int epi, bool may_split, int max_parts) {
+  if (spx <= 0) return INT_MAX / 2;
+  const int r = F % spx;
+  int cost = F / spx * (k_tiles + epi);
+  if (r > 0) {
+    int S = 0;
+    if (may_split && 2 * r <= spx) {
+      S = spx / r;
+      S = S > max_parts ? max_parts : S;
+      S = S > k_tiles / 4 ? k_tiles / 4 : S;
+      S = (S >= 2 && 8 * r * S <= 256) ? S : 0;
+    }
+    cost += S ? k_tiles / S + 16 : k_tiles + epi;    // 16: two more launches, pipeline fill, the reduction
+  }
+  return cost;
+}
+
 // Rows of M tile i of an expert with cnt rows in nt = ceil(cnt / BM) tiles.  When
 // the last tile would hold at most BM/2 rows, it and the one before it share
 // their rows evenly instead: a nearly empty tile still streams a whole weight
@@ -67,6 +109,11 @@ struct PlanReq {
   int max_parts;    // most parts a tile is cut into
   int32_t *plan;
   int32_t *tail;    // split scratch (header and entries), or NULL
+  int32_t *skinny;  // skinny list, or NULL: every row goes through the 256-row tiles
+  int cus;          // workgroups of the persistent launch (a multiple of 8)
+  int epi_cost;     // the epilogue of a 256-row tile, in K steps
+  int skinny_pct;   // a K step of a skinny tile in percent of a K step of a 256-row tile; 0 = never use skinny
+                    // tiles; -n = always, with n workgroups per XCD
 };
 
 // Built by `nparts` workgroups of any size that is a multiple of 64 (all threads of each call
@@ -76,9 +123,11 @@ struct PlanReq {
 __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__ offsets, int E,
                                   int part = 0, int nparts = 1) {
   const int BM = rq.BM, max_tiles = rq.max_tiles, max_rows = rq.max_rows, n_tiles_n = rq.n_tiles_n;
-  const int spx = rq.spx, k_tiles = rq.k_tiles;
+  const int k_tiles = rq.k_tiles;
+  int spx = rq.spx;                 // lowered below by the workgroups given to skinny tiles
   int32_t *__restrict__ plan = rq.plan;
   int32_t *__restrict__ tail = rq.tail;
+  int32_t *__restrict__ skinny = rq.skinny;
   __shared__ int s_full[8];        // split last round: slots of XCD x from s_full[x] on go to the tail list
   __shared__ int s_used[8];        // tiles of XCD x
   __shared__ int s_parts;          // parts per tail tile, 0 = no split
@@ -90,16 +139,60 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     s_off[e] = v < max_rows ? v : max_rows;          // never plan past the caller's bound
   }
   __syncthreads();
+  __shared__ int s_ns;             // workgroups per XCD given to skinny tiles (0: every row in 256-row tiles)
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
+    // Skinny tiles or not: tile counts both ways, then the cheaper plan by the model above.
+    int ns_wgs = 0;
+    if (skinny && rq.skinny_pct != 0 && rq.cus >= 64) {
+      int nl0 = 0, nl1 = 0, nk1 = 0;                // 256-row tiles without / with skinny tiles, skinny M tiles
+      for (int e = lane; e < E; e += 64) {
+        int cnt = s_off[e + 1] - s_off[e];
+        cnt = cnt > 0 ? cnt : 0;
+        const int nt = (cnt + BM - 1) / BM, r = cnt % BM;
+        const int sk = (r > 0 && r <= kSkinnyRows) ? 1 : 0;
+        nl0 += nt;
+        nl1 += nt - sk;
+        nk1 += sk;
+      }
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) {
+        nl0 += __shfl_xor(nl0, off, 64);
+        nl1 += __shfl_xor(nl1, off, 64);
+        nk1 += __shfl_xor(nk1, off, 64);
+      }
+      if (nk1 > 0 && rq.skinny_pct < 0) {
+        ns_wgs = -rq.skinny_pct < kSkinnyMaxWgs ? -rq.skinny_pct : kSkinnyMaxWgs;   // forced (tests, measurements)
+      } else if (nk1 > 0) {
+        const int cus_x = rq.cus / 8;
+        const bool may_split = spx > 0;
+        const int F0 = (nl0 * n_tiles_n + 7) / 8, F1 = (nl1 * n_tiles_n + 7) / 8, T_x = (nk1 * n_tiles_n + 7) / 8;
+        int best = rounds_cost(F0, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts);
+        const int sk_tile = (k_tiles * rq.skinny_pct + 99) / 100 + 3;         // one skinny tile, in K steps
+        for (int n = 1; n <= kSkinnyMaxWgs && n * 4 <= cus_x; ++n) {
+          const int main_c = rounds_cost(F1, cus_x - n, k_tiles, rq.epi_cost, may_split, rq.max_parts);
+          const int sk_c = (T_x + n - 1) / n * sk_tile;
+          const int c = main_c > sk_c ? main_c : sk_c;
+          if (c < best) { best = c; ns_wgs = n; }
+        }
+      }
+    }
+    if (lane == 0) s_ns = ns_wgs;
     int carry_l = 0, carry_s = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
       int cnt = e < E ? s_off[e + 1] - s_off[e] : 0;
       cnt = cnt > 0 ? cnt : 0;
       const int nt = (cnt + BM - 1) / BM;
-      const int ns = (nt == 1 && cnt <= BM / 2) ? 1 : 0;        // a short tile only when it is the expert's only one
-      const int nl = nt - ns;
+      int ns, nl;
+      if (ns_wgs) {
+        const int r = cnt % BM;                                   // ns counts skinny M tiles here
+        ns = (r > 0 && r <= kSkinnyRows) ? 1 : 0;
+        nl = nt - ns;
+      } else {
+        ns = (nt == 1 && cnt <= BM / 2) ? 1 : 0;                  // a short tile only when it is the expert's only one
+        nl = nt - ns;
+      }
       int inc_l = nl, inc_s = ns;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
@@ -124,8 +217,18 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   // tiles on XCD x, its slot j is long tile x*per_long + j for j < nl, else
   // short tile x*per_short + (j - nl).  The used slots of an XCD are a prefix:
   // the first idle entry ends its list.
+  const int ns_wgs = s_ns;                                       // published by the barrier above
+  const bool use_skinny = ns_wgs > 0;
+  if (spx > 0) spx -= ns_wgs;
   const int total_long = s_long[E] * n_tiles_n;
-  const int total_short = s_short[E] * n_tiles_n;
+  const int total_short = use_skinny ? 0 : s_short[E] * n_tiles_n;   // skinny tiles are not in this plan
+  if (skinny && part == 0 && threadIdx.x == 0) {
+    const int T = use_skinny ? s_short[E] * n_tiles_n : 0;
+    skinny[0] = T;
+    skinny[1] = ns_wgs;
+    skinny[2] = (T + 7) / 8;
+    skinny[3] = 0;
+  }
   const int per_long = (total_long + 7) / 8;
   const int per_short = (total_short + 7) / 8;
   // The split last round (run by grouped_gemm_tail_kernel and splitk_reduce_kernel in ffn.hip).
@@ -199,6 +302,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     // for a M tiles, a token tile once for 32/a N tiles, and HBM traffic per
     // patch, which goes as 1/a + a/32, is near its minimum for a = 4..8.
     const int first = s_long[e] * n_tiles_n;
+    const int cnt_long = (use_skinny && ns) ? cnt - cnt % BM : cnt;   // rows the 256-row tiles hold
     for (int l = lane; l < nl * n_tiles_n; l += 64) {
       const int run = l / (kOrderGroupM * n_tiles_n);            // which run of M tiles
       const int run_first = run * kOrderGroupM;
@@ -208,10 +312,14 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       const int tn = in_run / run_size;
       const int logical = first + l;
       int first_row, rows;
-      tile_rows(cnt, nl, i, BM, first_row, rows);
+      tile_rows(cnt_long, nl, i, BM, first_row, rows);
       place(logical % per_long, logical / per_long, int4v{e, lo + first_row, rows, tn});   // hardware id = slot * 8 + XCD
     }
-    if (ns) {
+    if (ns && use_skinny) {
+      int4v *sk = reinterpret_cast<int4v *>(skinny + 4);
+      const int first_s = s_short[e] * n_tiles_n;
+      for (int tn = lane; tn < n_tiles_n; tn += 64) sk[first_s + tn] = int4v{e, lo + cnt_long, cnt - cnt_long, tn};
+    } else if (ns) {
       const int i = nl;                                          // the expert's last M tile
       const int first_s = s_short[e] * n_tiles_n;
       for (int tn = lane; tn < n_tiles_n; tn += 64) {
@@ -229,7 +337,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
 // ffn.hip
 // Snapshot of the tuning knobs (ccf_set_option) that a grouped GEMM's plan and launches depend on.
 struct GemmOptions {
-  int variant, split_tail, split_tail_min_kt, split_max_parts;
+  int variant, split_tail, split_tail_min_kt, split_max_parts, skinny_pct;
 };
 GemmOptions forward_options();
 bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, const GemmOptions &opt,

@@ -59,6 +59,11 @@ const char *ccf_last_error(void);
  *   "split_tail"      0 = off, 1 = default, n > 1 = for K of n*64 and more: the tiles of a launch's
  *                     last, partly filled round are cut along K and reduced by a second kernel
  *   "split_parts"     2..8 (default 8): most parts such a tile is cut into
+ *   "skinny"          0 = off, 1 = default: rows an expert has beyond its full 256-row tiles (at most 64)
+ *                     may run as 64-row tiles in a few workgroups set aside for them, when the tile plan's
+ *                     cost model says that beats a padded 256-row tile; n > 1 sets the model's cost of
+ *                     such a tile's K step in percent of a 256-row tile's (default 70); -n (1..4) forces
+ *                     them with n workgroups per XCD
  *   "dgrad_transpose" 0/1: the backward's input-gradient GEMM runs on a transposed copy of the
  *                     weight instead of reading the stored one
  *   "gate_waves"      4 or 16: cap on the gate kernel's wavefronts per workgroup

@@ -68,6 +68,7 @@ def test_ffn_backward_stages_with_split_last_round(transpose):
     T, d, f, E, k = 4096, 2048, 2048, 6, 2
     ops.set_option("dgrad_transpose", transpose)
     ops.set_option("split_tail", 4)
+    ops.set_option("skinny", 0)               # every row in 256-row tiles: the tile count this test is built on
     try:
         _ffn_backward_stages(T, d, f, E, k, -1, False, 7)
         g = torch.Generator().manual_seed(77)
@@ -84,6 +85,7 @@ def test_ffn_backward_stages_with_split_last_round(transpose):
     finally:
         ops.set_option("dgrad_transpose", 0)
         ops.set_option("split_tail", 1)
+        ops.set_option("skinny", 1)
 
 
 def _ffn_backward_stages(T, d, f, E, k, cap, skew, seed):

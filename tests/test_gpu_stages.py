@@ -312,6 +312,7 @@ def test_split_k_tail_at_its_default_threshold():
     off, pos = r["offsets"].cpu(), r["pos"].cpu()
     _say(f"split-K tail by default R={R} d={d} f={f} E={E} counts={r['counts'].tolist()}")
     out = {}
+    ops.set_option("skinny", 0)               # every row in 256-row tiles: the tile count this test is built on
     for mode in (1, 0):
         ops.set_option("split_tail", mode)
         try:
@@ -321,6 +322,7 @@ def test_split_k_tail_at_its_default_threshold():
             out[mode] = (h.cpu(), y.cpu())
         finally:
             ops.set_option("split_tail", 1)
+    ops.set_option("skinny", 1)
     buf = x[pos].float()
     h_ref = torch.zeros(R, f)
     y_ref = torch.zeros(R, d)
@@ -355,6 +357,7 @@ def test_split_k_tail_all_epilogues():
     scale = (torch.rand(R, generator=g) + 0.5).half()
     _say(f"split-K tail R={R} d={d} f={f} E={E} counts={r['counts'].tolist()}")
     results = {}
+    ops.set_option("skinny", 0)               # every row in 256-row tiles: the tile count this test is built on
     for mode in (0, 4):
         ops.set_option("split_tail", mode)
         try:
@@ -365,6 +368,7 @@ def test_split_k_tail_all_epilogues():
             results[mode] = [t.cpu() for t in (h, act, pre, y)]
         finally:
             ops.set_option("split_tail", 1)
+    ops.set_option("skinny", 1)
     buf = x[torch.div(pos, 1, rounding_mode="floor")].float()
     h_ref = torch.zeros(R, f)
     pre_ref = torch.zeros(R, f)
@@ -386,3 +390,61 @@ def test_split_k_tail_all_epilogues():
     assert O.max_abs_err(results[4][3], results[0][3].float()) <= MAX_ABS
     assert O.max_abs_err(results[4][0], results[0][0].float()) <= MAX_ABS
     assert not torch.equal(results[4][3], results[0][3]) and not torch.equal(results[4][0], results[0][0])
+
+
+@pytest.mark.parametrize("R,d,f,E,skew,seed,mode", [
+    (8192, 4096, 4096, 6, False, 31, 1),       # remainders of ~80 rows: above 64, stay in 256-row tiles
+    (8192 + 6 * 200, 4096, 4096, 6, False, 35, 1),   # remainders of ~25 rows, long K: the plan's own choice
+    (3000, 256, 512, 5, False, 32, -2),        # short K
+    (2100, 1024, 2048, 40, True, 33, -1),      # most experts are nothing but a skinny tile, some are empty
+    (1150, 512, 768, 3, False, 34, -3),        # remainders of 127, 130 and 125 rows: none is skinny, nothing to do
+    (2000, 512, 768, 7, False, 36, -4),        # remainders around 30 rows, N no multiple of 256
+])
+def test_skinny_tiles(R, d, f, E, skew, seed, mode):
+    """Rows beyond an expert's full 256-row tiles (at most 64) run as 64-row tiles in workgroups
+    the plan sets aside (mode 1: when its cost model says so; -n: forced, n workgroups per XCD).
+    All three forward epilogues with that path on and off, each against fp32; both paths add
+    over K in the same order and must agree bit for bit."""
+    from ccfuser_amd import ops
+    x, w1, b1, w2, b2, e_of_row = _ffn_case(R, d, f, E, seed, skew)
+    g = torch.Generator().manual_seed(seed)
+    scale = (torch.rand(R, generator=g) + 0.5).half()
+    r = ops.route(dev(e_of_row), E, 1)
+    off, pos = r["offsets"].cpu().tolist(), r["pos"].cpu()
+    rem = r["counts"].cpu() % 256
+    _say(f"skinny mode={mode} R={R} d={d} f={f} E={E} remainders={rem.tolist()[:12]}")
+    res = {}
+    for m in (mode, 0):
+        ops.set_option("skinny", m)
+        ops.set_option("split_tail", 0)           # keep the 256-row path unsplit: the comparison is about the skinny path
+        try:
+            h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True)
+            act, pre = ops.ffn1_keep(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1))
+            y = torch.zeros(R, d, dtype=torch.float16, device="cuda")
+            ops.ffn2(h, r["dst_row"], r["offsets"], R, dev(w2), dev(b2), y, row_scale=dev(scale))
+            torch.cuda.synchronize()
+            res[m] = [t.cpu() for t in (h, act, pre, y)]
+        finally:
+            ops.set_option("skinny", 1)
+            ops.set_option("split_tail", 1)
+    buf = x[pos].float()
+    pre_ref = torch.zeros(R, f)
+    for e in range(E):
+        lo, hi = off[e], off[e + 1]
+        if hi > lo:
+            pre_ref[lo:hi] = buf[lo:hi] @ w1[e].float().t() + b1[e].float()
+    h_ref = O.gelu_exact(pre_ref)
+    for m, (h, act, pre, y) in res.items():
+        assert O.max_abs_err(h, h_ref) <= MAX_ABS and O.mean_rel_err(h, h_ref) <= MEAN_REL, m
+        assert torch.equal(h, act), m
+        assert O.max_abs_err(pre, pre_ref) <= MAX_ABS, m
+        y_ref = torch.zeros(R, d)
+        hq = h.float()
+        for e in range(E):
+            lo, hi = off[e], off[e + 1]
+            if hi > lo:
+                y_ref[pos[lo:hi]] = (hq[lo:hi] @ w2[e].float().t() + b2[e].float()) * scale[lo:hi].float()[:, None]
+        assert O.max_abs_err(y, y_ref) <= MAX_ABS and O.mean_rel_err(y, y_ref) <= MEAN_REL, m
+    same = [torch.equal(a, b) for a, b in zip(res[mode], res[0])]
+    _say(f"  skinny on/off bitwise equal (h, act, pre, y): {same}")
+    assert all(same)
