@@ -172,8 +172,13 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
   // launch (they need the offsets only), which saves the GEMMs a small launch each
   PlanReq plans[2];
   const GemmOptions opt = forward_options();        // one snapshot for the plans and the GEMMs that consume them
+  // top-1 without a capacity limit: every token has one slot, its score is exactly 1 (the softmax of
+  // one logit) and its flat row is its token row, so FFN2 writes the layer output itself
+  const bool direct = top_k == 1 && capacity < 0;
+  // top-2 with the option on: FFN2's epilogue adds score * y into the zero-filled output
+  const bool fuse = opt.fused_combine && top_k == 2 && d_model % 8 == 0;
   const bool planned = forward_plan_request(1, n, num_expert, d_model, d_ffn, w.ffn_ws, opt, &plans[0]) &&
-                       forward_plan_request(2, n, num_expert, d_model, d_ffn, w.ffn_ws, opt, &plans[1]);
+                       forward_plan_request(fuse ? 3 : 2, n, num_expert, d_model, d_ffn, w.ffn_ws, opt, &plans[1]);
   if ((rc = route_with_plans(w.idx, n, num_expert, top_k, capacity, w.counts, w.offsets, w.pos, w.src_row,
                              w.dst_row, w.inv_pos, w.idx_kept, w.route_ws, w.route_bytes, st, plans,
                              planned ? 2 : 0)))
@@ -183,14 +188,17 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
                          w.ffn_ws, w.ffn_bytes, st, planned ? &opt : nullptr)))
     return rc;
   mark_stage(3, st);
-  // top-1 without a capacity limit: every token has one slot, its score is exactly 1 (the softmax of
-  // one logit) and its flat row is its token row, so FFN2 writes the layer output itself
-  const bool direct = top_k == 1 && capacity < 0;
-  if ((rc = ffn2_forward(w.h, nullptr, w.dst_row, w.offsets, n, num_expert, d_model, d_ffn, w2, b2,
+  if (fuse) {
+    if ((rc = launch_zero(static_cast<half_t *>(out), static_cast<size_t>(tokens) * d_model, st))) return rc;
+    if ((rc = ffn2_forward_combine(w.h, w.src_row, w.dst_row, w.offsets, n, num_expert, d_model, d_ffn, w2, b2,
+                                   w.score, out, w.ffn_ws, w.ffn_bytes, st, planned ? &opt : nullptr)))
+      return rc;
+    mark_stage(4, st);
+  } else if ((rc = ffn2_forward(w.h, nullptr, w.dst_row, w.offsets, n, num_expert, d_model, d_ffn, w2, b2,
                          nullptr, direct ? out : w.y_flat, w.ffn_ws, w.ffn_bytes, st, planned ? &opt : nullptr)))
     return rc;
-  mark_stage(4, st);
-  if (!direct) {
+  if (!fuse) mark_stage(4, st);
+  if (!direct && !fuse) {
     if ((rc = ccf_combine(w.y_flat, w.score, w.inv_pos, out, tokens, top_k, d_model, stream)))
       return rc;
   }

@@ -40,6 +40,7 @@ struct GroupedArgs {
   half_t *C2;               // [*, N] in sorted row order: the pre-activation, written by epilogue 2, read by epilogue 3
   const int32_t *c_rows;    // row of C for sorted row j, or NULL (identity)
   const half_t *row_scale;  // [rows] or NULL; NULL with the GELU epilogue
+  const int32_t *scale_rows; // epilogue 4: row_scale is read at scale_rows[j]; NULL elsewhere
   const int32_t *plan;
   int N, K;
   // K-segment form (weight gradients): the contraction runs over a per-expert
@@ -103,7 +104,9 @@ __device__ __forceinline__ float gelu_erf_grad(float v) {
 //   1  C = gelu(acc + bias)
 //   2  as 1, and C2 = acc + bias (the pre-activation a later backward needs)
 //   3  C = (acc + bias) * gelu'(C2): an input gradient taken straight through the GELU
-constexpr int kEpiPlain = 0, kEpiGelu = 1, kEpiGeluKeep = 2, kEpiGeluGrad = 3;
+//   4  C[c_rows[j]] += (acc + bias) * row_scale[scale_rows[j]] with packed fp16 atomic adds: the gate-weighted
+//      combine in the second GEMM's epilogue (C zero-filled by the caller, c_rows = token of sorted row j)
+constexpr int kEpiPlain = 0, kEpiGelu = 1, kEpiGeluKeep = 2, kEpiGeluGrad = 3, kEpiCombine = 4;
 
 // Row of the tile's row range [0, rows) that tile row r (0 .. BM-1) holds; padded
 // tile rows repeat a real one.  The 16x16x32 kernels give the upper and the
@@ -241,7 +244,8 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
   for (int tm = 0; tm < TM; ++tm) {
     const int j = row0 + R::local_row(acc16_row<Cfg>(tm, tid), rows);
     crow_v[tm] = (!kPlainRows && p.c_rows) ? p.c_rows[j] : j;
-    sc_v[tm] = (!kPlainRows && p.row_scale) ? static_cast<float>(p.row_scale[j]) : 1.0f;
+    if constexpr (kEpi == kEpiCombine) sc_v[tm] = static_cast<float>(p.row_scale[p.scale_rows[j]]);
+    else sc_v[tm] = (!kPlainRows && p.row_scale) ? static_cast<float>(p.row_scale[j]) : 1.0f;
   }
   static_for<0, TM>([&](auto T) {
     constexpr int tm = T.value;
@@ -260,7 +264,7 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
     const int j = row0 + lr;
     const float sc = sc_v[tm];
     half_t *dst = p.C + static_cast<size_t>(crow_v[tm]) * p.N;
-    if constexpr (kEpi == kEpiPlain) {
+    if constexpr (kEpi == kEpiPlain || kEpi == kEpiCombine) {
       // A lane holds columns 4q .. 4q+3 of every 16-column block (q = lane / 16).  Lanes q and
       // q^1 of a row trade halves of a pair of blocks, after which the even one holds eight
       // consecutive columns of the first block and the odd one of the second: half as many
@@ -280,7 +284,19 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
                                                      : (v[2 * tp + h][c] + bias_v[2 * tp + h][c]) * sc);
         const int c16 = col[2 * tp] - 4 * q + (q & 1) * 16 + 4 * (q & 2);   // first of this lane's 8 columns
         const half8 out = pair_exchange(o[0], o[1]);
-        if (real && c16 < p.N) *reinterpret_cast<half8 *>(dst + c16) = out;
+        if constexpr (kEpi == kEpiCombine) {
+          // eight columns as four packed fp16 atomic adds (no return value)
+          if (real && c16 < p.N) {
+            typedef unsigned uint4v_ __attribute__((ext_vector_type(4)));
+            const uint4v_ bits = __builtin_bit_cast(uint4v_, out);
+            half_t *at = dst + c16;
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+              asm volatile("global_atomic_pk_add_f16 %0, %1, off offset:%2" ::"v"(at), "v"(bits[u]), "n"(4 * u) : "memory");
+          }
+        } else {
+          if (real && c16 < p.N) *reinterpret_cast<half8 *>(dst + c16) = out;
+        }
       }
     } else if (real) {
       half_t *row2 = p.C2 + static_cast<size_t>(j) * p.N;           // epilogues 2 and 3 only
@@ -850,13 +866,14 @@ int g_split_tail = 1;        // 0: the last round of tiles is not cut along K
 constexpr int kSplitTailMinKT = 64;
 int g_split_tail_min_kt = kSplitTailMinKT;
 int g_split_max_parts = 8;
+int g_fused_combine = 0;     // 1: top-2 layers add the gate-weighted expert outputs in the second GEMM's epilogue
 int g_skinny_pct = 70;       // a K step of a skinny tile in percent of a 256-row tile's (plan model); 0: no skinny tiles
 
 // The tuning knobs a grouped GEMM's plan and launches depend on, read once per call: the plan
 // and the kernels that consume it must agree even if another thread calls ccf_set_option
 // between the routing stage (which builds the plans of the layer's forward call) and the GEMMs.
 GemmOptions current_options() {
-  return GemmOptions{g_variant, g_split_tail, g_split_tail_min_kt, g_split_max_parts, g_skinny_pct};
+  return GemmOptions{g_variant, g_split_tail, g_split_tail_min_kt, g_split_max_parts, g_skinny_pct, g_fused_combine};
 }
 
 struct Launch {
@@ -884,8 +901,11 @@ const Launch kVariants[] = {CCF_VARIANT(Cfg0), CCF_VARIANT(Cfg1), CCF_VARIANT(Cf
                             // pre-activation, "gelu" slot = input gradient through the GELU; not selectable
                             {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiGeluKeep>,
                              grouped_gemm_kernel<Cfg5, kEpiGeluGrad>, grouped_gemm_persistent_kernel<Cfg5, kEpiGeluKeep>,
-                             grouped_gemm_persistent_kernel<Cfg5, kEpiGeluGrad>}};
-constexpr int kKnVariant = 7, kTrainVariant = 8;
+                             grouped_gemm_persistent_kernel<Cfg5, kEpiGeluGrad>},
+                            // the combine epilogue ("plain" slot); not selectable
+                            {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiCombine>, nullptr,
+                             grouped_gemm_persistent_kernel<Cfg5, kEpiCombine>, nullptr}};
+constexpr int kKnVariant = 7, kTrainVariant = 8, kCombineVariant = 9;
 #undef CCF_VARIANT
 #undef CCF_VARIANT_P
 
@@ -955,11 +975,11 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
     g.tail = reinterpret_cast<int32_t *>(ws + plan_bytes(max_rows, E, N > K ? N : K));
     g.plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.tail) + kTailHead);
   }
-  const bool gelu = epi != kEpiPlain;
-  g.v = &kVariants[b_kn ? kKnVariant : (epi >= kEpiGeluKeep ? kTrainVariant : opt.variant)];
+  const bool gelu = epi != kEpiPlain && epi != kEpiCombine;
+  g.v = &kVariants[b_kn ? kKnVariant : (epi == kEpiCombine ? kCombineVariant : (epi >= kEpiGeluKeep ? kTrainVariant : opt.variant))];
   const Launch &v = *g.v;
   // which of the entry's two kernels: the K-N and training entries hold the GELU-gradient form in the second slot
-  g.second = b_kn ? epi == kEpiGeluGrad : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu);
+  g.second = b_kn ? epi == kEpiGeluGrad : (epi == kEpiCombine ? false : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu));
   const int max_tiles = max_tiles_for(max_rows, E, v.bm);
   const int n_tiles_n = (N + v.bn - 1) / v.bn;
   g.wgs = launched_wgs(max_tiles, n_tiles_n);                   // worst-case tile count
@@ -984,11 +1004,14 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
                  int N, int K, const half_t *B, const half_t *bias, int epi, half_t *C,
                  const int32_t *c_rows, const half_t *row_scale, void *workspace, hipStream_t stream,
                  const char *what, bool b_kn = false, half_t *C2 = nullptr, int region = 0,
-                 bool plan_ready = false, const GemmOptions *opt = nullptr) {
+                 bool plan_ready = false, const GemmOptions *opt = nullptr, const int32_t *scale_rows = nullptr) {
   CCF_REQUIRE(A && offsets && B && C && workspace, CCF_ERR_ARG, "%s: null pointer", what);
-  const bool gelu = epi != kEpiPlain;
-  CCF_REQUIRE(epi >= kEpiPlain && epi <= kEpiGeluGrad && (epi < kEpiGeluKeep || (C2 && aligned16(C2))), CCF_ERR_ARG,
+  const bool gelu = epi != kEpiPlain && epi != kEpiCombine;
+  CCF_REQUIRE(epi >= kEpiPlain && epi <= kEpiCombine &&
+                  (epi < kEpiGeluKeep || epi == kEpiCombine || (C2 && aligned16(C2))), CCF_ERR_ARG,
               "%s: epilogue %d needs the pre-activation buffer", what, epi);
+  CCF_REQUIRE(epi != kEpiCombine || (c_rows && row_scale && scale_rows && !b_kn && N % 8 == 0), CCF_ERR_ARG,
+              "%s: the combine epilogue needs token rows, scores and their index", what);
   // b_kn: B is [E, K, N] (the stored weight of the layer whose input gradient this is); Cfg5 kernels only
   CCF_REQUIRE(!b_kn || (N % Cfg5::BN == 0 && (epi == kEpiPlain || epi == kEpiGeluGrad) &&
                         static_cast<long long>(K) * N < (1ll << 31)), CCF_ERR_SHAPE,
@@ -1022,6 +1045,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.C2 = C2;
   p.c_rows = c_rows;
   p.row_scale = row_scale;
+  p.scale_rows = scale_rows;
   p.plan = plan;
   p.N = N;
   p.K = K;
@@ -1079,6 +1103,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.C2 = nullptr;
   p.c_rows = nullptr;
   p.row_scale = nullptr;
+  p.scale_rows = nullptr;
   p.plan = plan;
   p.N = N;
   p.K = 0;
@@ -1234,6 +1259,16 @@ extern "C" int ccf_set_option(const char *name, int value) {
     g_gate_waves = value;
     return CCF_OK;
   }
+  if (!strcmp(name, "fused_combine")) {
+    g_fused_combine = value != 0;
+    return CCF_OK;
+  }
+  if (!strcmp(name, "gate_tokens")) {
+    CCF_REQUIRE(value == 0 || value == 1 || value == 2 || value == 4, CCF_ERR_ARG,
+                "set_option: gate_tokens %d is none of 0, 1, 2, 4", value);
+    g_gate_tt = value;
+    return CCF_OK;
+  }
   return fail(CCF_ERR_ARG, "set_option: unknown option %s", name);
 }
 
@@ -1244,7 +1279,8 @@ extern "C" size_t ccf_ffn_workspace_bytes(int max_rows, int num_expert, int d_mo
 
 namespace ccf {
 
-// Plan requests of the layer's two forward GEMMs (which = 1: FFN1 with GELU, 2: FFN2), for a
+// Plan requests of the layer's two forward GEMMs (which = 1: FFN1 with GELU, 2: FFN2, 3: FFN2 with the
+// combine epilogue), for a
 // caller that builds the plans itself (the routing stage does) and then passes plan_ready.
 // False when the sizes are not ones the GEMM accepts: the caller then leaves the plan to it.
 GemmOptions forward_options() { return current_options(); }
@@ -1253,8 +1289,8 @@ bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *wo
                           PlanReq *out) {
   if (!workspace || max_rows <= 0 || E <= 0 || E > 1024 || d <= 0 || f <= 0 || d % 64 || f % 64) return false;
   const int N = which == 1 ? f : d, K = which == 1 ? d : f;
-  const GemmSetup gs = setup_gemm(max_rows, E, N, K, which == 1 ? kEpiGelu : kEpiPlain, false, workspace,
-                                  which == 1 ? 0 : 1, opt);
+  const GemmSetup gs = setup_gemm(max_rows, E, N, K, which == 1 ? kEpiGelu : (which == 3 ? kEpiCombine : kEpiPlain),
+                                  false, workspace, which == 1 ? 0 : 1, opt);
   if (gs.wgs >= (1ll << 31)) return false;
   *out = gs.req;
   return true;
@@ -1286,6 +1322,21 @@ int ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row, 
                       d_ffn, static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), kEpiPlain,
                       static_cast<half_t *>(y), dst_row, static_cast<const half_t *>(row_scale),
                       workspace, stream, "ffn2", false, nullptr, 1, plan_ready, planned);
+}
+
+// FFN2 with the combine in its epilogue: out[token_row[j]] += (h[j] * w2[e]^T + b2[e]) * score[flat_row[j]].
+// `out` must be zero; two addends per token make the result independent of their order.
+int ffn2_forward_combine(const void *h, const int32_t *token_row, const int32_t *flat_row, const int32_t *offsets,
+                         int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
+                         const void *score, void *out, void *workspace, size_t workspace_bytes, hipStream_t stream,
+                         const GemmOptions *planned) {
+  const size_t need = ccf_ffn_workspace_bytes(max_rows, num_expert, d_model, d_ffn);
+  CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
+              "ffn2: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  return grouped_gemm(static_cast<const half_t *>(h), nullptr, offsets, max_rows, num_expert, d_model, d_ffn,
+                      static_cast<const half_t *>(w2), static_cast<const half_t *>(b2), kEpiCombine,
+                      static_cast<half_t *>(out), token_row, static_cast<const half_t *>(score), workspace, stream,
+                      "ffn2 with combine", false, nullptr, 1, planned != nullptr, planned, flat_row);
 }
 
 }  // namespace ccf

@@ -20,6 +20,7 @@
 
 namespace ccf {
 int g_gate_waves = 16;   // wavefronts per gate workgroup when the weights sit in LDS; 4 forces the small one
+int g_gate_tt = 0;       // tokens a wavefront scores at a time (1, 2 or 4); 0 = by the token count
 namespace {
 
 constexpr int kMaxTopK = 8;
@@ -313,7 +314,7 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
   CCF_REQUIRE(aligned16(x) && aligned16(wg), CCF_ERR_ARG, "gate: x and wg must be 16-byte aligned");
   if (tokens == 0) return CCF_OK;
   // Enough wavefronts to hide HBM latency: fewer tokens per wavefront when the batch is small.
-  const int tt = tokens >= 32768 ? 4 : (tokens >= 8192 ? 2 : 1);
+  const int tt = g_gate_tt ? g_gate_tt : (tokens >= 32768 ? 4 : (tokens >= 8192 ? 2 : 1));
   const size_t esz = dtype == CCF_F16 ? 2 : 4;
   // the kernel always stages kGateEG weight rows (rows past the last expert repeat it)
   const size_t w_bytes = static_cast<size_t>(kGateEG) * d_model * esz;

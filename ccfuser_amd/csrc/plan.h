@@ -337,7 +337,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
 // ffn.hip
 // Snapshot of the tuning knobs (ccf_set_option) that a grouped GEMM's plan and launches depend on.
 struct GemmOptions {
-  int variant, split_tail, split_tail_min_kt, split_max_parts, skinny_pct;
+  int variant, split_tail, split_tail_min_kt, split_max_parts, skinny_pct, fused_combine;
 };
 GemmOptions forward_options();
 bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, const GemmOptions &opt,
@@ -350,6 +350,10 @@ int ffn2_forward(const void *h, const int32_t *src_row, const int32_t *dst_row, 
                  int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
                  const void *row_scale, void *y, void *workspace, size_t workspace_bytes,
                  hipStream_t stream, const GemmOptions *planned);
+int ffn2_forward_combine(const void *h, const int32_t *token_row, const int32_t *flat_row, const int32_t *offsets,
+                         int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
+                         const void *score, void *out, void *workspace, size_t workspace_bytes, hipStream_t stream,
+                         const GemmOptions *planned);
 // route.hip: ccf_route(), whose last launch also builds n_plans (0..2) tile plans from the offsets
 int route_with_plans(const int64_t *gate_idx, int n_flat, int num_expert, int top_k, int capacity,
                      int32_t *counts, int32_t *offsets, int64_t *pos, int32_t *src_row, int32_t *dst_row,

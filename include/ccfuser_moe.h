@@ -64,6 +64,10 @@ const char *ccf_last_error(void);
  *                     cost model says that beats a padded 256-row tile; n > 1 sets the model's cost of
  *                     such a tile's K step in percent of a 256-row tile's (default 70); -n (1..4) forces
  *                     them with n workgroups per XCD
+ *   "fused_combine"   0/1 (default 0): ccf_moe_forward with top_k = 2 adds the gate-weighted expert outputs
+ *                     into the output in the second GEMM's epilogue (packed fp16 atomic adds onto zeros)
+ *                     instead of running the combine pass; measured slower, kept for comparison
+ *   "gate_tokens"     0, 1, 2 or 4: tokens a gate wavefront scores at a time (0 = chosen by the token count)
  *   "dgrad_transpose" 0/1: the backward's input-gradient GEMM runs on a transposed copy of the
  *                     weight instead of reading the stored one
  *   "gate_waves"      4 or 16: cap on the gate kernel's wavefronts per workgroup

@@ -350,6 +350,34 @@ def test_full_size_ep_share_segments(workloads):
     assert torch.equal(y, ops.moe_ffn_segments(*args))
 
 
+def test_combine_in_the_second_gemm_epilogue(workloads):
+    """Option "fused_combine": for top-2 the second GEMM's epilogue adds score * y into the
+    zero-filled output with packed fp16 atomic adds instead of writing y_flat for a combine
+    pass (off by default: measured slower).  Two addends onto zero commute, so the result is
+    deterministic; it must meet the oracle's tolerance, with capacity drops too."""
+    from ccfuser_amd import ops
+    wl = workloads("c2_gshard", 1024)
+    t = dict(wl.tensors)
+    bg = t["bg"].clone().float()
+    bg[2] += 0.6                                   # expert 2 overflows its capacity: dropped slots add nothing
+    t["bg"] = bg.half()
+    names = ("x", "wg", "bg", "w1", "b1", "w2", "b2")
+    ref = O.moe_layer_forward(*[t[n] for n in names], wl.top_k, capacity=wl.capacity)
+    assert int((ref["idx_kept"] < 0).sum()) > 0
+    args = [t[n].cuda() for n in names]
+    _say(f"fused combine T={wl.tokens}")
+    ops.set_option("fused_combine", 1)
+    try:
+        a = ops.moe_forward(*args, wl.top_k, wl.capacity)
+        b = ops.moe_forward(*args, wl.top_k, wl.capacity)
+    finally:
+        ops.set_option("fused_combine", 0)
+    assert torch.equal(a, b)
+    assert O.max_abs_err(a.cpu(), ref["out"]) <= MAX_ABS and O.mean_rel_err(a.cpu(), ref["out"]) <= MEAN_REL
+    plain = ops.moe_forward(*args, wl.top_k, wl.capacity)
+    assert O.max_abs_err(a.cpu(), plain.float().cpu()) <= 4e-3
+
+
 def test_forward_replays_from_a_hip_graph(workloads):
     """The whole-layer call allocates nothing and never synchronises, so it can be captured
     into a HIP graph.  Replayed several times with fresh inputs, with eager work and
