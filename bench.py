@@ -90,6 +90,36 @@ def dense_hgemm_ceiling(rows, d, f, steps=30, warmup=15):
     return out
 
 
+def mfma_only_ceiling(lib, seconds=0.15):
+    """What the matrix cores sustain with nothing else in the way (ccf_probe_mfma: one workgroup
+    per CU, MFMAs on register operands, no memory traffic), with random and with constant
+    operands: each launch repeated until `seconds` have passed, the last launches timed."""
+    import ctypes as C
+    import torch
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.empty(cus * 256, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {}
+    for name, const in (("random_operands", 0), ("constant_operands", 1)):
+        flop = C.c_double()
+        iters = 2000                                              # ~2 ms per launch
+        t_end = time.perf_counter() + seconds
+        while time.perf_counter() < t_end:                        # lets the clock settle under this load
+            lib.ccf_probe_mfma(cus, iters, const, out.data_ptr(), C.byref(flop), stream)
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            lib.ccf_probe_mfma(cus, iters, const, out.data_ptr(), C.byref(flop), stream)
+        e1.record()
+        torch.cuda.synchronize()
+        tf = 10 * flop.value / (e0.elapsed_time(e1) * 1e-3) / 1e12
+        res[name] = {"tflops": tf, "frac_of_peak": tf / PEAK_FP16_TFLOPS}
+    res["what"] = (f"v_mfma_f32_16x16x32_f16 back to back on register operands, {cus} workgroups of 4 wavefronts, "
+                   "no memory traffic")
+    return res
+
+
 class HipEvents:
     """hipEvent_t handles through the HIP runtime (torch's events hide the handle)."""
 
@@ -248,7 +278,7 @@ def main():
                     help="ccf_set_option before the run (tuning knobs), may repeat")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense-ceiling", action="store_true",
-                    help="skip the vendor dense-GEMM measurement on the workload's GEMM shapes")
+                    help="skip the measured ceilings (vendor dense GEMM on the workload's shapes, MFMA-only loop)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (a known HBM traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -382,6 +412,9 @@ def main():
         ceil = dense_hgemm_ceiling(routed, d, f)
         line["dense_hgemm_ceiling"] = ceil
         line["roofline"]["frac_of_dense_hgemm_ceiling"] = ach / ceil[f"{dom}_shape"]["tflops"]
+        mf = mfma_only_ceiling(lib)
+        line["mfma_only_ceiling"] = mf
+        line["roofline"]["frac_of_mfma_only_random_operands"] = ach / mf["random_operands"]["tflops"]
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(line))

@@ -16,7 +16,7 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIB = HERE / "libccfuser_moe.so"
-SOURCES = ["api.hip", "gate.hip", "route.hip", "rows.hip", "bwd.hip", "ffn.hip"]
+SOURCES = ["api.hip", "gate.hip", "route.hip", "rows.hip", "bwd.hip", "ffn.hip", "probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = [
@@ -30,6 +30,7 @@ PER_FILE = {
     "gate.hip": ["-ffp-contract=off"],
     # the 16x16x32 main loop names its accumulation registers itself: nothing of the compiler's may live there
     "ffn.hip": ["-mllvm", "-amdgpu-spill-vgpr-to-agpr=0"],
+    "probe.hip": ["-mllvm", "-amdgpu-spill-vgpr-to-agpr=0"],
 }
 
 

@@ -295,6 +295,17 @@ int ccf_moe_forward(const void *x, const void *wg, const void *bg,
  */
 int ccf_moe_forward_set_events(void *const *events, int count);
 
+/*
+ * Measurement probe (no counterpart in the reference): `workgroups` workgroups of four
+ * wavefronts issue `iters` x 64 v_mfma_f32_16x16x32_f16 each on register operands, constant
+ * (zeros) or pseudo-random, with no memory traffic; *flop receives the flop count of the launch.
+ * Timed with events by the caller it gives the rate the matrix cores sustain: the nominal peak
+ * with constant operands, a lower, power-limited figure with random ones.
+ *   out: device buffer of workgroups * 256 floats (sums that keep the loop alive).
+ */
+int ccf_probe_mfma(int workgroups, int iters, int constant_operands, void *out, double *flop,
+                   ccf_stream_t stream);
+
 /* Bytes of workspace ccf_moe_ffn_segments needs. */
 size_t ccf_segments_workspace_bytes(int total_rows, int n_seg, int num_expert,
                                     int d_model, int d_ffn);

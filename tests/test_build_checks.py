@@ -36,3 +36,25 @@ def test_no_compiler_values_in_accumulation_registers(tmp_path):
         assert not stray, (name, stray[:5])
         assert "scratch_" not in body, name
         assert body.count("v_mfma_f32_16x16x32_f16") >= 128, name
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not Path("/opt/rocm/bin/hipcc").exists(),
+                    reason="hipcc not available")
+def test_probe_kernel_keeps_the_accumulation_registers_to_itself(tmp_path):
+    """The MFMA-only probe names all 256 accumulation registers in inline asm too: the compiler
+    must hold nothing of its own there (a value parked in one would be overwritten: it was the
+    index of the kernel's only store once), and must not spill."""
+    from ccfuser_amd import build as B
+    out = tmp_path / "probe.s"
+    cmd = [B.HIPCC, *B.COMMON, *B.PER_FILE.get("probe.hip", []), "-S", "--cuda-device-only",
+           str(B.CSRC / "probe.hip"), "-o", str(out)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    text = out.read_text()
+    m = re.search(r"^(_ZN3ccf\S*mfma_probe_kernel\S*):[^\n]*\n(.*?)s_endpgm", text, flags=re.S | re.M)
+    assert m
+    body = m.group(2)
+    stray = re.findall(r"^\s*(v_accvgpr_(?:write_b32 a\d+, v\d+|read_b32 v\d+, a\d+|mov_b32 .*))$", body, flags=re.M)
+    assert not stray, stray[:5]
+    assert "scratch_" not in body
+    assert body.count("v_mfma_f32_16x16x32_f16") == 64

@@ -448,3 +448,23 @@ def test_skinny_tiles(R, d, f, E, skew, seed, mode):
     same = [torch.equal(a, b) for a, b in zip(res[mode], res[0])]
     _say(f"  skinny on/off bitwise equal (h, act, pre, y): {same}")
     assert all(same)
+
+
+def test_mfma_probe_runs_and_counts_its_flop():
+    """ccf_probe_mfma: the MFMA-only loop bench.py times for its measured ceiling.  With zero
+    operands every sum it leaves is zero; the flop count is the closed form."""
+    import ctypes as C
+    from ccfuser_amd import _lib
+    lib = _lib.lib()
+    wgs, iters = 16, 10
+    out = torch.full((wgs * 256,), 7.0, dtype=torch.float32, device="cuda")
+    flop = C.c_double()
+    for const in (1, 0):
+        _lib.call("ccf_probe_mfma", wgs, iters, const, out.data_ptr(), C.byref(flop), None)
+        torch.cuda.synchronize()
+        assert flop.value == wgs * 4 * iters * 64 * 16 * 16 * 32 * 2
+        assert bool(torch.isfinite(out).all())
+        if const:
+            assert not out.any()
+    with pytest.raises(_lib.CcfError):
+        _lib.call("ccf_probe_mfma", 0, iters, 1, out.data_ptr(), C.byref(flop), None)
