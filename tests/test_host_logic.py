@@ -86,3 +86,17 @@ def test_functions_refuse_multi_gpu():
         functions.count_by_gate(torch.zeros(4, dtype=torch.long), 2, 2, 0)
     with pytest.raises(RuntimeError):
         functions.ensure_comm(torch.zeros(1), object())
+
+
+def test_integration_guide_constructor_example_is_valid():
+    """The constructor call INTEGRATION.md shows for replacing the layer (the reference's
+    positional order, transformer.py:435-461) must be accepted as written."""
+    import os
+    import re
+    from ccfuser_amd.mix_moe import MixMOETransformerMLP
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "INTEGRATION.md")).read()
+    m = re.search(r"mlp = (MixMOETransformerMLP\(.*?\))\.cuda\(\)", text, flags=re.S)
+    assert m, "the guide no longer shows the constructor call"
+    mlp = eval(m.group(1), {"MixMOETransformerMLP": MixMOETransformerMLP})
+    assert mlp.experts.htoh4.weight.shape[1:] == (14336, 4096) and mlp.top_k == 2
