@@ -52,7 +52,7 @@ int launch_bias_reduce(const float *partial, const int32_t *k_seg, int E, int C,
                        hipStream_t stream);
 
 // tuning knobs set through ccf_set_option()
-extern int g_gate_waves, g_gate_tt;   // gate.hip
+extern int g_gate_waves, g_gate_slots;   // gate.hip
 
 }  // namespace ccf
 

@@ -1255,7 +1255,7 @@ extern "C" int ccf_set_option(const char *name, int value) {
     return CCF_OK;
   }
   if (!strcmp(name, "gate_waves")) {
-    CCF_REQUIRE(value == 4 || value == 16, CCF_ERR_ARG, "set_option: gate_waves %d is neither 4 nor 16", value);
+    CCF_REQUIRE(value >= 1 && value <= 8, CCF_ERR_ARG, "set_option: gate_waves %d outside 1..8", value);
     g_gate_waves = value;
     return CCF_OK;
   }
@@ -1263,10 +1263,10 @@ extern "C" int ccf_set_option(const char *name, int value) {
     g_fused_combine = value != 0;
     return CCF_OK;
   }
-  if (!strcmp(name, "gate_tokens")) {
+  if (!strcmp(name, "gate_slots")) {
     CCF_REQUIRE(value == 0 || value == 1 || value == 2 || value == 4, CCF_ERR_ARG,
-                "set_option: gate_tokens %d is none of 0, 1, 2, 4", value);
-    g_gate_tt = value;
+                "set_option: gate_slots %d is none of 0, 1, 2, 4", value);
+    g_gate_slots = value;
     return CCF_OK;
   }
   return fail(CCF_ERR_ARG, "set_option: unknown option %s", name);

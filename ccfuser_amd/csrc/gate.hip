@@ -4,67 +4,37 @@
 // over the k selected logits (reference mix_moe/mix_moe/gates/naive_gate.py:31-38).
 //
 // The expert choice has to be reproducible bit for bit, so the fp32 sum is
-// taken in one fixed order that a CPU can replay: K is cut into chunks of 8;
-// lane l of a 64-lane wavefront owns chunks l, l+64, ... and adds their
-// products one element at a time; the 64 partial sums are folded by an xor
-// butterfly (32, 16, 8, 4, 2, 1); the bias is added last and the logit is
-// rounded once to the input dtype.  Multiplies and adds are kept separate
-// (contraction off), which changes nothing for fp16 inputs, whose products are
-// exact in fp32, and keeps fp32 inputs replayable without a fused multiply-add.
+// taken in one fixed order that a CPU can replay: K is cut into parts of 128
+// consecutive elements (the last may be shorter); a part's sum starts at zero
+// and takes its products one at a time in ascending K, acc = fma(x, w, acc);
+// the part sums are added one after the other in ascending order, starting from
+// the first; the bias is added last and the logit is rounded once to the input
+// dtype.  The product of two fp16 values is exact in fp32, so for fp16 inputs
+// the fused multiply-add is one rounding of acc + x*w however it is computed.
 //
-// One wavefront scores TT tokens at a time so that each 16-byte piece of wg it
-// reads feeds TT*8 multiply-adds; x is read from HBM once, wg comes from cache.
+// That chain is what a K = 1 fp32 MFMA computes per output element
+// (D = fma(A, B, C), round to nearest even: checked against fmaf chains on a
+// CPU), so for fp16 inputs a wavefront runs it for a whole tile of tokens x
+// experts at once: v_mfma_f32_32x32x1 (two 32 x 32 blocks) for more than 16
+// experts, v_mfma_f32_16x16x1 (four 16 x 16 blocks) otherwise, one instruction
+// per K element.  The blocks of an instruction are independent products, so a
+// block is either another group of tokens or the same tokens on another part
+// of K ("slot"): few tokens still fill the machine.  fp32 inputs keep multiply
+// and add separate (two roundings) and run on the vector unit.
 #include "ccf_common.h"
 
 #include <limits.h>
 
 namespace ccf {
-int g_gate_waves = 16;   // wavefronts per gate workgroup when the weights sit in LDS; 4 forces the small one
-int g_gate_tt = 0;       // tokens a wavefront scores at a time (1, 2 or 4); 0 = by the token count
+int g_gate_waves = 8;    // most wavefronts of a gate workgroup (each takes other parts of K), 1..8
+int g_gate_slots = 0;    // parts of K a wavefront works on at a time (1, 2, 4); 0 = by the token count
 namespace {
 
 constexpr int kMaxTopK = 8;
-constexpr int kGateEG = 8;   // experts accumulated per pass over x
+constexpr int kPart = 128;          // K elements of a part
+constexpr int kMaxWaves = 8;
 
-// Eight consecutive K elements as loaded, and acc += x[j] * w[j] for j = 0..7 in
-// order.  For fp16 the product is exact in fp32, so a fused multiply-add on the
-// fp16 operands (v_fma_mix_f32, no conversions) gives the same bits as a
-// multiply followed by an add; for fp32 the two stay separate.
-template <typename T>
-struct Chunk;
-
-template <>
-struct Chunk<half_t> {
-  half8 v;
-  __device__ inline void load(const half_t *p) { v = *reinterpret_cast<const half8 *>(p); }
-  __device__ inline void mac(const Chunk &w, float &acc) const {
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      acc = __builtin_fmaf(static_cast<float>(v[j]), static_cast<float>(w.v[j]), acc);
-  }
-};
-
-template <>
-struct Chunk<float> {
-  float4v lo, hi;
-  __device__ inline void load(const float *p) {
-    lo = reinterpret_cast<const float4v *>(p)[0];
-    hi = reinterpret_cast<const float4v *>(p)[1];
-  }
-  __device__ inline void mac(const Chunk &w, float &acc) const {
-#pragma clang fp contract(off)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float p = lo[j] * w.lo[j];
-      acc = acc + p;
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float p = hi[j] * w.hi[j];
-      acc = acc + p;
-    }
-  }
-};
+typedef float float32v __attribute__((ext_vector_type(32)));
 
 template <typename T>
 __device__ inline float round_to(float v) {
@@ -75,224 +45,359 @@ __device__ inline bool better(float v, int id, float bv, int bid) {
   return v > bv || (v == bv && id < bid);
 }
 
-// One level of the lane fold (see gate_kernel): LIVE values remain, partner lane
-// is lane ^ OFF.  Everything is resolved at compile time so v stays in registers.
-template <int LIVE, int OFF, int N>
-__device__ inline void fold_level(float (&v)[N], int lane) {
-  if constexpr (OFF >= 1) {
-    if constexpr (LIVE > 1) {
-      constexpr int HALF = LIVE / 2;
-      const bool upper = (lane & OFF) != 0;
+// The k best of a token so far (k <= KS), best first; ties keep the lower expert id.
+template <int KS>
+struct Best {
+  float v[KS];
+  int id[KS];
+  __device__ inline void clear() {
 #pragma unroll
-      for (int j = 0; j < HALF; ++j) {
-        const float keep = upper ? v[j + HALF] : v[j];
-        const float send = upper ? v[j] : v[j + HALF];
-        v[j] = keep + __shfl_xor(send, OFF, kWave);
-      }
-      fold_level<HALF, OFF / 2, N>(v, lane);
-    } else {
-      v[0] = v[0] + __shfl_xor(v[0], OFF, kWave);
-      fold_level<1, OFF / 2, N>(v, lane);
+    for (int s = 0; s < KS; ++s) {
+      v[s] = -INFINITY;
+      id[s] = INT_MAX;
     }
   }
-}
+  __device__ inline void offer(float nv, int nid, int k) {
+    float lv = v[0];
+    int li = id[0];
+#pragma unroll
+    for (int s = 1; s < KS; ++s)
+      if (s == k - 1) {
+        lv = v[s];
+        li = id[s];
+      }
+    if (!better(nv, nid, lv, li)) return;          // not among the k best
+#pragma unroll
+    for (int s = KS - 1; s >= 0; --s) {
+      if (s < k) {
+        const int up = s > 0 ? s - 1 : 0;
+        const bool ahead = s > 0 && better(nv, nid, v[up], id[up]);
+        const bool here = better(nv, nid, v[s], id[s]);
+        if (ahead) {                               // belongs further up: slot s takes its upper neighbour
+          v[s] = v[up];
+          id[s] = id[up];
+        } else if (here) {
+          v[s] = nv;
+          id[s] = nid;
+        }
+      }
+    }
+  }
+  // softmax over the k selected logits (slot 0 holds the maximum) and the writes
+  template <typename T>
+  __device__ inline void write(int t, int k, int64_t *__restrict__ idx_out, T *__restrict__ score_out) const {
+    float ex[KS];
+    float sum = 0.0f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      ex[s] = (s < k) ? expf(v[s] - v[0]) : 0.0f;
+      sum += ex[s];
+    }
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      if (s < k) {
+        idx_out[static_cast<size_t>(t) * k + s] = static_cast<int64_t>(id[s]);
+        score_out[static_cast<size_t>(t) * k + s] = static_cast<T>(ex[s] / sum);
+      }
+    }
+  }
+};
 
-template <int N, int OFF>
-__device__ inline void fold_lanes(float (&v)[N], int lane) {
-  fold_level<N, OFF, N>(v, lane);
-}
+template <int N>
+struct Mfma;
 
-// Workgroups are persistent: each stages an expert group's weight rows in LDS
-// once (when they fit, kWLds) and then walks over its share of the tokens, one
-// wavefront scoring TT tokens at a time.  The x chunks of up to kBatch passes
-// are requested together before any arithmetic (one memory round trip for
-// d_model <= 4096).  Logits of all experts are parked in LDS until the last
-// expert group is done, then each wavefront picks the top-k of its tokens.
-// None of this changes the order of the additions.
-template <typename T, int TT, bool kWLds, int GW>
-__global__ void __launch_bounds__(GW * 64)
-gate_kernel(const T *__restrict__ x, const T *__restrict__ wg, const T *__restrict__ bg,
-            int tokens, int d, int E, int k, int groups_per_block, int64_t *__restrict__ idx_out,
-            T *__restrict__ score_out, T *__restrict__ logits_out) {
-#pragma clang fp contract(off)
-  constexpr int kBatch = 8 / TT;                   // x chunks requested together per lane
-  extern __shared__ float s_logit[];               // [groups_per_block][GW wavefronts][TT][E], then weights
+template <>
+struct Mfma<32> {
+  typedef float32v Acc;
+  static constexpr int kRegs = 32;
+  __device__ static inline Acc run(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_32x32x1f32(a, b, c, 0, 0, 0);
+  }
+  // accumulator register v of a lane: block and row of that output element (column = lane % 32)
+  __device__ static constexpr int block(int v) { return v >> 4; }
+  __device__ static inline int row(int v, int lane) { return 8 * ((v & 15) >> 2) + 4 * (lane >> 5) + (v & 3); }
+};
+
+template <>
+struct Mfma<16> {
+  typedef float16v Acc;
+  static constexpr int kRegs = 16;
+  __device__ static inline Acc run(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, c, 0, 0, 0);
+  }
+  __device__ static constexpr int block(int v) { return v >> 2; }
+  __device__ static inline int row(int v, int lane) { return 4 * (lane >> 4) + (v & 3); }
+};
+
+// fp16 gate.  An MFMA has 64 / N blocks; with S = 1 << LS slots, block b of a wavefront is
+// token block b / S on slot b % S, so a wavefront covers TW = (64 / N / S) * N tokens and
+// S parts of K at a time, and the wavefronts of a workgroup (all on the same TW tokens)
+// cover waves * S parts per round.  Lane l of block b feeds row l % N of A with its
+// token's x and column l % N of B with its expert's weights, zero where K, the tokens or
+// the experts end (fma(0, 0, acc) = acc).
+//
+// A lane needs consecutive K of its own row, which is the opposite of a coalesced load, so
+// the operands take the way through LDS: per stage of 32 K elements the wavefront fetches
+// the 64 bytes of each of its 64 x rows and of its N*S weight rows with whole-line loads
+// (four lanes per row), two stages ahead of their use, parks them in registers, and writes
+// them into its own 10 KB of LDS one stage ahead; each lane then reads its row back in
+// 16-byte pieces.  Only that wavefront touches the region, so the stage loop has no barrier.
+//
+// After a round the part sums wait in LDS (the same region) and are added in ascending part
+// order onto the running sums; after the last round bias and rounding give the logits of one
+// tile of N experts, of which one thread per token keeps the k best (k <= KS).
+constexpr int kStageK = 32;                        // K elements of a stage
+constexpr int kRowBytes = 80;                      // a row's 64 bytes of a stage + 16: bank spread
+constexpr int kTileBytes = 64 * kRowBytes;         // one operand of a stage
+constexpr int kRegionFloats = 2 * kTileBytes / 4;  // a wavefront's LDS: two operand tiles, later its part sums
+
+template <int N, int LS, int KS>
+__global__ void __launch_bounds__(kMaxWaves * 64)
+gate_mfma_kernel(const half_t *__restrict__ x, const half_t *__restrict__ wg, const half_t *__restrict__ bg,
+                 int tokens, int d, int E, int k, int64_t *__restrict__ idx_out,
+                 half_t *__restrict__ score_out, half_t *__restrict__ logits_out) {
+  using M = Mfma<N>;
+  constexpr int kBlocks = 64 / N;
+  constexpr int S = 1 << LS;
+  static_assert(S <= kBlocks, "a slot is a block");
+  constexpr int TW = (kBlocks / S) * N;            // tokens of a workgroup
+  constexpr int kWLoads = N * S / 16;              // load instructions for the weight rows of a stage
+  constexpr int kLd = N + 1;                       // row stride of the logit tile in LDS (bank spread)
+  static_assert(64 * N * 4 <= kRegionFloats * 4, "part sums of a wavefront fit its region");
+  extern __shared__ float s_mem[];
+  const int waves = blockDim.x >> 6;
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
-  const int nchunk = d >> 3;
-  const int niter = (nchunk + kWave - 1) / kWave;
-  const int n_groups = (tokens + GW * TT - 1) / (GW * TT);
-  T *w_lds = reinterpret_cast<T *>(s_logit + static_cast<size_t>(groups_per_block) * GW * TT * E);
+  float *region = s_mem + static_cast<size_t>(wave) * kRegionFloats;
+  float *s_total = s_mem + static_cast<size_t>(waves) * kRegionFloats;   // [TW][kLd] running sums, then logits
+  const int t0 = blockIdx.x * TW;
+  const int nparts = (d + kPart - 1) / kPart;
+  const int per_round = waves * S;
+  const int rounds = (nparts + per_round - 1) / per_round;
 
-  for (int e0 = 0; e0 < E; e0 += kGateEG) {
-    const int ng = (E - e0) < kGateEG ? (E - e0) : kGateEG;
-    if (kWLds) {
-      __syncthreads();                             // previous group fully consumed
-      // always kGateEG rows (rows past E repeat the last expert and are discarded),
-      // 16-byte pieces, 8 loads in flight per lane
-      const int per_row = static_cast<int>(static_cast<size_t>(d) * sizeof(T) / 16);
-      const int total = kGateEG * per_row;
-      int4v *dst = reinterpret_cast<int4v *>(w_lds);
-      for (int i0 = threadIdx.x; i0 < total; i0 += GW * 64 * 8) {
-        int4v tmp[8];
+  // as a reader: my block, row, slot
+  const int blk = lane / N, r = lane % N;
+  const int slot = blk & (S - 1);
+  char *tile = reinterpret_cast<char *>(region);
+  const char *my_x = tile + lane * kRowBytes;                              // x row of lane l is row l of the tile
+  const char *my_w = tile + kTileBytes + (slot * N + r) * kRowBytes;       // weight rows: slot-major
+
+  // as a loader: four lanes per row, 16 rows per instruction
+  const int l_row = lane >> 2, l_piece = lane & 3;
+  char *park_at = tile + l_row * kRowBytes + l_piece * 16;
+  const half_t *x_src[4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int i = i0 + u * GW * 64;
-          if (i < total) {
-            int row = e0 + i / per_row;
-            row = row < E ? row : E - 1;
-            tmp[u] = reinterpret_cast<const int4v *>(wg + static_cast<size_t>(row) * d)[i % per_row];
+  for (int i = 0; i < 4; ++i) {
+    const int lr = 16 * i + l_row;
+    int t = t0 + ((lr / N) >> LS) * N + lr % N;
+    t = t < tokens ? t : tokens - 1;               // rows past the end repeat the last token
+    x_src[i] = x + static_cast<size_t>(t) * d + (((lr / N) & (S - 1)) * kPart + l_piece * 8);
+  }
+
+  Best<KS> best;
+  best.clear();
+
+  for (int e0 = 0; e0 < E; e0 += N) {              // tiles of N experts
+    const bool has_w = e0 + r < E;
+    // the bias of the column this thread finishes (the same for all its elements: the
+    // workgroup size is a multiple of N), asked for before the long part
+    float my_bias = 0.0f;
+    if (bg && e0 + static_cast<int>(threadIdx.x) % N < E) my_bias = static_cast<float>(bg[e0 + threadIdx.x % N]);
+    const half_t *w_src[kWLoads];
+#pragma unroll
+    for (int i = 0; i < kWLoads; ++i) {
+      const int wr = 16 * i + l_row;
+      int e = e0 + wr % N;
+      e = e < E ? e : E - 1;
+      w_src[i] = wg + static_cast<size_t>(e) * d + ((wr / N) * kPart + l_piece * 8);
+    }
+    for (int rd = 0; rd < rounds; ++rd) {
+      const int part0 = rd * per_round + wave * S;               // this wavefront's first part of the round
+      if (part0 < nparts) {                        // uniform per wavefront
+        int left = d - part0 * kPart;                            // the wavefront's first part is its longest
+        left = left < kPart ? left : kPart;
+        const int stages = (left + kStageK - 1) / kStageK;       // 1..4
+        const int k0 = part0 * kPart;
+        const int k_mine = k0 + slot * kPart;                    // where this lane's part starts (may be past d)
+        typename M::Acc acc;
+#pragma unroll
+        for (int v = 0; v < M::kRegs; ++v) acc[v] = 0.0f;
+
+        // Loads of stage s: every lane loads (from the start of the tensor where K has
+        // ended) and unwanted pieces become zero when they are used, so there is no branch
+        // around a load and the number of loads in flight is known where the waits go.
+        int4v xa[4], wa[kWLoads], xb[4], wb[kWLoads];
+        auto fetch = [&](int s, int4v (&xv)[4], int4v (&wv)[kWLoads]) {
+          const int ks = k0 + s * kStageK;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int kx = ks + (((16 * i + l_row) / N) & (S - 1)) * kPart + l_piece * 8;
+            xv[i] = *reinterpret_cast<const int4v *>(kx < d ? x_src[i] + ks : x);
+          }
+#pragma unroll
+          for (int i = 0; i < kWLoads; ++i) {
+            const int kw = ks + ((16 * i + l_row) / N) * kPart + l_piece * 8;
+            wv[i] = *reinterpret_cast<const int4v *>(kw < d ? w_src[i] + ks : wg);
+          }
+        };
+        auto park = [&](const int4v (&xv)[4], const int4v (&wv)[kWLoads]) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) *reinterpret_cast<int4v *>(park_at + 16 * i * kRowBytes) = xv[i];
+#pragma unroll
+          for (int i = 0; i < kWLoads; ++i)
+            *reinterpret_cast<int4v *>(park_at + kTileBytes + 16 * i * kRowBytes) = wv[i];
+        };
+        auto take = [&](int c, half8 &vx, half8 &vw) {
+          vx = *reinterpret_cast<const half8 *>(my_x + c * 16);
+          vw = *reinterpret_cast<const half8 *>(my_w + c * 16);
+        };
+        auto run = [&](int s, int c, const half8 &vx, const half8 &vw) {
+          const bool in = k_mine + s * kStageK + c * 8 < d;
+          const half8 zero = {};
+          const half8 xs = in ? vx : zero;
+          const half8 ws = (in && has_w) ? vw : zero;
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            acc = M::run(static_cast<float>(xs[j]), static_cast<float>(ws[j]), acc);
+        };
+        // One stage: its four pieces are read back two at a time; once the last read is on
+        // its way (the LDS works in order) the next stage's operands overwrite the tiles
+        // and the loads of the stage after that leave.  The scheduling barriers keep loads
+        // and LDS traffic where they are written: left alone, the scheduler sinks each
+        // load to just before its use.
+        half8 ax, aw, bx, bw;
+#define CCF_GATE_STAGE(s, PARK_NEXT)                                   \
+  do {                                                                 \
+    take(0, ax, aw);                                                   \
+    take(1, bx, bw);                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+    run(s, 0, ax, aw);                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+    take(2, ax, aw);                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+    run(s, 1, bx, bw);                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+    take(3, bx, bw);                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+    PARK_NEXT;                                                         \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+    run(s, 2, ax, aw);                                                 \
+    run(s, 3, bx, bw);                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+  } while (0)
+        fetch(0, xa, wa);
+        fetch(1, xb, wb);
+        __builtin_amdgcn_sched_barrier(0);
+        park(xa, wa);                              // stage 0
+        fetch(2, xa, wa);
+        __builtin_amdgcn_sched_barrier(0);
+        CCF_GATE_STAGE(0, park(xb, wb); fetch(3, xb, wb));
+        if (stages > 1) {
+          CCF_GATE_STAGE(1, park(xa, wa));
+          if (stages > 2) {
+            CCF_GATE_STAGE(2, park(xb, wb));
+            if (stages > 3) CCF_GATE_STAGE(3, (void)0);
           }
         }
+#undef CCF_GATE_STAGE
+        // part sums into the same region, [slot][token][expert]
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          if (i0 + u * GW * 64 < total) dst[i0 + u * GW * 64] = tmp[u];
+        for (int v = 0; v < M::kRegs; ++v) {
+          const int ob = M::block(v);
+          region[(static_cast<size_t>(ob & (S - 1)) * TW + (ob >> LS) * N + M::row(v, lane)) * N + r] = acc[v];
+        }
+      }
+      __syncthreads();
+      // running sums: the parts of this round in ascending order
+      for (int i = threadIdx.x; i < TW * N; i += blockDim.x) {
+        const int tok = i / N, col = i % N;
+        float t = rd == 0 ? 0.0f : s_total[tok * kLd + col];
+        for (int q = 0; q < per_round; ++q) {
+          const int p = rd * per_round + q;
+          if (p >= nparts) break;
+          const float ps = s_mem[static_cast<size_t>(q >> LS) * kRegionFloats + (q & (S - 1)) * TW * N + i];
+          t = p == 0 ? ps : t + ps;
+        }
+        if (rd == rounds - 1) {
+          const int e = e0 + col;
+          if (e < E) {
+            if (bg) t = t + my_bias;
+            t = round_to<half_t>(t);
+            if (logits_out && t0 + tok < tokens)
+              logits_out[static_cast<size_t>(t0 + tok) * E + e] = static_cast<half_t>(t);
+          }
+        }
+        s_total[tok * kLd + col] = t;
       }
       __syncthreads();
     }
-    const T *wbase = kWLds ? w_lds : wg + static_cast<size_t>(e0) * d;
-
-    for (int gi = 0; gi < groups_per_block; ++gi) {
-      const int grp = blockIdx.x + gi * gridDim.x;
-      if (grp >= n_groups) break;                  // uniform per workgroup
-      const int t0 = (grp * GW + wave) * TT;
-      float *mine = s_logit + (static_cast<size_t>(gi) * GW + wave) * TT * E;
-      const T *xrow[TT];
-#pragma unroll
-      for (int tt = 0; tt < TT; ++tt) {
-        int t = t0 + tt;
-        if (t > tokens - 1) t = tokens - 1;        // tail waves re-read the last token
-        xrow[tt] = x + static_cast<size_t>(t) * d;
-      }
-      float acc[TT][kGateEG];
-#pragma unroll
-      for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-        for (int g = 0; g < kGateEG; ++g) acc[tt][g] = 0.0f;
-
-      for (int it0 = 0; it0 < niter; it0 += kBatch) {
-        Chunk<T> xv[kBatch][TT];
-#pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-          const int c = lane + (it0 + i) * kWave;
-          if (c < nchunk) {
-#pragma unroll
-            for (int tt = 0; tt < TT; ++tt) xv[i][tt].load(xrow[tt] + c * 8);
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-          const int c = lane + (it0 + i) * kWave;
-          if (c < nchunk) {                        // lanes past the end of K skip the whole chunk
-#pragma unroll
-            for (int g = 0; g < kGateEG; ++g) {
-              Chunk<T> wv;
-              if (kWLds) {
-                wv.load(wbase + static_cast<size_t>(g) * d + c * 8);
-              } else {
-                const int row = (e0 + g) < E ? g : (E - 1 - e0);
-                wv.load(wbase + static_cast<size_t>(row) * d + c * 8);
-              }
-#pragma unroll
-              for (int tt = 0; tt < TT; ++tt) xv[i][tt].mac(wv, acc[tt][g]);
-            }
-          }
-        }
-      }
-      // Fold the 64 lane sums of all TT*kGateEG accumulators at once.  Level by
-      // level (xor 32, 16, ...) a lane keeps the half of the values its lane bit
-      // selects and adds the partner's copy of them, so N values cost N-1
-      // exchanges instead of 6N; the pairs added at each level, and therefore
-      // the bits of the result, are those of the plain butterfly.  Value i ends
-      // up in the lanes whose top log2(N) lane bits spell i.
-      constexpr int N = TT * kGateEG;
-      float v[N];
-#pragma unroll
-      for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-        for (int g = 0; g < kGateEG; ++g) v[tt * kGateEG + g] = acc[tt][g];
-      fold_lanes<N, 32>(v, lane);
-      {
-        constexpr int kBits = N == 32 ? 5 : (N == 16 ? 4 : 3);
-        static_assert(N == 8 || N == 16 || N == 32, "TT*kGateEG");
-        const int i = lane >> (6 - kBits);                      // value this lane holds
-        const int tt = i / kGateEG, g = i % kGateEG;
-        if ((lane & ((1 << (6 - kBits)) - 1)) == 0 && g < ng) {
-          float b = bg ? static_cast<float>(bg[e0 + g]) : 0.0f;
-          mine[tt * E + e0 + g] = round_to<T>(v[0] + b);
-        }
-      }
+    // one thread per token: the logits of this tile, ascending expert id
+    if (threadIdx.x < TW && t0 + threadIdx.x < tokens) {
+      const float *lg = s_total + threadIdx.x * kLd;
+      const int ne = (E - e0) < N ? (E - e0) : N;
+      for (int c = 0; c < ne; ++c) best.offer(lg[c], e0 + c, k);
     }
+    // s_total is next written after the next tile's first barrier, which these threads reach later
   }
-  __syncthreads();
+  if (threadIdx.x < TW && t0 + threadIdx.x < tokens)
+    best.template write<half_t>(t0 + threadIdx.x, k, idx_out, score_out);
+}
 
-  for (int gi = 0; gi < groups_per_block; ++gi) {
-    const int grp = blockIdx.x + gi * gridDim.x;
-    if (grp >= n_groups) break;
-    const int t0 = (grp * GW + wave) * TT;
-    const float *mine = s_logit + (static_cast<size_t>(gi) * GW + wave) * TT * E;
-#pragma unroll 1
-    for (int tt = 0; tt < TT; ++tt) {
-      const int t = t0 + tt;
-      if (t >= tokens) break;                      // uniform per wave
-      const float *lg = mine + tt * E;
-      if (logits_out)
-        for (int e = lane; e < E; e += kWave)
-          logits_out[static_cast<size_t>(t) * E + e] = static_cast<T>(lg[e]);
+// fp32 gate on the vector unit, one wavefront per token: lane l takes parts l, l + 64, ...
+// for eight experts at a time, multiply and add rounded separately; lanes 0..7 then add
+// the part sums in order.  The logits of the token wait in LDS for the selection.
+constexpr int kGroup32 = 8;
 
-      float sel_v[kMaxTopK];
-      int sel_id[kMaxTopK];
+__global__ void __launch_bounds__(64)
+gate_f32_kernel(const float *__restrict__ x, const float *__restrict__ wg, const float *__restrict__ bg,
+                int tokens, int d, int E, int k, int64_t *__restrict__ idx_out,
+                float *__restrict__ score_out, float *__restrict__ logits_out) {
+#pragma clang fp contract(off)
+  extern __shared__ float s_mem[];
+  const int lane = threadIdx.x;
+  const int nparts = (d + kPart - 1) / kPart;
+  float *s_logit = s_mem;                          // [E]
+  float *s_part = s_mem + E;                       // [kGroup32][nparts]
+  const int t = blockIdx.x;
+  const float *xrow = x + static_cast<size_t>(t) * d;
+  for (int e0 = 0; e0 < E; e0 += kGroup32) {
+    for (int p = lane; p < nparts; p += kWave) {
+      float acc[kGroup32];
 #pragma unroll
-      for (int s = 0; s < kMaxTopK; ++s) {
-        sel_v[s] = 0.0f;
-        sel_id[s] = -1;
-      }
+      for (int g = 0; g < kGroup32; ++g) acc[g] = 0.0f;
+      const int k_end = (p + 1) * kPart < d ? (p + 1) * kPart : d;
+      for (int kk = p * kPart; kk < k_end; kk += 4) {
+        const float4v xv = *reinterpret_cast<const float4v *>(xrow + kk);
 #pragma unroll
-      for (int s = 0; s < kMaxTopK; ++s) {
-        if (s < k) {
-          float bv = -INFINITY;
-          int bid = INT_MAX;
-          for (int e = lane; e < E; e += kWave) {
-            bool taken = false;
+        for (int g = 0; g < kGroup32; ++g) {
+          const int e = (e0 + g) < E ? (e0 + g) : E - 1;
+          const float4v wv = *reinterpret_cast<const float4v *>(wg + static_cast<size_t>(e) * d + kk);
 #pragma unroll
-            for (int q = 0; q < kMaxTopK; ++q) taken = taken || (q < s && sel_id[q] == e);
-            float v = lg[e];
-            if (!taken && better(v, e, bv, bid)) {
-              bv = v;
-              bid = e;
-            }
-          }
-#pragma unroll
-          for (int off = 32; off >= 1; off >>= 1) {
-            float ov = __shfl_xor(bv, off, kWave);
-            int oi = __shfl_xor(bid, off, kWave);
-            if (better(ov, oi, bv, bid)) {
-              bv = ov;
-              bid = oi;
-            }
-          }
-          sel_v[s] = bv;
-          sel_id[s] = bid;
-        }
-      }
-      if (lane == 0) {
-        // softmax over the k selected logits; slot 0 holds the maximum
-        float ex[kMaxTopK];
-        float sum = 0.0f;
-#pragma unroll
-        for (int s = 0; s < kMaxTopK; ++s) {
-          ex[s] = (s < k) ? expf(sel_v[s] - sel_v[0]) : 0.0f;
-          sum += ex[s];
-        }
-#pragma unroll
-        for (int s = 0; s < kMaxTopK; ++s) {
-          if (s < k) {
-            idx_out[static_cast<size_t>(t) * k + s] = static_cast<int64_t>(sel_id[s]);
-            score_out[static_cast<size_t>(t) * k + s] = static_cast<T>(ex[s] / sum);
+          for (int j = 0; j < 4; ++j) {
+            const float prod = xv[j] * wv[j];
+            acc[g] = acc[g] + prod;
           }
         }
       }
+#pragma unroll
+      for (int g = 0; g < kGroup32; ++g) s_part[g * nparts + p] = acc[g];
     }
+    __syncthreads();
+    if (lane < kGroup32 && e0 + lane < E) {
+      float s = s_part[lane * nparts];
+      for (int p = 1; p < nparts; ++p) s = s + s_part[lane * nparts + p];
+      if (bg) s = s + bg[e0 + lane];
+      s_logit[e0 + lane] = s;
+    }
+    __syncthreads();
+  }
+  if (logits_out)
+    for (int e = lane; e < E; e += kWave) logits_out[static_cast<size_t>(t) * E + e] = s_logit[e];
+  if (lane == 0) {
+    Best<kMaxTopK> best;
+    best.clear();
+    for (int e = 0; e < E; ++e) best.offer(s_logit[e], e, k);
+    best.write<float>(t, k, idx_out, score_out);
   }
 }
 
@@ -313,59 +418,61 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
   CCF_REQUIRE(dtype == CCF_F16 || dtype == CCF_F32, CCF_ERR_UNSUPPORTED, "gate: dtype %d", dtype);
   CCF_REQUIRE(aligned16(x) && aligned16(wg), CCF_ERR_ARG, "gate: x and wg must be 16-byte aligned");
   if (tokens == 0) return CCF_OK;
-  // Enough wavefronts to hide HBM latency: fewer tokens per wavefront when the batch is small.
-  const int tt = g_gate_tt ? g_gate_tt : (tokens >= 32768 ? 4 : (tokens >= 8192 ? 2 : 1));
-  const size_t esz = dtype == CCF_F16 ? 2 : 4;
-  // the kernel always stages kGateEG weight rows (rows past the last expert repeat it)
-  const size_t w_bytes = static_cast<size_t>(kGateEG) * d_model * esz;
-  const bool w_lds = w_bytes <= 65536;             // one expert group of weights fits next to the logits
-  // Wavefronts per workgroup: 16 (one workgroup per CU stages the weights once for 16
-  // wavefronts) when the weights sit in LDS, else 4 (two workgroups per CU).
-  const int gw = (w_lds && g_gate_waves != 4) ? 16 : 4;
-  const int n_groups = (tokens + gw * tt - 1) / (gw * tt);
-  const int max_blocks = gw == 16 ? 256 : 512;     // persistent workgroups
-  int blocks = n_groups < max_blocks ? n_groups : max_blocks;
-  int groups_per_block = (n_groups + blocks - 1) / blocks;
-  // the logits of a workgroup's tokens wait in LDS: more workgroups when they would not fit
-  const size_t per_group = sizeof(float) * gw * tt * static_cast<size_t>(tot_expert);
-  const size_t lds_budget = 160 * 1024 - (w_lds ? w_bytes : 0);
-  if (per_group * groups_per_block > lds_budget && per_group <= lds_budget) {
-    groups_per_block = static_cast<int>(lds_budget / per_group);
-    blocks = (n_groups + groups_per_block - 1) / groups_per_block;
+  const int nparts = (d_model + kPart - 1) / kPart;
+  if (dtype == CCF_F32) {
+    const size_t lds = sizeof(float) * (static_cast<size_t>(tot_expert) + static_cast<size_t>(kGroup32) * nparts);
+    CCF_REQUIRE(lds <= 64 * 1024, CCF_ERR_SHAPE, "gate: fp32 d_model=%d needs %zu bytes of LDS", d_model, lds);
+    hipLaunchKernelGGL(gate_f32_kernel, dim3(tokens), dim3(64), lds, as_stream(stream),
+                       static_cast<const float *>(x), static_cast<const float *>(wg),
+                       static_cast<const float *>(bg), tokens, d_model, tot_expert, top_k, idx_out,
+                       static_cast<float *>(score_out), static_cast<float *>(logits_out));
+    return check_launch("gate_f32_kernel");
   }
-  dim3 grid(blocks), block(gw * 64);
-  const size_t lds = per_group * groups_per_block + (w_lds ? w_bytes : 0);
+  // Tile and slots.  With S slots a wavefront covers 64 / S tokens, so S grows while the
+  // token count would leave CUs without a workgroup and K has parts for the slots.
+  const int n = tot_expert > 16 ? 32 : 16;
+  const int blocks_per_mfma = 64 / n;
+  int ls = 0;
+  if (g_gate_slots) {
+    while ((2 << ls) <= g_gate_slots && (2 << ls) <= blocks_per_mfma) ++ls;
+  } else {
+    while ((2 << ls) <= blocks_per_mfma && (2 << ls) <= nparts &&
+           (tokens + (64 >> ls) - 1) / (64 >> ls) < 512)
+      ++ls;
+  }
+  const int slots = 1 << ls;
+  const int tw = 64 >> ls;
+  int waves = (nparts + slots - 1) / slots;
+  int cap = g_gate_waves < kMaxWaves ? g_gate_waves : kMaxWaves;
+  cap = cap < 1 ? 1 : cap;
+  waves = waves < cap ? waves : cap;
+  const size_t lds = sizeof(float) * (static_cast<size_t>(waves) * kRegionFloats + static_cast<size_t>(tw) * (n + 1));
   CCF_REQUIRE(lds <= 160 * 1024, CCF_ERR_SHAPE, "gate: %zu bytes of LDS needed", lds);
-#define CCF_GATE_LAUNCH(TYPE, TT, WL, GWV)                                                            \
+  dim3 grid((tokens + tw - 1) / tw), block(waves * 64);
+#define CCF_GATE_LAUNCH(NN, LSV, KSV)                                                              \
   do {                                                                                             \
-    auto kern = gate_kernel<TYPE, TT, WL, GWV>;                                                    \
+    auto kern = gate_mfma_kernel<NN, LSV, KSV>;                                                    \
     if (lds > 65536) {                                                                             \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                     \
                                          hipFuncAttributeMaxDynamicSharedMemorySize,               \
                                          static_cast<int>(lds));                                   \
       if (e != hipSuccess) return fail(CCF_ERR_HIP, "gate: LDS attribute: %s", hipGetErrorString(e)); \
     }                                                                                              \
-    hipLaunchKernelGGL(kern, grid, block, lds, as_stream(stream), static_cast<const TYPE *>(x),    \
-                       static_cast<const TYPE *>(wg), static_cast<const TYPE *>(bg), tokens,      \
-                       d_model, tot_expert, top_k, groups_per_block, idx_out,                      \
-                       static_cast<TYPE *>(score_out),                                             \
-                       static_cast<TYPE *>(logits_out));                                           \
+    hipLaunchKernelGGL(kern, grid, block, lds, as_stream(stream), static_cast<const half_t *>(x),  \
+                       static_cast<const half_t *>(wg), static_cast<const half_t *>(bg), tokens,   \
+                       d_model, tot_expert, top_k, idx_out, static_cast<half_t *>(score_out),      \
+                       static_cast<half_t *>(logits_out));                                         \
   } while (0)
-#define CCF_GATE_TT(TYPE, WL, GWV)                    \
-  do {                                                \
-    if (tt == 4) CCF_GATE_LAUNCH(TYPE, 4, WL, GWV);   \
-    else if (tt == 2) CCF_GATE_LAUNCH(TYPE, 2, WL, GWV); \
-    else CCF_GATE_LAUNCH(TYPE, 1, WL, GWV);           \
+#define CCF_GATE_K(NN, LSV)                                                  \
+  do {                                                                       \
+    if (top_k <= 2) CCF_GATE_LAUNCH(NN, LSV, 2); else CCF_GATE_LAUNCH(NN, LSV, kMaxTopK); \
   } while (0)
-#define CCF_GATE_W(TYPE)                                              \
-  do {                                                                \
-    if (!w_lds) CCF_GATE_TT(TYPE, false, 4);                          \
-    else if (gw == 16) CCF_GATE_TT(TYPE, true, 16);                   \
-    else CCF_GATE_TT(TYPE, true, 4);                                  \
-  } while (0)
-  if (dtype == CCF_F16) CCF_GATE_W(half_t); else CCF_GATE_W(float);
-#undef CCF_GATE_W
-#undef CCF_GATE_TT
+  if (n == 32) {
+    if (ls == 0) CCF_GATE_K(32, 0); else CCF_GATE_K(32, 1);
+  } else {
+    if (ls == 0) CCF_GATE_K(16, 0); else if (ls == 1) CCF_GATE_K(16, 1); else CCF_GATE_K(16, 2);
+  }
+#undef CCF_GATE_K
 #undef CCF_GATE_LAUNCH
-  return check_launch("gate_kernel");
+  return check_launch("gate_mfma_kernel");
 }

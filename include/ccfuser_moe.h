@@ -67,19 +67,22 @@ const char *ccf_last_error(void);
  *   "fused_combine"   0/1 (default 0): ccf_moe_forward with top_k = 2 adds the gate-weighted expert outputs
  *                     into the output in the second GEMM's epilogue (packed fp16 atomic adds onto zeros)
  *                     instead of running the combine pass; measured slower, kept for comparison
- *   "gate_tokens"     0, 1, 2 or 4: tokens a gate wavefront scores at a time (0 = chosen by the token count)
+ *   "gate_slots"      0, 1, 2 or 4: parts of K a gate wavefront works on at a time, which divides the tokens
+ *                     of a workgroup by the same number (0 = chosen by the token count)
  *   "dgrad_transpose" 0/1: the backward's input-gradient GEMM runs on a transposed copy of the
  *                     weight instead of reading the stored one
- *   "gate_waves"      4 or 16: cap on the gate kernel's wavefronts per workgroup
+ *   "gate_waves"      1..8 (default 8): most wavefronts of a gate workgroup; each takes other parts of K
  */
 int ccf_set_option(const char *name, int value);
 
 /* ------------------------------------------------------------------ gate */
 
 /*
- * Top-k gate: logits = x * wg^T + bg (fp32 accumulation in a fixed order,
- * rounded once to the input dtype), top-k per token (slot 0 = largest, ties to
- * the lower expert id), softmax over the k selected logits.
+ * Top-k gate: logits = x * wg^T + bg (fp32 accumulation in a fixed order:
+ * parts of 128 consecutive K elements, each a chain of multiply-adds in
+ * ascending K from zero, the part sums added in ascending order, the bias
+ * last; rounded once to the input dtype), top-k per token (slot 0 = largest,
+ * ties to the lower expert id), softmax over the k selected logits.
  * Replaces NaiveGate.forward, mix_moe/mix_moe/gates/naive_gate.py:26-45.
  *   x [tokens, d_model], wg [tot_expert, d_model], bg [tot_expert] or NULL,
  *   idx_out int64 [tokens, top_k], score_out [tokens, top_k] in the input

@@ -60,8 +60,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-WAVE = 64          # lanes in the fixed accumulation order
-CHUNK = 8          # consecutive K elements one lane consumes per step
+PART = 128         # consecutive K elements whose products are summed as one chain
 
 
 # --------------------------------------------------------------------------
@@ -71,40 +70,31 @@ def gate_logits(x: torch.Tensor, wg: torch.Tensor, bg: Optional[torch.Tensor]) -
     """``x @ wg.T + bg`` accumulated in fp32 in a fixed order; returns fp32 [T, E].
 
     Follows ``self.gate(inp)`` (naive_gate.py:31).  The order: K is cut into
-    chunks of 8; lane ``l`` of 64 owns chunks ``l, l+64, ...`` and adds their
-    products one element at a time in ascending K; the 64 partial sums are then
-    combined by a butterfly ``v += v[lane ^ off]`` for off = 32,16,8,4,2,1; the
-    bias is added last.  Products of two fp16 values are exact in fp32, so for
-    fp16 inputs fused and unfused multiply-add agree; for fp32 inputs the
-    multiply is rounded before the add (no fused multiply-add).
+    parts of 128 consecutive elements (the last may be shorter); a part's sum
+    starts at zero and takes its products one at a time in ascending K; the
+    part sums are added one after the other in ascending order, starting from
+    the first; the bias is added last.  Products of two fp16 values are exact
+    in fp32, so for fp16 inputs ``acc + x*w`` with the product rounded first is
+    the same number as a fused multiply-add; for fp32 inputs the multiply is
+    rounded before the add (no fused multiply-add).
     """
     T, d = x.shape
     E = wg.shape[0]
-    if d % CHUNK:
+    if d % 8:
         raise ValueError("d_model must be a multiple of 8")
-    nchunk = d // CHUNK
-    niter = -(-nchunk // WAVE)
-    pad = niter * WAVE * CHUNK - d
-    x32 = x.detach().to(torch.float32).numpy()
-    w32 = wg.detach().to(torch.float32).numpy()
-    if pad:
-        x32 = np.concatenate([x32, np.zeros((T, pad), np.float32)], axis=1)
-        w32 = np.concatenate([w32, np.zeros((E, pad), np.float32)], axis=1)
-    ws = w32.reshape(E, niter, WAVE, CHUNK)
+    x32 = np.ascontiguousarray(x.detach().to(torch.float32).numpy().T)     # [d, T]
+    w32 = np.ascontiguousarray(wg.detach().to(torch.float32).numpy().T)    # [d, E]
     out = np.empty((T, E), np.float32)
-    lanes = np.arange(WAVE)
-    step = max(1, (1 << 22) // max(1, E * WAVE))      # bound the temporaries
+    step = max(1, (1 << 22) // max(1, E))              # bound the temporaries
     for t0 in range(0, T, step):
-        xs = x32[t0:t0 + step].reshape(-1, niter, WAVE, CHUNK)
-        acc = np.zeros((xs.shape[0], E, WAVE), np.float32)
-        for i in range(niter):
-            live = min(WAVE, nchunk - i * WAVE)       # lanes past the end skip the add
-            for j in range(CHUNK):
-                prod = xs[:, None, i, :live, j] * ws[None, :, i, :live, j]
-                acc[:, :, :live] = acc[:, :, :live] + prod
-        for off in (32, 16, 8, 4, 2, 1):
-            acc = acc + acc[:, :, lanes ^ off]
-        out[t0:t0 + step] = acc[:, :, 0]
+        xs = x32[:, t0:t0 + step]
+        total = None
+        for p0 in range(0, d, PART):
+            acc = np.zeros((xs.shape[1], E), np.float32)
+            for k in range(p0, min(p0 + PART, d)):
+                acc = acc + xs[k][:, None] * w32[k][None, :]
+            total = acc if total is None else total + acc
+        out[t0:t0 + step] = total
     if bg is not None:
         out = out + bg.detach().to(torch.float32).numpy()[None, :]
     return torch.from_numpy(out)

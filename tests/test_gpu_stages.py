@@ -48,24 +48,40 @@ def test_gate_bit_exact(T, d, E, k, dtype, seed):
     assert torch.allclose(score.float().sum(-1).cpu(), torch.ones(T), atol=2e-3)
 
 
-@pytest.mark.parametrize("waves", [4, 16])
-@pytest.mark.parametrize("T,d,E,k", [(5000, 512, 8, 2), (9000, 256, 32, 1), (40000, 128, 16, 2)])
-def test_gate_workgroup_sizes(waves, T, d, E, k):
-    """Both workgroup shapes of the gate, with several token groups per workgroup
-    and (T >= 8192, 32768) two and four tokens per wavefront."""
+_GATE_CASES = {}
+
+
+def _gate_case(T, d, E, k):
+    key = (T, d, E, k)
+    if key not in _GATE_CASES:
+        g = torch.Generator().manual_seed(T + E)
+        x = torch.randn(T, d, generator=g).half()
+        wg = (torch.randn(E, d, generator=g) * 0.05).half()
+        bg = (torch.randn(E, generator=g) * 0.05).half()
+        _GATE_CASES[key] = (x, wg, bg) + tuple(O.naive_gate(x, wg, bg, k))
+    return _GATE_CASES[key]
+
+
+@pytest.mark.parametrize("slots,waves", [(0, 8), (1, 2), (2, 1), (4, 8), (1, 8)])
+@pytest.mark.parametrize("T,d,E,k", [(5000, 512, 8, 2), (9000, 256, 32, 1), (40001, 128, 16, 2),
+                                     (33000, 768, 32, 1), (300, 4096, 12, 2), (2100, 2048, 70, 4),
+                                     (77, 8192, 8, 2), (130, 520, 40, 3)])
+def test_gate_launch_shapes(slots, waves, T, d, E, k):
+    """Every way the gate spreads a problem over the machine gives the oracle's bits: 1, 2
+    or 4 parts of K per wavefront (fewer tokens per workgroup), 1 to 8 wavefronts per
+    workgroup (several rounds of parts when K is long), both tile widths (16 and 32
+    experts, 1 to 3 tiles), a ragged last token group, a short last part."""
     from ccfuser_amd import ops
-    _say(f"gate waves={waves} T={T} d={d} E={E} k={k}")
-    g = torch.Generator().manual_seed(T)
-    x = torch.randn(T, d, generator=g).half()
-    wg = (torch.randn(E, d, generator=g) * 0.05).half()
-    bg = (torch.randn(E, generator=g) * 0.05).half()
-    idx_ref, score_ref, logits_ref = O.naive_gate(x, wg, bg, k)
+    _say(f"gate slots={slots} waves={waves} T={T} d={d} E={E} k={k}")
+    x, wg, bg, idx_ref, score_ref, logits_ref = _gate_case(T, d, E, k)
+    ops.set_option("gate_slots", slots)
     ops.set_option("gate_waves", waves)
     try:
         idx, score, logits = ops.gate_topk_softmax(dev(x), dev(wg), dev(bg), k, return_logits=True)
         torch.cuda.synchronize()
     finally:
-        ops.set_option("gate_waves", 16)
+        ops.set_option("gate_slots", 0)
+        ops.set_option("gate_waves", 8)
     assert torch.equal(logits.cpu(), logits_ref), "logits differ bitwise"
     assert torch.equal(idx.cpu(), idx_ref), "expert choice differs"
     assert (score.cpu().float() - score_ref.float()).abs().max() <= 1e-3

@@ -34,9 +34,9 @@ def test_logits_match_linear(T, d, E, dtype):
 
 def test_logits_order_is_the_documented_one():
     """Brute-force replay of the documented order with Python floats rounded to fp32
-    at every step, on a case large enough to use two chunks per lane."""
+    at every step, on a case with two full parts and a short third one."""
     g = torch.Generator().manual_seed(3)
-    d = 8 * 64 + 8 * 3                     # 67 chunks: lanes 0..2 own two chunks
+    d = 128 * 2 + 8 * 3
     x = torch.randn(2, d, generator=g).half()
     w = torch.randn(3, d, generator=g).half()
     b = torch.randn(3, generator=g).half()
@@ -44,17 +44,37 @@ def test_logits_order_is_the_documented_one():
     f32 = np.float32
     for t in range(2):
         for e in range(3):
-            lanes = [f32(0)] * 64
-            for c in range(d // 8):
-                l = c % 64
-                for j in range(8):
-                    k = c * 8 + j
-                    lanes[l] = f32(lanes[l] + f32(f32(x[t, k].item()) * f32(w[e, k].item())))
-            for off in (32, 16, 8, 4, 2, 1):
-                lanes = [f32(lanes[l] + lanes[l ^ off]) for l in range(64)]
-            assert f32(lanes[0] + f32(b[e].item())) == got[t, e].item()
-    # lanes hold identical values after the butterfly (the kernel reads lane 0)
-    assert len({float(v) for v in lanes}) == 1
+            parts = []
+            for p0 in range(0, d, 128):
+                acc = f32(0)
+                for k in range(p0, min(p0 + 128, d)):
+                    acc = f32(acc + f32(f32(x[t, k].item()) * f32(w[e, k].item())))
+                parts.append(acc)
+            total = parts[0]
+            for p in parts[1:]:
+                total = f32(total + p)
+            assert f32(total + f32(b[e].item())) == got[t, e].item()
+
+
+def test_logits_chain_is_a_chain_of_fused_multiply_adds():
+    """For fp16 inputs every product is exact in fp32, so each step of a part's chain is
+    one rounding of the exact acc + x*w: replayed here with exact rational arithmetic."""
+    from fractions import Fraction
+    g = torch.Generator().manual_seed(11)
+    d = 128 + 16
+    x = (torch.randn(1, d, generator=g) * 8).half()
+    w = (torch.randn(2, d, generator=g) * 0.01).half()
+    got = O.gate_logits(x, w, None)
+    for e in range(2):
+        parts = []
+        for p0 in range(0, d, 128):
+            acc = np.float32(0)
+            for k in range(p0, min(p0 + 128, d)):
+                exact = Fraction(float(acc)) + Fraction(x[0, k].item()) * Fraction(w[e, k].item())
+                acc = np.float32(float(exact))          # exact sums here fit a double: one rounding to fp32
+                assert Fraction(float(np.float64(float(exact)))) == exact
+            parts.append(acc)
+        assert np.float32(parts[0] + parts[1]) == got[0, e].item()
 
 
 @pytest.mark.parametrize("k", [1, 2, 4])
