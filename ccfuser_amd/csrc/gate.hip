@@ -428,8 +428,8 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
                        static_cast<float *>(score_out), static_cast<float *>(logits_out));
     return check_launch("gate_f32_kernel");
   }
-  // Tile and slots.  With S slots a wavefront covers 64 / S tokens, so S grows while the
-  // token count would leave CUs without a workgroup and K has parts for the slots.
+  // Tile and slots.  With S slots a wavefront covers 64 / S tokens, so S grows while there
+  // are fewer than four workgroups per CU and K has parts for the slots.
   const int n = tot_expert > 16 ? 32 : 16;
   const int blocks_per_mfma = 64 / n;
   int ls = 0;
@@ -437,7 +437,7 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
     while ((2 << ls) <= g_gate_slots && (2 << ls) <= blocks_per_mfma) ++ls;
   } else {
     while ((2 << ls) <= blocks_per_mfma && (2 << ls) <= nparts &&
-           (tokens + (64 >> ls) - 1) / (64 >> ls) < 512)
+           (tokens + (64 >> ls) - 1) / (64 >> ls) < 1024)
       ++ls;
   }
   const int slots = 1 << ls;

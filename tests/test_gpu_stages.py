@@ -87,6 +87,37 @@ def test_gate_launch_shapes(slots, waves, T, d, E, k):
     assert (score.cpu().float() - score_ref.float()).abs().max() <= 1e-3
 
 
+@pytest.mark.parametrize("E,k", [(32, 2), (8, 1), (70, 3)])
+def test_gate_logits_that_are_nothing_but_rounding_error(E, k):
+    """Inputs whose exact logits are zero: inside every part of 128 the second half of the
+    products repeats the first half, permuted and negated (weights are powers of two, so
+    every product is exact).  What is left is the rounding error of the fp32 chain, which
+    depends on the order of the additions and on every rounding being to nearest even;
+    scaled into fp16's range it must equal the oracle's bit for bit."""
+    from ccfuser_amd import ops
+    _say(f"gate rounding residue E={E} k={k}")
+    g = torch.Generator().manual_seed(E)
+    T, d = 300, 512
+    x = torch.empty(T, d)
+    w = torch.empty(E, d)
+    for p0 in range(0, d, 128):
+        perm = torch.randperm(64, generator=g)
+        xa = torch.randn(T, 64, generator=g) * 2.0 ** torch.randint(0, 7, (T, 64), generator=g)
+        wa = 2.0 ** torch.randint(2, 8, (E, 64), generator=g) * (torch.randint(0, 2, (E, 64), generator=g) * 2 - 1)
+        x[:, p0:p0 + 64] = xa
+        w[:, p0:p0 + 64] = wa
+        x[:, p0 + 64:p0 + 128] = -xa[:, perm]
+        w[:, p0 + 64:p0 + 128] = wa[:, perm]
+    x, w = x.half(), w.half()
+    assert torch.equal((x.double() @ w.double().t()), torch.zeros(T, E, dtype=torch.float64))
+    idx_ref, score_ref, logits_ref = O.naive_gate(x, w, None, k)
+    assert (logits_ref != 0).float().mean() > 0.5          # the residue is there
+    idx, score, logits = ops.gate_topk_softmax(dev(x), dev(w), None, k, return_logits=True)
+    torch.cuda.synchronize()
+    assert torch.equal(logits.cpu(), logits_ref), "rounding residue differs"
+    assert torch.equal(idx.cpu(), idx_ref)
+
+
 def test_gate_ties_go_to_lower_expert():
     from ccfuser_amd import ops
     x = torch.ones(8, 64, dtype=torch.float16)
