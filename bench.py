@@ -265,6 +265,71 @@ def bench_backward(a, wl, ops):
     print(json.dumps(line))
 
 
+def bench_overlap(a, wl, ops):
+    """Does the gate + count/scan/pos of a layer hide under the work in front of it?  The
+    reference plans the next MoE layer on a Python thread while attention runs
+    (transformer.py:102-145, 376-423); here the planning is a few kernels on a side stream.
+    Timed: a dense fp16 GEMM of the layer's token count (standing in for the block in front,
+    [T, d] x [d, d]) followed by the staged layer forward, with the assignment issued inline,
+    and with it issued on the side stream before the GEMM."""
+    import torch
+    from ccfuser_amd.mix_moe import MixMOETransformerMLP
+    t = wl.tensors
+    T, d, f, E, k = wl.tokens, wl.d_model, wl.d_ffn, wl.num_expert, wl.top_k
+    K, W = a.steps, a.warmup
+    cf = None if wl.capacity < 0 else wl.capacity * E / (T * k)
+    mlp = MixMOETransformerMLP("naive", {"num_local_expert": E, "hidden_size": f}, d, 0, 1,
+                               total_batch_size=T, top_k=k, capacity_factor=cf, fused=False,
+                               popular_expert_num=0).half().cuda()
+    with torch.no_grad():
+        mlp.gate.gate.weight.copy_(t["wg"]); mlp.gate.gate.bias.copy_(t["bg"])
+        mlp.experts.htoh4.weight.copy_(t["w1"]); mlp.experts.htoh4.bias.copy_(t["b1"])
+        mlp.experts.h4toh.weight.copy_(t["w2"]); mlp.experts.h4toh.bias.copy_(t["b2"])
+    x = t["x"].cuda()
+    g = torch.Generator(device="cuda").manual_seed(3)
+    pa = torch.randn(T, d, device="cuda", generator=g).half()
+    pb = (torch.randn(d, d, device="cuda", generator=g) * 0.02).half()
+    pc = torch.empty(T, d, device="cuda", dtype=torch.float16)
+
+    def front():
+        torch.matmul(pa, pb, out=pc)
+
+    def inline():
+        front()
+        return mlp(x)
+
+    def ahead():
+        mlp.async_expert_assignment(x)
+        front()
+        return mlp(x)
+
+    def assign_only():
+        mlp.async_expert_assign.capacity = mlp._capacity(T)
+        mlp.async_expert_assign.process_data(mlp.gate, x, E, 1)
+
+    out = {}
+    with torch.no_grad():
+        same = torch.equal(inline(), ahead())
+        for name, fn in (("front_gemm", front), ("assignment", assign_only), ("inline", inline), ("ahead", ahead)):
+            for _ in range(W):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(K):
+                fn()
+            torch.cuda.synchronize()
+            out[name] = (time.perf_counter() - t0) / K * 1e3
+    line = {
+        "metric": "moe_layer_with_assignment_ahead_ms", "value": out["ahead"], "unit": "ms",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": out["ahead"], "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"{wl.name}: {wl.description}; a [T,d]x[d,d] GEMM in front of the staged layer "
+                               "forward, gate + count/scan/pos inline or on a side stream ahead of that GEMM"},
+        "ms": out, "hidden_us": (out["inline"] - out["ahead"]) * 1e3, "outputs_bit_equal": bool(same),
+    }
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -285,6 +350,9 @@ def main():
     ap.add_argument("--backward", action="store_true",
                     help="time a training step (forward + backward through the mirrored module) "
                          "instead of the forward; prints its own metric")
+    ap.add_argument("--overlap", action="store_true",
+                    help="time the staged forward behind a dense GEMM with the gate and routing issued inline "
+                         "and ahead on a side stream; prints its own metric")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU's share only: this build has no collectives or sharding "
@@ -319,6 +387,8 @@ def main():
 
     if a.backward:
         return bench_backward(a, wl, ops)
+    if a.overlap:
+        return bench_overlap(a, wl, ops)
 
     segments = a.workload == "c4_ep_share"
     if segments:
