@@ -343,56 +343,50 @@ gate_mfma_kernel(const half_t *__restrict__ x, const half_t *__restrict__ wg, co
     best.template write<half_t>(t0 + threadIdx.x, k, idx_out, score_out);
 }
 
-// fp32 gate on the vector unit, one wavefront per token: lane l takes parts l, l + 64, ...
-// for eight experts at a time, multiply and add rounded separately; lanes 0..7 then add
-// the part sums in order.  The logits of the token wait in LDS for the selection.
-constexpr int kGroup32 = 8;
-
+// fp32 gate on the vector unit, one wavefront per token: a lane takes one (expert, part)
+// pair at a time and walks the part in ascending K, multiply and add rounded separately;
+// lanes then add each expert's part sums in order.  The logits of the token wait in LDS
+// for the selection.
 __global__ void __launch_bounds__(64)
 gate_f32_kernel(const float *__restrict__ x, const float *__restrict__ wg, const float *__restrict__ bg,
-                int tokens, int d, int E, int k, int64_t *__restrict__ idx_out,
+                int tokens, int d, int E, int k, int group, int64_t *__restrict__ idx_out,
                 float *__restrict__ score_out, float *__restrict__ logits_out) {
 #pragma clang fp contract(off)
   extern __shared__ float s_mem[];
   const int lane = threadIdx.x;
   const int nparts = (d + kPart - 1) / kPart;
   float *s_logit = s_mem;                          // [E]
-  float *s_part = s_mem + E;                       // [kGroup32][nparts]
+  float *s_part = s_mem + E;                       // [group][nparts]: `group` experts at a time
   const int t = blockIdx.x;
   const float *xrow = x + static_cast<size_t>(t) * d;
-  for (int e0 = 0; e0 < E; e0 += kGroup32) {
-    for (int p = lane; p < nparts; p += kWave) {
-      float acc[kGroup32];
-#pragma unroll
-      for (int g = 0; g < kGroup32; ++g) acc[g] = 0.0f;
+  for (int e0 = 0; e0 < E; e0 += group) {
+    const int ne = (E - e0) < group ? (E - e0) : group;
+    for (int q = lane; q < ne * nparts; q += kWave) {   // part fastest: neighbours read neighbouring K
+      const int e = e0 + q / nparts, p = q % nparts;
+      const float *wrow = wg + static_cast<size_t>(e) * d;
       const int k_end = (p + 1) * kPart < d ? (p + 1) * kPart : d;
+      float acc = 0.0f;
       for (int kk = p * kPart; kk < k_end; kk += 4) {
         const float4v xv = *reinterpret_cast<const float4v *>(xrow + kk);
+        const float4v wv = *reinterpret_cast<const float4v *>(wrow + kk);
 #pragma unroll
-        for (int g = 0; g < kGroup32; ++g) {
-          const int e = (e0 + g) < E ? (e0 + g) : E - 1;
-          const float4v wv = *reinterpret_cast<const float4v *>(wg + static_cast<size_t>(e) * d + kk);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float prod = xv[j] * wv[j];
-            acc[g] = acc[g] + prod;
-          }
+        for (int j = 0; j < 4; ++j) {
+          const float prod = xv[j] * wv[j];
+          acc = acc + prod;
         }
       }
-#pragma unroll
-      for (int g = 0; g < kGroup32; ++g) s_part[g * nparts + p] = acc[g];
+      s_part[q] = acc;
     }
     __syncthreads();
-    if (lane < kGroup32 && e0 + lane < E) {
-      float s = s_part[lane * nparts];
-      for (int p = 1; p < nparts; ++p) s = s + s_part[lane * nparts + p];
-      if (bg) s = s + bg[e0 + lane];
-      s_logit[e0 + lane] = s;
+    for (int g = lane; g < ne; g += kWave) {
+      float s = s_part[g * nparts];
+      for (int p = 1; p < nparts; ++p) s = s + s_part[g * nparts + p];
+      if (bg) s = s + bg[e0 + g];
+      s_logit[e0 + g] = s;
+      if (logits_out) logits_out[static_cast<size_t>(t) * E + e0 + g] = s;
     }
     __syncthreads();
   }
-  if (logits_out)
-    for (int e = lane; e < E; e += kWave) logits_out[static_cast<size_t>(t) * E + e] = s_logit[e];
   if (lane == 0) {
     Best<kMaxTopK> best;
     best.clear();
@@ -420,11 +414,14 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
   if (tokens == 0) return CCF_OK;
   const int nparts = (d_model + kPart - 1) / kPart;
   if (dtype == CCF_F32) {
-    const size_t lds = sizeof(float) * (static_cast<size_t>(tot_expert) + static_cast<size_t>(kGroup32) * nparts);
+    // part sums of as many experts at a time as 32 KB hold
+    int group = 8192 / nparts;
+    group = group < 1 ? 1 : (group > tot_expert ? tot_expert : group);
+    const size_t lds = sizeof(float) * (static_cast<size_t>(tot_expert) + static_cast<size_t>(group) * nparts);
     CCF_REQUIRE(lds <= 64 * 1024, CCF_ERR_SHAPE, "gate: fp32 d_model=%d needs %zu bytes of LDS", d_model, lds);
     hipLaunchKernelGGL(gate_f32_kernel, dim3(tokens), dim3(64), lds, as_stream(stream),
                        static_cast<const float *>(x), static_cast<const float *>(wg),
-                       static_cast<const float *>(bg), tokens, d_model, tot_expert, top_k, idx_out,
+                       static_cast<const float *>(bg), tokens, d_model, tot_expert, top_k, group, idx_out,
                        static_cast<float *>(score_out), static_cast<float *>(logits_out));
     return check_launch("gate_f32_kernel");
   }

@@ -30,6 +30,7 @@ def dev(t):
     (100, 2048, 64, 2, torch.float16, 4),
     (77, 512, 70, 4, torch.float16, 5),
     (512, 256, 4, 1, torch.float32, 6),
+    (300, 1032, 70, 3, torch.float32, 8),
     (64, 8, 2, 2, torch.float16, 7),
 ])
 def test_gate_bit_exact(T, d, E, k, dtype, seed):
