@@ -32,6 +32,10 @@ def dev(t):
     (512, 256, 4, 1, torch.float32, 6),
     (300, 1032, 70, 3, torch.float32, 8),
     (64, 8, 2, 2, torch.float16, 7),
+    (1, 8, 1, 1, torch.float16, 9),
+    (3, 64, 1024, 8, torch.float16, 10),
+    (70, 16384, 4, 2, torch.float16, 11),
+    (5, 136, 17, 8, torch.float16, 12),
 ])
 def test_gate_bit_exact(T, d, E, k, dtype, seed):
     from ccfuser_amd import ops
