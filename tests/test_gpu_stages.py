@@ -123,6 +123,38 @@ def test_gate_logits_that_are_nothing_but_rounding_error(E, k):
     assert torch.equal(idx.cpu(), idx_ref)
 
 
+def test_gate_random_shapes():
+    """Thirty seeded random shapes (1..2500 tokens, K a multiple of 8 up to 3000, 1..140
+    experts, any top-k the shape allows) under random launch shapes, all bitwise."""
+    from ccfuser_amd import ops
+    import random
+    rng = random.Random(20240607)
+    try:
+        for case in range(30):
+            T = rng.choice([1, 2, 15, 16, 17, 63, 64, 65, rng.randint(66, 2500)])
+            d = 8 * rng.randint(1, 375)
+            E = rng.choice([1, 2, 3, 8, 15, 16, 17, 31, 32, 33, 64, rng.randint(65, 140)])
+            k = rng.randint(1, min(E, 8))
+            slots, waves = rng.choice([0, 1, 2, 4]), rng.randint(1, 8)
+            _say(f"gate random case {case}: T={T} d={d} E={E} k={k} slots={slots} waves={waves}")
+            g = torch.Generator().manual_seed(case)
+            x = (torch.randn(T, d, generator=g) * 2.0 ** rng.randint(-3, 3)).half()
+            wg = (torch.randn(E, d, generator=g) * 0.05).half()
+            bg = (torch.randn(E, generator=g) * 0.05).half() if case % 3 else None
+            idx_ref, score_ref, logits_ref = O.naive_gate(x, wg, bg, k)
+            ops.set_option("gate_slots", slots)
+            ops.set_option("gate_waves", waves)
+            idx, score, logits = ops.gate_topk_softmax(dev(x), dev(wg), None if bg is None else dev(bg), k,
+                                                       return_logits=True)
+            torch.cuda.synchronize()
+            assert torch.equal(logits.cpu(), logits_ref), f"case {case}: logits differ bitwise"
+            assert torch.equal(idx.cpu(), idx_ref), f"case {case}: expert choice differs"
+            assert (score.cpu().float() - score_ref.float()).abs().max() <= 1e-3
+    finally:
+        ops.set_option("gate_slots", 0)
+        ops.set_option("gate_waves", 8)
+
+
 def test_gate_ties_go_to_lower_expert():
     from ccfuser_amd import ops
     x = torch.ones(8, 64, dtype=torch.float16)
