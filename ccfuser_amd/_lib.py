@@ -48,6 +48,7 @@ SIGNATURES = {
     "ccf_moe_forward": (_i, [_p] * 7 + [_i] * 6 + [_p] * 6 + [_p, _sz, _p]),
     "ccf_moe_forward_set_events": (_i, [C.POINTER(_p), _i]),
     "ccf_probe_mfma": (_i, [_i, _i, _i, _p, C.POINTER(C.c_double), _p]),
+    "ccf_probe_mfma_chain": (_i, [_p, _p, _i, _i, _p, _p]),
     "ccf_segments_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "ccf_moe_ffn_segments": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),
 }

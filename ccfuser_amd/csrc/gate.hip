@@ -395,8 +395,38 @@ gate_f32_kernel(const float *__restrict__ x, const float *__restrict__ wg, const
   }
 }
 
+// Probe of the arithmetic the fp16 gate rests on: one wavefront runs a chain of `steps` K = 1
+// fp32 MFMAs, acc = mfma(a[s][lane], b[s][lane], acc), and leaves its accumulator registers
+// as out[reg][lane].
+template <int N>
+__global__ void __launch_bounds__(64)
+mfma_chain_probe_kernel(const float *__restrict__ a, const float *__restrict__ b, int steps,
+                        float *__restrict__ out) {
+  using M = Mfma<N>;
+  typename M::Acc acc;
+#pragma unroll
+  for (int v = 0; v < M::kRegs; ++v) acc[v] = 0.0f;
+  const int lane = threadIdx.x;
+  for (int s = 0; s < steps; ++s) acc = M::run(a[s * 64 + lane], b[s * 64 + lane], acc);
+#pragma unroll
+  for (int v = 0; v < M::kRegs; ++v) out[v * 64 + lane] = acc[v];
+}
+
 }  // namespace
 }  // namespace ccf
+
+extern "C" int ccf_probe_mfma_chain(const float *a, const float *b, int steps, int tile, float *out,
+                                    ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(a && b && out, CCF_ERR_ARG, "probe_mfma_chain: null pointer");
+  CCF_REQUIRE(steps >= 0 && (tile == 16 || tile == 32), CCF_ERR_ARG,
+              "probe_mfma_chain: steps=%d tile=%d (16 or 32)", steps, tile);
+  if (tile == 32)
+    hipLaunchKernelGGL(mfma_chain_probe_kernel<32>, dim3(1), dim3(64), 0, as_stream(stream), a, b, steps, out);
+  else
+    hipLaunchKernelGGL(mfma_chain_probe_kernel<16>, dim3(1), dim3(64), 0, as_stream(stream), a, b, steps, out);
+  return check_launch("mfma_chain_probe_kernel");
+}
 
 extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *bg, int tokens,
                                      int d_model, int tot_expert, int top_k, int dtype,

@@ -309,6 +309,19 @@ int ccf_moe_forward_set_events(void *const *events, int count);
 int ccf_probe_mfma(int workgroups, int iters, int constant_operands, void *out, double *flop,
                    ccf_stream_t stream);
 
+/*
+ * Probe of the arithmetic the fp16 gate rests on (no counterpart in the reference): one
+ * wavefront runs a chain of `steps` K = 1 fp32 MFMAs, acc = mfma(a[s][lane], b[s][lane], acc),
+ * with v_mfma_f32_32x32x1_2b_f32 (tile = 32: two 32 x 32 blocks, 32 accumulator registers) or
+ * v_mfma_f32_16x16x1_4b_f32 (tile = 16: four 16 x 16 blocks, 16 registers), and writes its
+ * accumulator registers as out[reg][lane].  Block b takes rows from a and columns from b of
+ * lanes b*tile .. b*tile + tile - 1.  The tests compare every output with a chain of fused
+ * multiply-adds on the CPU.
+ *   a, b: device, [steps][64] floats; out: device, [tile][64] floats.
+ */
+int ccf_probe_mfma_chain(const float *a, const float *b, int steps, int tile, float *out,
+                         ccf_stream_t stream);
+
 /* Bytes of workspace ccf_moe_ffn_segments needs. */
 size_t ccf_segments_workspace_bytes(int total_rows, int n_seg, int num_expert,
                                     int d_model, int d_ffn);

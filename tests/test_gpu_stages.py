@@ -155,6 +155,49 @@ def test_gate_random_shapes():
         ops.set_option("gate_waves", 8)
 
 
+@pytest.mark.parametrize("tile", [32, 16])
+def test_mfma_chain_equals_a_chain_of_fused_multiply_adds(tile):
+    """What the fp16 gate rests on: a chain of K = 1 fp32 MFMAs gives, per output element,
+    the bits of acc = fma(a, b, acc) step by step (round to nearest even), on operands that
+    fp16 can hold with exponents spread over 16 binades, so that sums cancel and every
+    rounding matters.  Products of such operands are exact in fp32, which lets numpy replay
+    the chain with a multiply and an add.  Also pins which accumulator register of which lane
+    holds which element, as the gate kernel assumes it."""
+    import numpy as np
+    from ccfuser_amd import _lib
+    _say(f"mfma chain probe tile={tile}")
+    steps, blocks, regs = 768, 64 // tile, 32 if tile == 32 else 16
+    g = torch.Generator().manual_seed(tile)
+
+    def operands():
+        v = torch.randn(steps, 64, generator=g) * 2.0 ** torch.randint(-8, 9, (steps, 64), generator=g).float()
+        return v.half().float()                                      # representable in fp16
+
+    for trial in range(6):
+        a, b = operands(), operands()
+        out = torch.full((regs, 64), float("nan"), dtype=torch.float32, device="cuda")
+        a_dev, b_dev = a.cuda(), b.cuda()
+        _lib.call("ccf_probe_mfma_chain", a_dev.data_ptr(), b_dev.data_ptr(), steps, tile,
+                  out.data_ptr(), None)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        an, bn = a.numpy(), b.numpy()
+        for blk in range(blocks):
+            ab, bb = an[:, blk * tile:(blk + 1) * tile], bn[:, blk * tile:(blk + 1) * tile]
+            acc = np.zeros((tile, tile), np.float32)
+            for s_ in range(steps):
+                acc = acc + ab[s_][:, None] * bb[s_][None, :]
+            for v in range(regs):
+                if (v >> 4 if tile == 32 else v >> 2) != blk:
+                    continue
+                for lane in range(64):
+                    if tile == 32:
+                        row, col = 8 * ((v & 15) >> 2) + 4 * (lane >> 5) + (v & 3), lane & 31
+                    else:
+                        row, col = 4 * (lane >> 4) + (v & 3), lane & 15
+                    assert got[v, lane] == acc[row, col], (trial, blk, v, lane)
+
+
 def test_gate_ties_go_to_lower_expert():
     from ccfuser_amd import ops
     x = torch.ones(8, 64, dtype=torch.float16)
