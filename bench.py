@@ -482,7 +482,7 @@ def main():
         ceil = dense_hgemm_ceiling(routed, d, f)
         line["dense_hgemm_ceiling"] = ceil
         line["roofline"]["frac_of_dense_hgemm_ceiling"] = ach / ceil[f"{dom}_shape"]["tflops"]
-        mf = mfma_only_ceiling(lib)
+        mf = mfma_only_ceiling(_lib.probe_lib())
         line["mfma_only_ceiling"] = mf
         line["roofline"]["frac_of_mfma_only_random_operands"] = ach / mf["random_operands"]["tflops"]
     if not a.no_cpu_baseline:

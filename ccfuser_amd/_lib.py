@@ -47,11 +47,18 @@ SIGNATURES = {
     "ccf_moe_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "ccf_moe_forward": (_i, [_p] * 7 + [_i] * 6 + [_p] * 6 + [_p, _sz, _p]),
     "ccf_moe_forward_set_events": (_i, [C.POINTER(_p), _i]),
-    "ccf_probe_mfma": (_i, [_i, _i, _i, _p, C.POINTER(C.c_double), _p]),
-    "ccf_probe_mfma_chain": (_i, [_p, _p, _i, _i, _p, _p]),
     "ccf_segments_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "ccf_moe_ffn_segments": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),
 }
+
+
+# libccfuser_probe.so (include/ccfuser_probe.h): measurement probes, not part of the product ABI
+PROBE_LIB_PATH = LIB_PATH.with_name("libccfuser_probe.so")
+PROBE_SIGNATURES = {
+    "ccf_probe_mfma": (_i, [_i, _i, _i, _p, C.POINTER(C.c_double), _p]),
+    "ccf_probe_mfma_chain": (_i, [_p, _p, _i, _i, _p, _p]),
+}
+_probe: Optional[C.CDLL] = None
 
 
 class CcfError(RuntimeError):
@@ -77,6 +84,21 @@ def lib() -> C.CDLL:
             fn.argtypes = args
         _lib = handle
     return _lib
+
+
+def probe_lib() -> C.CDLL:
+    """The loaded probe library (bench.py and one GPU test use it); raises if it has not been built."""
+    global _probe
+    if _probe is None:
+        if not PROBE_LIB_PATH.exists():
+            raise RuntimeError(f"{PROBE_LIB_PATH} is missing: run `python -m ccfuser_amd.build`")
+        handle = C.CDLL(str(PROBE_LIB_PATH))
+        for name, (res, args) in PROBE_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _probe = handle
+    return _probe
 
 
 def call(name: str, *args) -> None:

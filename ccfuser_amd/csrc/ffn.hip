@@ -109,16 +109,12 @@ __device__ __forceinline__ float gelu_erf_grad(float v) {
 constexpr int kEpiPlain = 0, kEpiGelu = 1, kEpiGeluKeep = 2, kEpiGeluGrad = 3, kEpiCombine = 4;
 
 // Row of the tile's row range [0, rows) that tile row r (0 .. BM-1) holds; padded
-// tile rows repeat a real one.  The 16x16x32 kernels give the upper and the
-// lower half of the tile (one row of wavefronts each) half of the rows each,
-// so that a partly filled tile skips MFMAs in both; the others fill from the top.
+// tile rows repeat a real one.  The upper and the lower half of the tile (one row
+// of wavefronts each) get half of the rows each, so that a partly filled tile
+// skips MFMAs in both.
 template <class Cfg>
 __device__ __forceinline__ int tile_row_to_local(int r, int rows) {
-  if constexpr (Cfg::SCHED == 4) {
-    return Ring16Mainloop<Cfg>::local_row(r, rows);
-  } else {
-    return r < rows ? r : rows - 1;
-  }
+  return Ring16Mainloop<Cfg>::local_row(r, rows);
 }
 
 // Global source of every tile load of this lane for the tile of plan entry
@@ -324,83 +320,18 @@ __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0
   });
 }
 
+// One workgroup per tile (the form used when K is too short for the persistent kernel).
 template <class Cfg, int kEpi, bool kSeg = false, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_kernel(GroupedArgs p) {
-  constexpr bool kGelu = kEpi == kEpiGelu;
-  static_assert(kEpi <= kEpiGelu || Cfg::SCHED == 4, "epilogues 2 and 3 exist for the 16x16x32 kernels only");
-  using ML = GemmMainloop<Cfg>;
   const int4v ent = reinterpret_cast<const int4v *>(p.plan)[blockIdx.x];
   const int e = ent[0];
   if (e < 0) return;                                 // surplus workgroup of the worst-case grid
-  const int row0 = ent[1];
-  const int rows = ent[2];
-  const int tile_n = ent[3];
-  const int n0 = tile_n * Cfg::BN;
-
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
   tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
-
-  const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
-  if constexpr (Cfg::SCHED == 4) {
-    Ring16Mainloop<Cfg, kKN>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, rows, p.N);
-    epilogue16<Cfg, kEpi, kSeg>(p, e, row0, rows, n0);
-    return;
-  } else {
-  typename ML::acc_t acc[Cfg::TM][Cfg::TN];
-#pragma unroll
-  for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-    for (int tn = 0; tn < Cfg::TN; ++tn)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
-
-  if constexpr (Cfg::SCHED == 0) {
-    ML::run(acc, a_src, b_src, p.K);
-  } else if constexpr (Cfg::SCHED == 3) {
-    RingMainloop<Cfg>::run(acc, a_src, b_src, p.K, rows);
-  } else {
-    ML::run_pingpong(acc, a_src, b_src, p.K);
-  }
-
-  // Epilogue: bias (+ GELU) (+ row scale), fp16, 8-byte stores through the row index.
-  float bias_v[Cfg::TN][4][4];
-  int col[Cfg::TN][4];
-#pragma unroll
-  for (int tn = 0; tn < Cfg::TN; ++tn)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      col[tn][q] = n0 + acc_col4<Cfg>(tn, q);
-      half4 bv = {0, 0, 0, 0};
-      if (p.bias && col[tn][q] < p.N) bv = *reinterpret_cast<const half4 *>(bias_e + col[tn][q]);
-#pragma unroll
-      for (int c = 0; c < 4; ++c) bias_v[tn][q][c] = static_cast<float>(bv[c]);
-    }
-#pragma unroll
-  for (int tm = 0; tm < Cfg::TM; ++tm) {
-    const int lr = acc_row<Cfg>(tm);
-    if (lr < rows) {
-      const int j = row0 + lr;
-      const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
-      const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
-      half_t *dst = p.C + crow * p.N;
-#pragma unroll
-      for (int tn = 0; tn < Cfg::TN; ++tn)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          half4 o;
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            float v = acc[tm][tn][4 * q + c] + bias_v[tn][q][c];
-            if (kGelu) v = gelu_erf(v);
-            o[c] = static_cast<half_t>(v * sc);
-          }
-          if (col[tn][q] < p.N) *reinterpret_cast<half4 *>(dst + col[tn][q]) = o;
-        }
-    }
-  }
-  }
+  Ring16Mainloop<Cfg, kKN>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, ent[2], p.N);
+  epilogue16<Cfg, kEpi, kSeg>(p, e, ent[1], ent[2], ent[3] * Cfg::BN);
 }
 
 // ---- skinny tiles -----------------------------------------------------------------
@@ -846,20 +777,13 @@ splitk_reduce_kernel(GroupedArgs p) {
   }
 }
 
-// ---- variants -------------------------------------------------------------------
-// 256x256x64 tiles throughout (the most flop per byte pulled from L2 that the
-// register file allows).  What differs is how the tile loads are pipelined and
-// how the wavefronts split the tile; variant 0 is the default, the others are
-// kept for measurement (ccf_set_option("gemm_variant", n)).
-using Cfg0 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 2, 3>;   // 8 wavefronts of 128x64, five-slot ring
-using Cfg1 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 4, 3>;   // 4 wavefronts of 128x128, five-slot ring
-using Cfg2 = GemmCfg<256, 256, 64, 2, 4, 2, 1, 1, 0>;   // 8 wavefronts, two whole-tile stages
-using Cfg3 = GemmCfg<256, 256, 32, 2, 4, 4, 1, 2, 1>;   // 8 wavefronts, BK=32 x 4 stages, ping-pong
-using Cfg4 = GemmCfg<256, 128, 32, 2, 2, 3, 2, 2, 0>;   // 4 wavefronts, 72 KB LDS: two workgroups per CU
-using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 2, 1, 8, 4>;   // 4 wavefronts of 128x128, 16x16x32 MFMA, mid-tile barrier
-// variant 6: Cfg5 again, persistent workgroups
+// ---- kernel table -----------------------------------------------------------------
+// 256x256x64 tiles (the most flop per byte pulled from L2 that the register file allows), four
+// wavefronts of 128x128.  ccf_set_option("gemm_variant", n): 0 = persistent workgroups (default),
+// 1 = one workgroup per tile for every K (otherwise only K below four K tiles runs that way).
+using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 8>;
 
-constexpr int kDefaultVariant = 6;
+constexpr int kDefaultVariant = 0;
 int g_variant = kDefaultVariant;
 int g_dgrad_transpose = 0;   // 1: input gradients always on a transposed copy of the weight
 int g_split_tail = 1;        // 0: the last round of tiles is not cut along K
@@ -876,6 +800,8 @@ GemmOptions current_options() {
   return GemmOptions{g_variant, g_split_tail, g_split_tail_min_kt, g_split_max_parts, g_skinny_pct, g_fused_combine};
 }
 
+// The kernels of one family of epilogues: `first` and `second` are two epilogue forms, each as
+// the one-workgroup-per-tile kernel and as the persistent kernel.
 struct Launch {
   int bm, bn, threads;
   void (*plain)(GroupedArgs);
@@ -886,28 +812,24 @@ struct Launch {
 };
 constexpr int kPersistentMinKT = 4;
 
-#define CCF_VARIANT(C) {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>, nullptr, nullptr}
-#define CCF_VARIANT_P(C)                                                                          \
-  {C::BM, C::BN, C::THREADS, grouped_gemm_kernel<C, false>, grouped_gemm_kernel<C, true>,          \
-   grouped_gemm_persistent_kernel<C, false>, grouped_gemm_persistent_kernel<C, true>}
-const Launch kVariants[] = {CCF_VARIANT(Cfg0), CCF_VARIANT(Cfg1), CCF_VARIANT(Cfg2), CCF_VARIANT(Cfg3),
-                            CCF_VARIANT(Cfg4), CCF_VARIANT(Cfg5), CCF_VARIANT_P(Cfg5),
-                            // B stored [E, K, N] (input gradients on the stored weight); not selectable
+const Launch kVariants[] = {// forward: "plain" = bias and row scale, "gelu" = bias and GELU
+                            {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiPlain>,
+                             grouped_gemm_kernel<Cfg5, kEpiGelu>, grouped_gemm_persistent_kernel<Cfg5, kEpiPlain>,
+                             grouped_gemm_persistent_kernel<Cfg5, kEpiGelu>},
+                            // B stored [E, K, N] (input gradients on the stored weight)
                             {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiPlain, false, true>,
                              grouped_gemm_kernel<Cfg5, kEpiGeluGrad, false, true>,
                              grouped_gemm_persistent_kernel<Cfg5, kEpiPlain, false, true>,
                              grouped_gemm_persistent_kernel<Cfg5, kEpiGeluGrad, false, true>},
-                            // training forms of the default kernels: "plain" = GELU that keeps the
-                            // pre-activation, "gelu" slot = input gradient through the GELU; not selectable
+                            // training forms: "plain" = GELU that keeps the pre-activation,
+                            // "gelu" slot = input gradient through the GELU
                             {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiGeluKeep>,
                              grouped_gemm_kernel<Cfg5, kEpiGeluGrad>, grouped_gemm_persistent_kernel<Cfg5, kEpiGeluKeep>,
                              grouped_gemm_persistent_kernel<Cfg5, kEpiGeluGrad>},
-                            // the combine epilogue ("plain" slot); not selectable
+                            // the combine epilogue ("plain" slot)
                             {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiCombine>, nullptr,
                              grouped_gemm_persistent_kernel<Cfg5, kEpiCombine>, nullptr}};
-constexpr int kKnVariant = 7, kTrainVariant = 8, kCombineVariant = 9;
-#undef CCF_VARIANT
-#undef CCF_VARIANT_P
+constexpr int kFwdVariant = 0, kKnVariant = 1, kTrainVariant = 2, kCombineVariant = 3;
 
 // Compute units of the current device, rounded down to whole XCD rounds of 8.
 int persistent_grid() {
@@ -922,12 +844,12 @@ int persistent_grid() {
   }
   return cached;
 }
-constexpr int kNumVariants = kKnVariant;             // what ccf_set_option accepts
-constexpr int kMinBM = 128;
+constexpr int kNumVariants = 2;                      // what ccf_set_option accepts
+constexpr int kMinBM = 256;
 
 int max_tiles_for(int max_rows, int E, int bm) { return (max_rows + bm - 1) / bm + E; }
 
-constexpr int kMinBN = 128;
+constexpr int kMinBN = 256;
 
 // Workspace of one grouped GEMM: the split-K tail area, then the tile plan.  A second plan
 // (region 1: header and entries of its own, then the plan; the partial tiles are shared) follows
@@ -976,14 +898,14 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
     g.plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.tail) + kTailHead);
   }
   const bool gelu = epi != kEpiPlain && epi != kEpiCombine;
-  g.v = &kVariants[b_kn ? kKnVariant : (epi == kEpiCombine ? kCombineVariant : (epi >= kEpiGeluKeep ? kTrainVariant : opt.variant))];
+  g.v = &kVariants[b_kn ? kKnVariant : (epi == kEpiCombine ? kCombineVariant : (epi >= kEpiGeluKeep ? kTrainVariant : kFwdVariant))];
   const Launch &v = *g.v;
   // which of the entry's two kernels: the K-N and training entries hold the GELU-gradient form in the second slot
   g.second = b_kn ? epi == kEpiGeluGrad : (epi == kEpiCombine ? false : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu));
   const int max_tiles = max_tiles_for(max_rows, E, v.bm);
   const int n_tiles_n = (N + v.bn - 1) / v.bn;
   g.wgs = launched_wgs(max_tiles, n_tiles_n);                   // worst-case tile count
-  g.grid = v.persistent_plain && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
+  g.grid = opt.variant == 0 && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
   // the last, partly filled round is cut along K and spread over all workgroups (forward forms;
   // worth its two small launches only where a tile is long: K of 4096 and more)
   g.split = opt.split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && g.grid >= 8 && g.grid <= g.wgs &&
@@ -1117,10 +1039,10 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const int grid = persistent_grid();
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;
-    hipLaunchKernelGGL((grouped_gemm_persistent_kernel<Cfg5, false, true>), dim3(static_cast<unsigned>(g)),
+    hipLaunchKernelGGL((grouped_gemm_persistent_kernel<Cfg5, kEpiPlain, true>), dim3(static_cast<unsigned>(g)),
                        dim3(Cfg5::THREADS), 0, stream, p, static_cast<int>(wgs / 8));
   } else {
-    hipLaunchKernelGGL((grouped_gemm_kernel<Cfg5, false, true>), dim3(static_cast<unsigned>(wgs)),
+    hipLaunchKernelGGL((grouped_gemm_kernel<Cfg5, kEpiPlain, true>), dim3(static_cast<unsigned>(wgs)),
                        dim3(Cfg5::THREADS), 0, stream, p);
   }
   return check_launch(what);

@@ -22,6 +22,7 @@
 // of K ("slot"): few tokens still fill the machine.  fp32 inputs keep multiply
 // and add separate (two roundings) and run on the vector unit.
 #include "ccf_common.h"
+#include "mfma_f32.h"
 
 #include <limits.h>
 
@@ -33,8 +34,6 @@ namespace {
 constexpr int kMaxTopK = 8;
 constexpr int kPart = 128;          // K elements of a part
 constexpr int kMaxWaves = 8;
-
-typedef float float32v __attribute__((ext_vector_type(32)));
 
 template <typename T>
 __device__ inline float round_to(float v) {
@@ -103,31 +102,6 @@ struct Best {
   }
 };
 
-template <int N>
-struct Mfma;
-
-template <>
-struct Mfma<32> {
-  typedef float32v Acc;
-  static constexpr int kRegs = 32;
-  __device__ static inline Acc run(float a, float b, Acc c) {
-    return __builtin_amdgcn_mfma_f32_32x32x1f32(a, b, c, 0, 0, 0);
-  }
-  // accumulator register v of a lane: block and row of that output element (column = lane % 32)
-  __device__ static constexpr int block(int v) { return v >> 4; }
-  __device__ static inline int row(int v, int lane) { return 8 * ((v & 15) >> 2) + 4 * (lane >> 5) + (v & 3); }
-};
-
-template <>
-struct Mfma<16> {
-  typedef float16v Acc;
-  static constexpr int kRegs = 16;
-  __device__ static inline Acc run(float a, float b, Acc c) {
-    return __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, c, 0, 0, 0);
-  }
-  __device__ static constexpr int block(int v) { return v >> 2; }
-  __device__ static inline int row(int v, int lane) { return 4 * (lane >> 4) + (v & 3); }
-};
 
 // fp16 gate.  An MFMA has 64 / N blocks; with S = 1 << LS slots, block b of a wavefront is
 // token block b / S on slot b % S, so a wavefront covers TW = (64 / N / S) * N tokens and
@@ -395,38 +369,8 @@ gate_f32_kernel(const float *__restrict__ x, const float *__restrict__ wg, const
   }
 }
 
-// Probe of the arithmetic the fp16 gate rests on: one wavefront runs a chain of `steps` K = 1
-// fp32 MFMAs, acc = mfma(a[s][lane], b[s][lane], acc), and leaves its accumulator registers
-// as out[reg][lane].
-template <int N>
-__global__ void __launch_bounds__(64)
-mfma_chain_probe_kernel(const float *__restrict__ a, const float *__restrict__ b, int steps,
-                        float *__restrict__ out) {
-  using M = Mfma<N>;
-  typename M::Acc acc;
-#pragma unroll
-  for (int v = 0; v < M::kRegs; ++v) acc[v] = 0.0f;
-  const int lane = threadIdx.x;
-  for (int s = 0; s < steps; ++s) acc = M::run(a[s * 64 + lane], b[s * 64 + lane], acc);
-#pragma unroll
-  for (int v = 0; v < M::kRegs; ++v) out[v * 64 + lane] = acc[v];
-}
-
 }  // namespace
 }  // namespace ccf
-
-extern "C" int ccf_probe_mfma_chain(const float *a, const float *b, int steps, int tile, float *out,
-                                    ccf_stream_t stream) {
-  using namespace ccf;
-  CCF_REQUIRE(a && b && out, CCF_ERR_ARG, "probe_mfma_chain: null pointer");
-  CCF_REQUIRE(steps >= 0 && (tile == 16 || tile == 32), CCF_ERR_ARG,
-              "probe_mfma_chain: steps=%d tile=%d (16 or 32)", steps, tile);
-  if (tile == 32)
-    hipLaunchKernelGGL(mfma_chain_probe_kernel<32>, dim3(1), dim3(64), 0, as_stream(stream), a, b, steps, out);
-  else
-    hipLaunchKernelGGL(mfma_chain_probe_kernel<16>, dim3(1), dim3(64), 0, as_stream(stream), a, b, steps, out);
-  return check_launch("mfma_chain_probe_kernel");
-}
 
 extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *bg, int tokens,
                                      int d_model, int tot_expert, int top_k, int dtype,

@@ -8,14 +8,14 @@
 // WMMA tile with fp16 accumulators fed by cp.async; this one is built for
 // CDNA4 instead:
 //
-//   * v_mfma_f32_32x32x16_f16, fp32 accumulators, 64-lane wavefronts;
+//   * v_mfma_f32_16x16x32_f16, fp32 accumulators in named accumulation
+//     registers, 64-lane wavefronts;
 //   * tiles go HBM/L2 -> LDS with global_load_lds_dwordx4 (no VGPR staging);
 //     the LDS image is forced to be linear in lane order, so the XOR swizzle
 //     that keeps ds_read_b128 conflict-free is applied on the global side:
 //     the lane that owns LDS slot (row, c') fetches K-chunk c' ^ swz(row);
-//   * LDS is multi-buffered (STAGES), one workgroup barrier per K tile;
-//   * each stage is its own __shared__ object so the compiler can tell that a
-//     tile in flight does not alias the tile being read.
+//   * the A half and the B half of a K tile are slots of a five-slot LDS ring,
+//     one workgroup barrier per K tile, in the middle of the tile.
 #pragma once
 
 #include "ccf_common.h"
@@ -140,314 +140,27 @@ __device__ __forceinline__ int fresh_tid() {
   return t;
 }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int WGS_PER_CU_ = 1,
-          int DMA_EVERY_ = 2, int SCHED_ = 0>
+// Tile shape (BM x BN x BK), wavefront grid (WM x WN) and the pacing of the tile loads.
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int DMA_EVERY_>
 struct GemmCfg {
-  // 0: every wavefront interleaves MFMAs, LDS reads and tile loads.
-  // 1, 2: ping-pong.  The wavefronts form two groups (1: by wave/4, the two that
-  // share a SIMD; 2: by wave%2) that alternate between a memory phase (LDS
-  // fragment reads + tile loads) and a compute phase (a burst of MFMAs on
-  // fragments already in registers), one workgroup barrier per phase, so that
-  // a stall while issuing memory instructions never delays an MFMA.
-  // 3: as 0, with the K tiles held in the five-slot ring (RingMainloop).
-  static constexpr int SCHED = SCHED_;
   static constexpr int DMA_EVERY = DMA_EVERY_;         // one tile load behind every n-th MFMA
-  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr int NW = WM * WN;
-  static constexpr int WGS_PER_CU = WGS_PER_CU_;
-  static constexpr int MIN_WAVES_PER_SIMD = (NW * WGS_PER_CU + 3) / 4;   // register budget
+  static constexpr int MIN_WAVES_PER_SIMD = (NW + 3) / 4;   // register budget
   static constexpr int THREADS = NW * 64;
   static constexpr int WTM = BM / WM, WTN = BN / WN;   // wavefront tile
-  static constexpr int TM = WTM / 32, TN = WTN / 32;   // 32x32 MFMA blocks per wavefront
   static constexpr int CPR = BK / 8;                   // 16-byte chunks per tile row
   static constexpr int ROWS_PER_DMA = 64 / CPR;        // tile rows one wavefront load covers
   static constexpr int A_DMA = BM / ROWS_PER_DMA / NW; // loads per wavefront per tile
   static constexpr int B_DMA = BN / ROWS_PER_DMA / NW;
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int KSTEPS = BK / 16;
-  static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wavefront tile");
+  static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "wavefront tile");
   static_assert(BM % (ROWS_PER_DMA * NW) == 0 && BN % (ROWS_PER_DMA * NW) == 0, "dma split");
-  static_assert(STAGES >= 2 && STAGES <= 6, "stages");
 };
 
-// One workgroup's main loop.  a_row_ptr(r) / b_row_ptr(r) give the global
-// address of K element 0 of tile row r (already clamped to a valid row).
+// Which rows of a tile, and which 16-byte K chunk of them, a lane fetches with its tile loads.
 template <class Cfg>
 struct GemmMainloop {
-  using acc_t = float16v;
-
-  template <int S>
-  static __device__ __forceinline__ lds_char *stage() {
-    return stage_buf<S, Cfg::STAGE_BYTES>();
-  }
-
-  // Issue the loads of one K tile into stage S.
-  template <int S>
-  static __device__ __forceinline__ void issue(const half_t *const (&a_src)[Cfg::A_DMA],
-                                               const half_t *const (&b_src)[Cfg::B_DMA],
-                                               int k_elem, int wave) {
-    lds_char *base = stage<S>();
-#pragma unroll
-    for (int i = 0; i < Cfg::A_DMA; ++i)
-      lds_dma16(a_src[i] + k_elem, base + (i * Cfg::NW + wave) * 1024);
-#pragma unroll
-    for (int i = 0; i < Cfg::B_DMA; ++i)
-      lds_dma16(b_src[i] + k_elem, base + Cfg::A_BYTES + (i * Cfg::NW + wave) * 1024);
-  }
-
-  // Order in which the TM+TN operand fragments of one K step are read from
-  // LDS: a0, b0 .. b(TN-1), a1 .. a(TM-1), so that the first MFMA of the step
-  // can issue as early as possible.
-  static constexpr int FRAGS = Cfg::TM + Cfg::TN;
-  static constexpr int a_seq(int tm) { return tm == 0 ? 0 : Cfg::TN + tm; }
-  static constexpr int b_seq(int tn) { return 1 + tn; }
-
-  template <int S, int KS, int I>
-  static __device__ __forceinline__ void read_frag(half8 (&a)[Cfg::TM], half8 (&b)[Cfg::TN],
-                                                   const int (&a_off)[Cfg::KSTEPS],
-                                                   const int (&b_off)[Cfg::KSTEPS]) {
-    const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage<S>()));
-    if constexpr (I == 0) {
-      a[0] = lds_read_b128<0>(base + a_off[KS]);
-    } else if constexpr (I <= Cfg::TN) {
-      b[I - 1] = lds_read_b128<Cfg::A_BYTES + (I - 1) * 32 * Cfg::CPR * 16>(base + b_off[KS]);
-    } else {
-      a[I - Cfg::TN] = lds_read_b128<(I - Cfg::TN) * 32 * Cfg::CPR * 16>(base + a_off[KS]);
-    }
-  }
-
-  // The i-th tile load of this wavefront (A loads first, then B) into stage S.
-  template <int S, int I>
-  static __device__ __forceinline__ void issue_one(const half_t *const (&a_src)[Cfg::A_DMA],
-                                                   const half_t *const (&b_src)[Cfg::B_DMA],
-                                                   int k_elem, int wave) {
-    lds_char *base = stage<S>();
-    if constexpr (I < Cfg::A_DMA) {
-      lds_dma16(a_src[I] + k_elem, base + (I * Cfg::NW + wave) * 1024);
-    } else {
-      lds_dma16(b_src[I - Cfg::A_DMA] + k_elem,
-                base + Cfg::A_BYTES + ((I - Cfg::A_DMA) * Cfg::NW + wave) * 1024);
-    }
-  }
-
-  // MFMAs over the K tile held in stage S.  The fragments of K step ks+1 are
-  // read between the MFMAs of step ks into a second register set, and (PREFETCH)
-  // the loads of a later K tile into stage NEXT are issued between MFMAs too,
-  // one behind every DMA_EVERY-th MFMA from the start of the tile: a wavefront
-  // issues in order, so a tile load that waits for a free slot in the texture
-  // address queue would otherwise hold up every MFMA behind it, while issued in
-  // the shadow of an MFMA (32 clocks in the pipe) it costs nothing.  The LDS
-  // reads are inline asm (the compiler would otherwise make every LDS read
-  // wait for the tile loads in flight), so the lgkmcnt waits are placed here:
-  // LDS reads return in order, and before MFMA i of a step the reads still
-  // allowed in flight are the later fragments of this step plus the fragments
-  // of the next step issued so far.  Scheduling fences keep the source order.
-  template <int S, int NEXT, bool PREFETCH>
-  static __device__ __forceinline__ void compute(acc_t (&acc)[Cfg::TM][Cfg::TN],
-                                                 const half_t *const (&a_src)[Cfg::A_DMA],
-                                                 const half_t *const (&b_src)[Cfg::B_DMA],
-                                                 const int (&a_off)[Cfg::KSTEPS],
-                                                 const int (&b_off)[Cfg::KSTEPS], int k_pre,
-                                                 int wave) {
-    constexpr int PER_STEP = Cfg::TM * Cfg::TN;
-    constexpr int PER_TILE = Cfg::A_DMA + Cfg::B_DMA;
-    half8 a[2][Cfg::TM], b[2][Cfg::TN];
-    if constexpr (PREFETCH && Cfg::DMA_EVERY == 0) {       // all tile loads up front
-      static_for<0, PER_TILE>([&](auto I) { issue_one<NEXT, I.value>(a_src, b_src, k_pre, wave); });
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    static_for<0, FRAGS>([&](auto I) { read_frag<S, 0, I.value>(a[0], b[0], a_off, b_off); });
-    __builtin_amdgcn_sched_barrier(0);
-    static_for<0, Cfg::KSTEPS>([&](auto KS) {
-      constexpr int ks = KS.value;
-      constexpr int cur = ks & 1;
-      constexpr bool more = ks + 1 < Cfg::KSTEPS;
-      static_for<0, PER_STEP>([&](auto II) {
-        constexpr int i = II.value;
-        constexpr int tm = i / Cfg::TN, tn = i % Cfg::TN;
-        constexpr int need = a_seq(tm) > b_seq(tn) ? a_seq(tm) : b_seq(tn);
-        constexpr int next_issued = more ? (i < FRAGS ? i : FRAGS) : 0;
-        wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
-        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
-        if constexpr (more && i < FRAGS) read_frag<S, ks + 1, i>(a[cur ^ 1], b[cur ^ 1], a_off, b_off);
-        constexpr int m = ks * PER_STEP + i;                 // MFMA index within the tile
-        if constexpr (PREFETCH && Cfg::DMA_EVERY > 0) {
-          if constexpr (m % (Cfg::DMA_EVERY > 0 ? Cfg::DMA_EVERY : 1) == 0 &&
-                        m / (Cfg::DMA_EVERY > 0 ? Cfg::DMA_EVERY : 1) < PER_TILE)
-            issue_one<NEXT, m / (Cfg::DMA_EVERY > 0 ? Cfg::DMA_EVERY : 1)>(a_src, b_src, k_pre, wave);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      });
-    });
-    // a tile with fewer MFMAs than load slots: issue the rest now
-    if constexpr (PREFETCH && Cfg::DMA_EVERY > 0) {
-      constexpr int slots = (Cfg::KSTEPS * PER_STEP + Cfg::DMA_EVERY - 1) / (Cfg::DMA_EVERY > 0 ? Cfg::DMA_EVERY : 1);
-      static_for<(slots < PER_TILE ? slots : PER_TILE), PER_TILE>(
-          [&](auto I) { issue_one<NEXT, I.value>(a_src, b_src, k_pre, wave); });
-    }
-  }
-
-  template <int S>
-  struct Step {
-    static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
-                                               const half_t *const (&a_src)[Cfg::A_DMA],
-                                               const half_t *const (&b_src)[Cfg::B_DMA],
-                                               const int (&a_off)[Cfg::KSTEPS],
-                                               const int (&b_off)[Cfg::KSTEPS], int kt, int KT,
-                                               int wave) {
-      constexpr int NEXT = (S + Cfg::STAGES - 1) % Cfg::STAGES;   // stage of tile kt+STAGES-1
-      constexpr int PER_TILE = Cfg::A_DMA + Cfg::B_DMA;
-      if (kt >= KT) return;                                        // uniform
-      // Past the end the prefetch re-reads the last K tile into a stage nobody
-      // reads any more: the loop stays free of branches and the wait counts fixed.
-      int kpre = kt + Cfg::STAGES - 1;
-      kpre = kpre < KT ? kpre : KT - 1;
-      compute<S, NEXT, true>(acc, a_src, b_src, a_off, b_off, kpre * Cfg::BK, wave);
-      // tile kt+1 must have landed before anyone reads it: leave at most the
-      // loads of the STAGES-2 younger tiles in flight.
-      wait_vmcnt<PER_TILE *(Cfg::STAGES - 2)>();
-      block_barrier();
-    }
-  };
-
-  static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
-                                             const half_t *const (&a_src)[Cfg::A_DMA],
-                                             const half_t *const (&b_src)[Cfg::B_DMA], int K) {
-    const int wave = threadIdx.x >> 6;
-    const int lane = threadIdx.x & 63;
-    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-    const int KT = K / Cfg::BK;
-
-    // Per-lane LDS read offsets: row = lane % 32 of each 32x32 block, K-chunk
-    // 2*ks + lane/32.
-    int a_off[Cfg::KSTEPS], b_off[Cfg::KSTEPS];
-    {
-      const int ra = wm * Cfg::WTM + (lane & 31);
-      const int rb = wn * Cfg::WTN + (lane & 31);
-#pragma unroll
-      for (int ks = 0; ks < Cfg::KSTEPS; ++ks) {
-        const int c = ks * 2 + (lane >> 5);
-        a_off[ks] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
-        b_off[ks] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
-      }
-    }
-
-    // Prologue: tiles 0 .. STAGES-2.
-    static_for<0, Cfg::STAGES - 1>([&](auto S) {
-      if (S.value < KT) issue<S.value>(a_src, b_src, S.value * Cfg::BK, wave);
-    });
-    // tile 0 landed; younger prologue tiles may stay in flight
-    if (KT >= Cfg::STAGES - 1) {
-      wait_vmcnt<(Cfg::A_DMA + Cfg::B_DMA) * (Cfg::STAGES - 2)>();
-    } else {
-      wait_vmcnt<0>();
-    }
-    block_barrier();
-
-    for (int kt0 = 0; kt0 < KT; kt0 += Cfg::STAGES) {
-      static_for<0, Cfg::STAGES>([&](auto S) {
-        Step<S.value>::run(acc, a_src, b_src, a_off, b_off, kt0 + S.value, KT, wave);
-      });
-    }
-    wait_vmcnt<0>();      // the redundant tail prefetches
-  }
-
-  // ---- ping-pong schedule ---------------------------------------------------
-  // Barrier that first waits for every LDS read in flight; the fragment
-  // registers are tied to the wait so no MFMA can be scheduled above it.
-  static __device__ __forceinline__ void pp_barrier_after_reads(half8 (&a)[Cfg::KSTEPS][Cfg::TM],
-                                                                half8 (&b)[Cfg::KSTEPS][Cfg::TN]) {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int ks = 0; ks < Cfg::KSTEPS; ++ks) {
-#pragma unroll
-      for (int i = 0; i < Cfg::TM; ++i) asm volatile("" : "+v"(a[ks][i]));
-#pragma unroll
-      for (int i = 0; i < Cfg::TN; ++i) asm volatile("" : "+v"(b[ks][i]));
-    }
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-  }
-
-  template <int S>
-  struct PingPong {
-    // memory phase of K slice kt (held in stage S), then compute phase
-    static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
-                                               const half_t *const (&a_src)[Cfg::A_DMA],
-                                               const half_t *const (&b_src)[Cfg::B_DMA],
-                                               const int (&a_off)[Cfg::KSTEPS],
-                                               const int (&b_off)[Cfg::KSTEPS], int kt, int KT,
-                                               int wave) {
-      constexpr int NEXT = (S + Cfg::STAGES - 1) % Cfg::STAGES;
-      constexpr int PER_TILE = Cfg::A_DMA + Cfg::B_DMA;
-      if (kt >= KT) return;                                        // uniform
-      int kpre = kt + Cfg::STAGES - 1;
-      kpre = kpre < KT ? kpre : KT - 1;
-      half8 a[Cfg::KSTEPS][Cfg::TM], b[Cfg::KSTEPS][Cfg::TN];
-      // --- memory phase
-      static_for<0, Cfg::KSTEPS>([&](auto KS) {
-        static_for<0, FRAGS>([&](auto I) {
-          read_frag<S, KS.value, I.value>(a[KS.value], b[KS.value], a_off, b_off);
-        });
-      });
-      static_for<0, PER_TILE>([&](auto I) { issue_one<NEXT, I.value>(a_src, b_src, kpre * Cfg::BK, wave); });
-      __builtin_amdgcn_sched_barrier(0);
-      wait_vmcnt<PER_TILE *(Cfg::STAGES - 2)>();
-      pp_barrier_after_reads(a, b);
-      // --- compute phase
-      static_for<0, Cfg::KSTEPS>([&](auto KS) {
-        static_for<0, Cfg::TM * Cfg::TN>([&](auto II) {
-          constexpr int tm = II.value / Cfg::TN, tn = II.value % Cfg::TN;
-          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[KS.value][tn], a[KS.value][tm],
-                                                               acc[tm][tn], 0, 0, 0);
-        });
-      });
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  static __device__ __forceinline__ void run_pingpong(acc_t (&acc)[Cfg::TM][Cfg::TN],
-                                                      const half_t *const (&a_src)[Cfg::A_DMA],
-                                                      const half_t *const (&b_src)[Cfg::B_DMA],
-                                                      int K) {
-    const int wave = threadIdx.x >> 6;
-    const int lane = threadIdx.x & 63;
-    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-    const int KT = K / Cfg::BK;
-    const int group = Cfg::SCHED == 1 ? (wave >> 2) & 1 : wave & 1;
-    int a_off[Cfg::KSTEPS], b_off[Cfg::KSTEPS];
-    {
-      const int ra = wm * Cfg::WTM + (lane & 31);
-      const int rb = wn * Cfg::WTN + (lane & 31);
-#pragma unroll
-      for (int ks = 0; ks < Cfg::KSTEPS; ++ks) {
-        const int c = ks * 2 + (lane >> 5);
-        a_off[ks] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
-        b_off[ks] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
-      }
-    }
-    // Prologue: slices 0 .. STAGES-2 (past the end: the last slice again).
-    static_for<0, Cfg::STAGES - 1>([&](auto S) {
-      const int k = S.value < KT ? S.value : KT - 1;
-      issue<S.value>(a_src, b_src, k * Cfg::BK, wave);
-    });
-    wait_vmcnt<(Cfg::A_DMA + Cfg::B_DMA) * (Cfg::STAGES - 2)>();
-    block_barrier();
-    // The second group runs one phase behind the first.
-    if (group == 1) __builtin_amdgcn_s_barrier();
-    for (int kt0 = 0; kt0 < KT; kt0 += Cfg::STAGES) {
-      static_for<0, Cfg::STAGES>([&](auto S) {
-        PingPong<S.value>::run(acc, a_src, b_src, a_off, b_off, kt0 + S.value, KT, wave);
-      });
-    }
-    if (group == 0) __builtin_amdgcn_s_barrier();
-    wait_vmcnt<0>();
-  }
-
   // Tile row this lane fetches with its i-th A (or B) load, and the K-chunk.
   // tid: threadIdx.x, or fresh_tid() where the values derived from it must not
   // be computed early and kept in registers.
@@ -463,154 +176,13 @@ struct GemmMainloop {
   static __device__ __forceinline__ int dma_chunk(int row) { return dma_chunk(row, threadIdx.x); }
 };
 
-// ---- five-slot ring ------------------------------------------------------------
+// ---- five-slot ring, v_mfma_f32_16x16x32_f16, barrier in mid-tile ----------------
 // 256x256x64 tiles need 64 KB of LDS per K tile, so only two whole tiles fit in
-// the CU's 160 KB, and with two stages a tile's loads must all have landed
-// before the next tile's can be issued: the memory pipe drains once per K tile
-// (measured: 12 TB/s into LDS against 16 TB/s when loads of two tiles overlap).
-// Here the A half and the B half of a K tile are separate 32 KB slots of a ring
-// of five.  While tile k is computed, A(k+1) is resident, B(k+1) and A(k+2) are
-// in flight; at the end of the step only B(k+1) must have landed, A(k+2) keeps
-// flying across the barrier.  Every load is a whole 128-byte line and there is
-// still one barrier per K tile.
-template <class Cfg>
-struct RingMainloop {
-  using acc_t = float16v;
-  using Base = GemmMainloop<Cfg>;
-  static_assert(Cfg::A_BYTES == Cfg::B_BYTES, "ring slots are one size");
-  static constexpr int NSLOT = 5;
-  static constexpr int FRAGS = Cfg::TM + Cfg::TN;
-
-  template <int S>
-  static __device__ __forceinline__ lds_char *slot() {
-    return stage_buf<100 + S, Cfg::A_BYTES>();
-  }
-
-  template <int SLOT, int N>
-  static __device__ __forceinline__ void issue_all(const half_t *const (&src)[N], int k_elem, int wave) {
-    static_for<0, N>([&](auto I) {
-      lds_dma16(src[I.value] + k_elem, slot<SLOT>() + (I.value * Cfg::NW + wave) * 1024);
-    });
-  }
-
-  template <int SA, int SB, int KS, int I>
-  static __device__ __forceinline__ void read_frag(half8 (&a)[Cfg::TM], half8 (&b)[Cfg::TN],
-                                                   const int (&a_off)[Cfg::KSTEPS],
-                                                   const int (&b_off)[Cfg::KSTEPS]) {
-    const uint32_t base_a = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(slot<SA>()));
-    const uint32_t base_b = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(slot<SB>()));
-    if constexpr (I == 0) {
-      a[0] = lds_read_b128<0>(base_a + a_off[KS]);
-    } else if constexpr (I <= Cfg::TN) {
-      b[I - 1] = lds_read_b128<(I - 1) * 32 * Cfg::CPR * 16>(base_b + b_off[KS]);
-    } else {
-      a[I - Cfg::TN] = lds_read_b128<(I - Cfg::TN) * 32 * Cfg::CPR * 16>(base_a + a_off[KS]);
-    }
-  }
-
-  // FULL: every 32-row block of this wavefront holds real rows.  Otherwise only
-  // the first live_m blocks do (the tail tile of an expert), and the MFMAs of
-  // the padded blocks are skipped: they would only burn power.
-  template <int U, bool FULL>
-  struct Step {
-    static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
-                                               const half_t *const (&a_src)[Cfg::A_DMA],
-                                               const half_t *const (&b_src)[Cfg::B_DMA],
-                                               const int (&a_off)[Cfg::KSTEPS],
-                                               const int (&b_off)[Cfg::KSTEPS], int kt, int KT,
-                                               int wave, int live_m) {
-      constexpr int SA = (2 * U) % NSLOT, SB = (2 * U + 1) % NSLOT;       // tile kt
-      constexpr int WB = (2 * U + 3) % NSLOT, WA = (2 * U + 4) % NSLOT;   // B(kt+1), A(kt+2)
-      constexpr int PER_STEP = Cfg::TM * Cfg::TN;
-      constexpr int LOADS = Cfg::A_DMA + Cfg::B_DMA;
-      if (kt >= KT) return;                                               // uniform
-      // past the end the last K tile is fetched again into slots nobody reads
-      const int kb = ((kt + 1 < KT) ? kt + 1 : KT - 1) * Cfg::BK;
-      const int ka = ((kt + 2 < KT) ? kt + 2 : KT - 1) * Cfg::BK;
-      half8 a[2][Cfg::TM], b[2][Cfg::TN];
-      static_for<0, FRAGS>([&](auto I) { read_frag<SA, SB, 0, I.value>(a[0], b[0], a_off, b_off); });
-      __builtin_amdgcn_sched_barrier(0);
-      static_for<0, Cfg::KSTEPS>([&](auto KS) {
-        constexpr int ks = KS.value;
-        constexpr int cur = ks & 1;
-        constexpr bool more = ks + 1 < Cfg::KSTEPS;
-        static_for<0, PER_STEP>([&](auto II) {
-          constexpr int i = II.value;
-          constexpr int tm = i / Cfg::TN, tn = i % Cfg::TN;
-          constexpr int need = Base::a_seq(tm) > Base::b_seq(tn) ? Base::a_seq(tm) : Base::b_seq(tn);
-          constexpr int next_issued = more ? (i < FRAGS ? i : FRAGS) : 0;
-          wait_lgkmcnt<FRAGS - 1 - need + next_issued>(a[cur][tm], b[cur][tn]);
-          if (FULL || tm < live_m)
-            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[cur][tn], a[cur][tm], acc[tm][tn], 0, 0, 0);
-          if constexpr (more && i < FRAGS) read_frag<SA, SB, ks + 1, i>(a[cur ^ 1], b[cur ^ 1], a_off, b_off);
-          constexpr int m = ks * PER_STEP + i;
-          if constexpr (m % Cfg::DMA_EVERY == 0 && m / Cfg::DMA_EVERY < LOADS) {
-            constexpr int l = m / Cfg::DMA_EVERY;                         // B loads first, then A
-            if constexpr (l < Cfg::B_DMA) {
-              lds_dma16(b_src[l] + kb, slot<WB>() + (l * Cfg::NW + wave) * 1024);
-            } else {
-              lds_dma16(a_src[l - Cfg::B_DMA] + ka, slot<WA>() + ((l - Cfg::B_DMA) * Cfg::NW + wave) * 1024);
-            }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      });
-      static_assert((Cfg::KSTEPS * PER_STEP + Cfg::DMA_EVERY - 1) / Cfg::DMA_EVERY >= LOADS,
-                    "not enough MFMA slots for the tile loads");
-      // B(kt+1) and everything older have landed; A(kt+2) may stay in flight
-      wait_vmcnt<Cfg::A_DMA>();
-      block_barrier();
-    }
-  };
-
-  // rows: real rows of this M tile (1..BM).
-  static __device__ __forceinline__ void run(acc_t (&acc)[Cfg::TM][Cfg::TN],
-                                             const half_t *const (&a_src)[Cfg::A_DMA],
-                                             const half_t *const (&b_src)[Cfg::B_DMA], int K,
-                                             int rows) {
-    const int wave = threadIdx.x >> 6;
-    const int lane = threadIdx.x & 63;
-    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-    const int KT = K / Cfg::BK;
-    int live_m = (rows - wm * Cfg::WTM + 31) / 32;       // 32-row blocks of this wavefront with real rows
-    live_m = live_m < 0 ? 0 : (live_m > Cfg::TM ? Cfg::TM : live_m);
-    live_m = __builtin_amdgcn_readfirstlane(live_m);
-    int a_off[Cfg::KSTEPS], b_off[Cfg::KSTEPS];
-    {
-      const int ra = wm * Cfg::WTM + (lane & 31);
-      const int rb = wn * Cfg::WTN + (lane & 31);
-#pragma unroll
-      for (int ks = 0; ks < Cfg::KSTEPS; ++ks) {
-        const int c = ks * 2 + (lane >> 5);
-        a_off[ks] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
-        b_off[ks] = (rb * Cfg::CPR + (c ^ swz<Cfg::CPR>(rb))) * 16;
-      }
-    }
-    // Prologue: A(0) -> slot 0, B(0) -> slot 1, A(1) -> slot 2.
-    issue_all<0>(a_src, 0, wave);
-    issue_all<1>(b_src, 0, wave);
-    issue_all<2>(a_src, (KT > 1 ? 1 : 0) * Cfg::BK, wave);
-    wait_vmcnt<Cfg::A_DMA>();
-    block_barrier();
-    if (live_m == Cfg::TM) {
-      for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
-        static_for<0, NSLOT>([&](auto U) {
-          Step<U.value, true>::run(acc, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave, live_m);
-        });
-      }
-    } else {
-      for (int kt0 = 0; kt0 < KT; kt0 += NSLOT) {
-        static_for<0, NSLOT>([&](auto U) {
-          Step<U.value, false>::run(acc, a_src, b_src, a_off, b_off, kt0 + U.value, KT, wave, live_m);
-        });
-      }
-    }
-    wait_vmcnt<0>();
-  }
-};
-
-// ---- five-slot ring, v_mfma_f32_16x16x32_f16, early barrier ----------------------
-// Same ring of A and B half-tile slots, with three differences.
+// the CU's 160 KB, and with two whole-tile stages a tile's loads must all have
+// landed before the next tile's can be issued: the memory pipe drains once per K
+// tile (measured: 12 TB/s into LDS against 16 TB/s when loads of two tiles
+// overlap).  Here the A half and the B half of a K tile are separate 32 KB slots
+// of a ring of five; every load is a whole 128-byte line.
 //
 // * The MFMA is the 16x16x32 form.  It moves a quarter of the accumulator
 //   registers per flop of the 32x32x16 form, and on data that is not constant
@@ -958,24 +530,6 @@ template <class Cfg>
 __device__ __forceinline__ int acc16_col4(int tn, int tid) {
   const int wave = tid >> 6, lane = tid & 63;
   return (wave % Cfg::WN) * Cfg::WTN + tn * 16 + 4 * (lane >> 4);
-}
-
-// The weight fragment is the first MFMA operand and the token fragment the
-// second, so a lane owns ONE token row per 32x32 block and, per group of four
-// accumulator registers, four consecutive output columns:
-//   row = wm*WTM + tm*32 + lane%32
-//   col = wn*WTN + tn*32 + 8*(r/4) + 4*(lane/32) + r%4
-// which lets the epilogue look up row data once per block and store 8 bytes at
-// a time.
-template <class Cfg>
-__device__ __forceinline__ int acc_row(int tm) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  return (wave / Cfg::WN) * Cfg::WTM + tm * 32 + (lane & 31);
-}
-template <class Cfg>
-__device__ __forceinline__ int acc_col4(int tn, int q) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  return (wave % Cfg::WN) * Cfg::WTN + tn * 32 + 8 * q + 4 * (lane >> 5);
 }
 
 }  // namespace ccf

@@ -1,4 +1,7 @@
-// Measurement probe: what the matrix cores sustain with nothing else in the way.
+// libccfuser_probe.so: two measurement probes, built apart from the product library
+// (libccfuser_moe.so exports the MoE path only).  Neither has a counterpart in the reference.
+//
+// 1. What the matrix cores sustain with nothing else in the way.
 //
 // One workgroup of four wavefronts per CU (the grouped GEMM's shape: one wavefront per SIMD,
 // 8 x 8 blocks of v_mfma_f32_16x16x32_f16 per wavefront) issues MFMAs back to back on operand
@@ -6,13 +9,22 @@
 // the chip reaches its nominal rate; with random operands the same loop runs slower, because
 // the data-dependent switching power makes the power limit lower the clock.  That second
 // figure is the ceiling any fp16 GEMM on real data has on this hardware; bench.py reports it
-// beside the nominal peak.  No counterpart in the reference.
-#include "ccf_common.h"
+// beside the nominal peak.
+//
+// 2. The arithmetic the fp16 gate rests on: a chain of K = 1 fp32 MFMAs on one wavefront, for a
+// test that compares every accumulator with a chain of fused multiply-adds on the CPU.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-#include <type_traits>
+#include "../../include/ccfuser_probe.h"
+#include "mfma_f32.h"
 
 namespace ccf {
 namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? 0 : 4; }
 
 __device__ inline half8 probe_fragment(unsigned &x, float scale, int constant) {
   half8 v;
@@ -78,13 +90,45 @@ mfma_probe_kernel(float *out, int iters, int constant) {
 }  // namespace ccf
 
 extern "C" int ccf_probe_mfma(int workgroups, int iters, int constant_operands, void *out, double *flop,
-                              ccf_stream_t stream) {
+                              void *stream) {
   using namespace ccf;
-  CCF_REQUIRE(out && flop, CCF_ERR_ARG, "probe_mfma: null pointer");
-  CCF_REQUIRE(workgroups > 0 && workgroups <= 4096 && iters > 0, CCF_ERR_ARG, "probe_mfma: bad size");
-  hipLaunchKernelGGL(mfma_probe_kernel, dim3(workgroups), dim3(256), 0, as_stream(stream), static_cast<float *>(out),
-                     iters, constant_operands);
+  if (!out || !flop || workgroups <= 0 || workgroups > 4096 || iters <= 0) return 1;
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<float *>(out), iters, constant_operands);
   // 4 wavefronts x iters x 64 MFMAs of 16 x 16 x 32 x 2 flop
   *flop = static_cast<double>(workgroups) * 4.0 * iters * (kProbeBlocks * kProbeBlocks) * (16.0 * 16.0 * 32.0 * 2.0);
-  return check_launch("mfma_probe_kernel");
+  return launch_status();
+}
+
+namespace ccf {
+namespace {
+
+// One wavefront runs a chain of `steps` K = 1 fp32 MFMAs, acc = mfma(a[s][lane], b[s][lane], acc),
+// and leaves its accumulator registers as out[reg][lane].
+template <int N>
+__global__ void __launch_bounds__(64)
+mfma_chain_probe_kernel(const float *__restrict__ a, const float *__restrict__ b, int steps,
+                        float *__restrict__ out) {
+  using M = Mfma<N>;
+  typename M::Acc acc;
+#pragma unroll
+  for (int v = 0; v < M::kRegs; ++v) acc[v] = 0.0f;
+  const int lane = threadIdx.x;
+  for (int s = 0; s < steps; ++s) acc = M::run(a[s * 64 + lane], b[s * 64 + lane], acc);
+#pragma unroll
+  for (int v = 0; v < M::kRegs; ++v) out[v * 64 + lane] = acc[v];
+}
+
+}  // namespace
+}  // namespace ccf
+
+extern "C" int ccf_probe_mfma_chain(const float *a, const float *b, int steps, int tile, float *out, void *stream) {
+  using namespace ccf;
+  if (!a || !b || !out || steps < 0 || (tile != 16 && tile != 32)) return 1;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (tile == 32)
+    hipLaunchKernelGGL(mfma_chain_probe_kernel<32>, dim3(1), dim3(64), 0, st, a, b, steps, out);
+  else
+    hipLaunchKernelGGL(mfma_chain_probe_kernel<16>, dim3(1), dim3(64), 0, st, a, b, steps, out);
+  return launch_status();
 }

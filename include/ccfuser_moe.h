@@ -55,7 +55,8 @@ const char *ccf_last_error(void);
 /*
  * Tuning knobs (no counterpart in the reference).  Process-wide; not meant to
  * be changed while work is in flight.
- *   "gemm_variant"    grouped-GEMM main-loop variant of the FFN entry points; -1 restores the default
+ *   "gemm_variant"    0 (default, also -1) = the grouped GEMMs run as persistent workgroups, one per CU;
+ *                     1 = one workgroup per tile for every K (otherwise only K < 256 runs that way)
  *   "split_tail"      0 = off, 1 = default, n > 1 = for K of n*64 and more: the tiles of a launch's
  *                     last, partly filled round are cut along K and reduced by a second kernel
  *   "split_parts"     2..8 (default 8): most parts such a tile is cut into
@@ -297,30 +298,6 @@ int ccf_moe_forward(const void *x, const void *wg, const void *bg,
  * [0] and [1] or [4] and [5].  count = 0 switches the recording off.
  */
 int ccf_moe_forward_set_events(void *const *events, int count);
-
-/*
- * Measurement probe (no counterpart in the reference): `workgroups` workgroups of four
- * wavefronts issue `iters` x 64 v_mfma_f32_16x16x32_f16 each on register operands, constant
- * (zeros) or pseudo-random, with no memory traffic; *flop receives the flop count of the launch.
- * Timed with events by the caller it gives the rate the matrix cores sustain: the nominal peak
- * with constant operands, a lower, power-limited figure with random ones.
- *   out: device buffer of workgroups * 256 floats (sums that keep the loop alive).
- */
-int ccf_probe_mfma(int workgroups, int iters, int constant_operands, void *out, double *flop,
-                   ccf_stream_t stream);
-
-/*
- * Probe of the arithmetic the fp16 gate rests on (no counterpart in the reference): one
- * wavefront runs a chain of `steps` K = 1 fp32 MFMAs, acc = mfma(a[s][lane], b[s][lane], acc),
- * with v_mfma_f32_32x32x1_2b_f32 (tile = 32: two 32 x 32 blocks, 32 accumulator registers) or
- * v_mfma_f32_16x16x1_4b_f32 (tile = 16: four 16 x 16 blocks, 16 registers), and writes its
- * accumulator registers as out[reg][lane].  Block b takes rows from a and columns from b of
- * lanes b*tile .. b*tile + tile - 1.  The tests compare every output with a chain of fused
- * multiply-adds on the CPU.
- *   a, b: device, [steps][64] floats; out: device, [tile][64] floats.
- */
-int ccf_probe_mfma_chain(const float *a, const float *b, int steps, int tile, float *out,
-                         ccf_stream_t stream);
 
 /* Bytes of workspace ccf_moe_ffn_segments needs. */
 size_t ccf_segments_workspace_bytes(int total_rows, int n_seg, int num_expert,

@@ -45,6 +45,55 @@ def test_every_declaration_cites_the_reference_or_says_it_has_none():
         assert ok, f"{name}: declaration comment names no reference interface"
 
 
+def _split_args(text, start):
+    """Arguments of the call whose opening parenthesis is at text[start]: split at top-level commas."""
+    depth, args, cur = 0, [], []
+    for ch in text[start:]:
+        if ch in "([{":
+            depth += 1
+            if depth == 1:
+                continue
+        elif ch in ")]}":
+            depth -= 1
+            if depth == 0:
+                break
+        if ch == "," and depth == 1:
+            args.append("".join(cur).strip())
+            cur = []
+        else:
+            cur.append(ch)
+    last = "".join(cur).strip()
+    if last and last != "void":
+        args.append(last)
+    return args
+
+
+def header_arity():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    return {m.group(1): len(_split_args(text, m.end() - 1)) for m in re.finditer(r"\b(ccf_[a-z0-9_]+)\s*\(", text)}
+
+
+def test_integration_guide_calls_match_the_header():
+    """Every ccf_*( call inside a code block of INTEGRATION.md passes as many arguments as the
+    header declares for that function, so the guide's snippets cannot drift from the ABI."""
+    arity = header_arity()
+    guide = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = re.findall(r"```(?:cpp|c)\n(.*?)```", guide, flags=re.S)
+    assert blocks, "no C/C++ code block found in INTEGRATION.md"
+    seen = 0
+    for code in blocks:
+        code = re.sub(r"/\*.*?\*/", "", code, flags=re.S)
+        code = re.sub(r"//[^\n]*", "", code)
+        for m in re.finditer(r"\b(ccf_[a-z0-9_]+)\s*\(", code):
+            name = m.group(1)
+            assert name in arity, f"INTEGRATION.md calls {name}, which the header does not declare"
+            got = len(_split_args(code, m.end() - 1))
+            assert got == arity[name], f"INTEGRATION.md passes {got} arguments to {name}; the header declares {arity[name]}"
+            seen += 1
+    assert seen >= 4
+
+
 def test_version_and_sizes(lib):
     assert lib.ccf_version() >= 100
     assert lib.ccf_route_workspace_bytes(32768, 32) > 0

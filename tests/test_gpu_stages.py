@@ -177,8 +177,8 @@ def test_mfma_chain_equals_a_chain_of_fused_multiply_adds(tile):
         a, b = operands(), operands()
         out = torch.full((regs, 64), float("nan"), dtype=torch.float32, device="cuda")
         a_dev, b_dev = a.cuda(), b.cuda()
-        _lib.call("ccf_probe_mfma_chain", a_dev.data_ptr(), b_dev.data_ptr(), steps, tile,
-                  out.data_ptr(), None)
+        assert _lib.probe_lib().ccf_probe_mfma_chain(a_dev.data_ptr(), b_dev.data_ptr(), steps, tile,
+                                                     out.data_ptr(), None) == 0
         torch.cuda.synchronize()
         got = out.cpu().numpy()
         an, bn = a.numpy(), b.numpy()
@@ -348,7 +348,7 @@ def _ffn_case(R, d, f, E, seed, skew=False):
     return x, w1, b1, w2, b2, e_of_row
 
 
-@pytest.mark.parametrize("variant", list(range(7)))
+@pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("R,d,f,E,skew,seed", [
     (512, 256, 1024, 4, False, 0),
     (700, 768, 3072, 32, True, 1),
@@ -582,16 +582,15 @@ def test_mfma_probe_runs_and_counts_its_flop():
     operands every sum it leaves is zero; the flop count is the closed form."""
     import ctypes as C
     from ccfuser_amd import _lib
-    lib = _lib.lib()
+    probe = _lib.probe_lib()
     wgs, iters = 16, 10
     out = torch.full((wgs * 256,), 7.0, dtype=torch.float32, device="cuda")
     flop = C.c_double()
     for const in (1, 0):
-        _lib.call("ccf_probe_mfma", wgs, iters, const, out.data_ptr(), C.byref(flop), None)
+        assert probe.ccf_probe_mfma(wgs, iters, const, out.data_ptr(), C.byref(flop), None) == 0
         torch.cuda.synchronize()
         assert flop.value == wgs * 4 * iters * 64 * 16 * 16 * 32 * 2
         assert bool(torch.isfinite(out).all())
         if const:
             assert not out.any()
-    with pytest.raises(_lib.CcfError):
-        _lib.call("ccf_probe_mfma", 0, iters, 1, out.data_ptr(), C.byref(flop), None)
+    assert probe.ccf_probe_mfma(0, iters, 1, out.data_ptr(), C.byref(flop), None) == 1
