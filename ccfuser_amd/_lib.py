@@ -37,6 +37,7 @@ SIGNATURES = {
     "ccf_local_gather": (_i, [_p, _p, _p, _i, _i, _p]),
     "ccf_combine": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
     "ccf_ffn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "ccf_ffn_plan_info": (_i, [_p, _i, _i, _i, _i, _i, C.POINTER(C.c_int32), _p]),
     "ccf_ffn1_forward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p, _p, _sz, _p]),
     "ccf_ffn2_forward": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
     "ccf_combine_backward": (_i, [_p, _p, _p, _p, _i, _i, _i, _p, _p, _p]),

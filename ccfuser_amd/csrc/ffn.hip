@@ -54,6 +54,7 @@ struct GroupedArgs {
   float *partial;
   // skinny list (layout in plan.h) of this GEMM, or NULL
   const int32_t *skinny;
+  float *sk_partial;        // partial tiles of the skinny tiles when they run as a launch of their own
 };
 
 // erf-form GELU, v * Phi(v) with Phi(v) = 0.5 + 0.5*erf(v/sqrt2) = 0.5 + u*Q(u^2), u = v
@@ -358,6 +359,104 @@ __device__ __forceinline__ void mfma16_v(float4v &acc, const half8 &w, const hal
   asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(t));
 }
 
+// Accumulators of one 64 x 256 skinny tile: wavefront w owns columns 64 w .. 64 w + 63, block (tm, tn) of a lane is
+// row 16 tm + lane % 16, columns 64 w + 16 tn + 4 (lane / 16) .. + 3.
+typedef float4v SkinnyAcc[SkinnyCfg::TM][SkinnyCfg::TN];
+
+// This lane's fragment chunk of row block 0, per K half (16x16x32 operand: row lane % 16, K chunk lane / 16).
+__device__ __forceinline__ void skinny_frag_offsets(int tid, uint32_t (&a_off)[2], uint32_t (&b_off)[2]) {
+  using C = SkinnyCfg;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int ra = lane & 15, rb = wave * 64 + (lane & 15);
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub) {
+    const int c = sub * 4 + (lane >> 4);
+    a_off[sub] = (ra * 8 + (c ^ swz<8>(ra))) * 16;
+    b_off[sub] = C::A_BYTES + (rb * 8 + (c ^ swz<8>(rb))) * 16;
+  }
+}
+
+// acc = the tile of list entry `ent` over K tiles [kt0, kt0 + nkt) (nkt >= 1), accumulated over K in 32-wide steps
+// in ascending order.  All four wavefronts of the workgroup call it together.
+__device__ __forceinline__ void skinny_mainloop(const GroupedArgs &p, const int4v ent, int kt0, int nkt, SkinnyAcc &acc,
+                                                const uint32_t (&a_off)[2], const uint32_t (&b_off)[2], int tid,
+                                                lds_char *lds, uint32_t lds_base) {
+  using C = SkinnyCfg;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // = the wavefront's 64 columns
+  const int e = ent[0], row0 = ent[1], rows = ent[2], n0 = ent[3] * C::BN;
+  int live_m = (rows + 15) / 16;                                   // 16-row blocks with real rows
+  live_m = __builtin_amdgcn_readfirstlane(live_m > C::TM ? C::TM : live_m);
+  // global source of every tile load of this lane, at K tile kt0
+  const half_t *a_src[C::A_DMA], *b_src[C::B_DMA];
+  const half_t *Be = p.B + static_cast<size_t>(e) * p.N * p.K + static_cast<size_t>(kt0) * C::BK;
+#pragma unroll
+  for (int j = 0; j < C::A_DMA; ++j) {
+    const int r = (j * 4 + wave) * 8 + (lane >> 3);
+    int g = row0 + (r < rows ? r : rows - 1);                      // padded tile rows re-read the last real row
+    if (p.a_rows) g = p.a_rows[g];
+    a_src[j] = p.A + static_cast<size_t>(g) * p.K + static_cast<size_t>(kt0) * C::BK + ((lane & 7) ^ swz<8>(r)) * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < C::B_DMA; ++j) {
+    const int r = (j * 4 + wave) * 8 + (lane >> 3);
+    const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
+    b_src[j] = Be + static_cast<size_t>(n) * p.K + ((lane & 7) ^ swz<8>(r)) * 8;
+  }
+  auto issue = [&](int kt, int stage) {                            // K tile kt0 + kt into a stage
+    const int k_elem = (kt < nkt ? kt : nkt - 1) * C::BK;          // past the end: the last tile again, into a stage nobody reads
+    lds_char *base = lds + stage * C::STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < C::A_DMA; ++j) lds_dma16(a_src[j] + k_elem, base + (j * 4 + wave) * 1024);
+#pragma unroll
+    for (int j = 0; j < C::B_DMA; ++j) lds_dma16(b_src[j] + k_elem, base + C::A_BYTES + (j * 4 + wave) * 1024);
+  };
+#pragma unroll
+  for (int tm = 0; tm < C::TM; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < C::TN; ++tn) acc[tm][tn] = float4v{0, 0, 0, 0};
+  wait_vmcnt<0>();                                                 // the previous tile's stores: the waits below count loads only
+  block_barrier();                                                 // and its last LDS reads are done
+  issue(0, 0);
+  issue(1, 1);
+  issue(2, 2);
+  int stage = 0;
+  for (int kt = 0; kt < nkt; ++kt) {
+    // K tile kt has landed for this wavefront (the loads of the two tiles behind it may be in flight), then for all
+    wait_vmcnt<2 * C::LOADS>();
+    block_barrier();
+    // behind the barrier everyone is done with K tile kt-1, whose stage takes K tile kt+3
+    issue(kt + 3, stage >= 1 ? stage - 1 : C::STAGES - 1);
+    const uint32_t sb = lds_base + stage * C::STAGE_BYTES;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      half8 a[C::TM], b[C::TN];
+      static_for<0, C::TN>([&](auto J) { b[J.value] = lds_read_b128<J.value * 2048>(sb + b_off[sub]); });
+      static_for<0, C::TM>([&](auto I) { a[I.value] = lds_read_b128<I.value * 2048>(sb + a_off[sub]); });
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int q = 0; q < C::TM; ++q) asm volatile("" : "+v"(a[q]));
+#pragma unroll
+      for (int q = 0; q < C::TN; ++q) asm volatile("" : "+v"(b[q]));
+      static_for<0, C::TM>([&](auto I) {
+        constexpr int tm = I.value;
+        if (tm < live_m) {                                         // uniform
+#pragma unroll
+          for (int tn = 0; tn < C::TN; ++tn) mfma16_v(acc[tm][tn], b[tn], a[tm]);
+        }
+      });
+    }
+    stage = stage == C::STAGES - 1 ? 0 : stage + 1;
+  }
+  wait_vmcnt<0>();                                                 // the redundant loads past the end
+  // the MFMAs are opaque to the compiler: keep the distance it would keep before their results are read
+  asm volatile("s_nop 15\n s_nop 15" ::: "memory");
+#pragma unroll
+  for (int tm = 0; tm < C::TM; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < C::TN; ++tn) asm volatile("" : "+v"(acc[tm][tn]));
+}
+
 template <int kEpi>
 __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, int ns, int xcd, lds_char *lds,
                                             uint32_t lds_base) {
@@ -366,95 +465,19 @@ __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, in
   const int T = p.skinny[0], per_x = p.skinny[2];
   const int4v *list = reinterpret_cast<const int4v *>(p.skinny + 4);
   const int tid = fresh_tid(), lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // = the wavefront's 64 columns
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int KT = p.K / C::BK;
-  // this lane's fragment chunk of row block 0, per K half (16x16x32 operand: row lane%16, K chunk lane/16)
   uint32_t a_off[2], b_off[2];
-  {
-    const int ra = lane & 15, rb = wave * 64 + (lane & 15);
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      const int c = sub * 4 + (lane >> 4);
-      a_off[sub] = (ra * 8 + (c ^ swz<8>(ra))) * 16;
-      b_off[sub] = C::A_BYTES + (rb * 8 + (c ^ swz<8>(rb))) * 16;
-    }
-  }
+  skinny_frag_offsets(tid, a_off, b_off);
   for (int i = worker; i < per_x; i += ns) {
     const int w = xcd * per_x + i;
     if (w >= T) break;
     const int4v ent = list[w];
     const int e = ent[0], row0 = ent[1], rows = ent[2], n0 = ent[3] * C::BN;
-    int live_m = (rows + 15) / 16;                                 // 16-row blocks with real rows
+    int live_m = (rows + 15) / 16;
     live_m = __builtin_amdgcn_readfirstlane(live_m > C::TM ? C::TM : live_m);
-    // global source of every tile load of this lane
-    const half_t *a_src[C::A_DMA], *b_src[C::B_DMA];
-    const half_t *Be = p.B + static_cast<size_t>(e) * p.N * p.K;
-#pragma unroll
-    for (int j = 0; j < C::A_DMA; ++j) {
-      const int r = (j * 4 + wave) * 8 + (lane >> 3);
-      int g = row0 + (r < rows ? r : rows - 1);                    // padded tile rows re-read the last real row
-      if (p.a_rows) g = p.a_rows[g];
-      a_src[j] = p.A + static_cast<size_t>(g) * p.K + ((lane & 7) ^ swz<8>(r)) * 8;
-    }
-#pragma unroll
-    for (int j = 0; j < C::B_DMA; ++j) {
-      const int r = (j * 4 + wave) * 8 + (lane >> 3);
-      const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-      b_src[j] = Be + static_cast<size_t>(n) * p.K + ((lane & 7) ^ swz<8>(r)) * 8;
-    }
-    auto issue = [&](int kt, int stage) {                          // K tile kt into a stage
-      const int k_elem = (kt < KT ? kt : KT - 1) * C::BK;          // past the end: the last tile again, into a stage nobody reads
-      lds_char *base = lds + stage * C::STAGE_BYTES;
-#pragma unroll
-      for (int j = 0; j < C::A_DMA; ++j) lds_dma16(a_src[j] + k_elem, base + (j * 4 + wave) * 1024);
-#pragma unroll
-      for (int j = 0; j < C::B_DMA; ++j) lds_dma16(b_src[j] + k_elem, base + C::A_BYTES + (j * 4 + wave) * 1024);
-    };
-    float4v acc[C::TM][C::TN];
-#pragma unroll
-    for (int tm = 0; tm < C::TM; ++tm)
-#pragma unroll
-      for (int tn = 0; tn < C::TN; ++tn) acc[tm][tn] = float4v{0, 0, 0, 0};
-    wait_vmcnt<0>();                                               // the previous tile's stores: the waits below count loads only
-    block_barrier();                                               // and its last LDS reads are done
-    issue(0, 0);
-    issue(1, 1);
-    issue(2, 2);
-    int stage = 0;
-    for (int kt = 0; kt < KT; ++kt) {
-      // K tile kt has landed for this wavefront (the loads of the two tiles behind it may be in flight), then for all
-      wait_vmcnt<2 * C::LOADS>();
-      block_barrier();
-      // behind the barrier everyone is done with K tile kt-1, whose stage takes K tile kt+3
-      issue(kt + 3, stage >= 1 ? stage - 1 : C::STAGES - 1);
-      const uint32_t sb = lds_base + stage * C::STAGE_BYTES;
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
-        half8 a[C::TM], b[C::TN];
-        static_for<0, C::TN>([&](auto J) { b[J.value] = lds_read_b128<J.value * 2048>(sb + b_off[sub]); });
-        static_for<0, C::TM>([&](auto I) { a[I.value] = lds_read_b128<I.value * 2048>(sb + a_off[sub]); });
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-        for (int q = 0; q < C::TM; ++q) asm volatile("" : "+v"(a[q]));
-#pragma unroll
-        for (int q = 0; q < C::TN; ++q) asm volatile("" : "+v"(b[q]));
-        static_for<0, C::TM>([&](auto I) {
-          constexpr int tm = I.value;
-          if (tm < live_m) {                                       // uniform
-#pragma unroll
-            for (int tn = 0; tn < C::TN; ++tn) mfma16_v(acc[tm][tn], b[tn], a[tm]);
-          }
-        });
-      }
-      stage = stage == C::STAGES - 1 ? 0 : stage + 1;
-    }
-    wait_vmcnt<0>();                                               // the redundant loads past the end
-    // the MFMAs are opaque to the compiler: keep the distance it would keep before their results are read
-    asm volatile("s_nop 15\n s_nop 15" ::: "memory");
-#pragma unroll
-    for (int tm = 0; tm < C::TM; ++tm)
-#pragma unroll
-      for (int tn = 0; tn < C::TN; ++tn) asm volatile("" : "+v"(acc[tm][tn]));
+    SkinnyAcc acc;
+    skinny_mainloop(p, ent, 0, KT, acc, a_off, b_off, tid, lds, lds_base);
     // epilogue: bias, GELU or row scale, fp16 through the row index; 8-byte stores
     const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
     const int colb = n0 + wave * 64 + 4 * (lane >> 4);             // column of block tn = colb + 16 tn
@@ -492,6 +515,90 @@ __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, in
     }
   }
   wait_vmcnt<0>();
+}
+
+// The skinny list as a launch of its own (plan.h): workgroup w of W takes K steps [w q, (w + 1) q) of the sequence
+// "tile 0's K steps, tile 1's, ..." and leaves one raw fp32 partial tile per list entry it touches, in fragment order
+// (block (tm, tn) of thread t at float4 index (4 tm + tn) * 256 + t), in its slots w * kSkTailSegs + 0, 1, ...
+__device__ __forceinline__ void skinny_tail_role(const GroupedArgs &p, int w, lds_char *lds, uint32_t lds_base) {
+  using C = SkinnyCfg;
+  if (!p.skinny) return;
+  const int T = p.skinny[0], q = p.skinny[3];
+  if (T <= 0 || q <= 0) return;
+  const int KT = p.K / C::BK;
+  const int total = T * KT;
+  const int s0 = w * q;
+  if (s0 >= total) return;
+  const int s1 = s0 + q < total ? s0 + q : total;
+  const int4v *list = reinterpret_cast<const int4v *>(p.skinny + 4);
+  const int tid = fresh_tid();
+  uint32_t a_off[2], b_off[2];
+  skinny_frag_offsets(tid, a_off, b_off);
+  int t = s0 / KT;
+  for (int seg = 0; seg < kSkTailSegs && t * KT < s1; ++seg, ++t) {
+    const int k0 = (s0 > t * KT ? s0 : t * KT) - t * KT;
+    const int k1 = (s1 < (t + 1) * KT ? s1 : (t + 1) * KT) - t * KT;
+    SkinnyAcc acc;
+    skinny_mainloop(p, list[t], k0, k1 - k0, acc, a_off, b_off, tid, lds, lds_base);
+    float4v *out = reinterpret_cast<float4v *>(p.sk_partial) +
+                   static_cast<size_t>(w * kSkTailSegs + seg) * (C::TM * C::TN * 256) + tid;
+#pragma unroll
+    for (int tm = 0; tm < C::TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < C::TN; ++tn) out[(tm * C::TN + tn) * 256] = acc[tm][tn];
+  }
+  wait_vmcnt<0>();
+}
+
+// Row block tm (16 rows) of skinny tile t: the sum of its partial tiles in K order, then the epilogue.
+// One workgroup of 256 threads; thread t holds what thread t of the producing workgroup held.
+template <int kEpi>
+__device__ __forceinline__ void skinny_reduce_block(const GroupedArgs &p, int t, int tm) {
+  using C = SkinnyCfg;
+  const int q = p.skinny[3];
+  const int KT = p.K / C::BK;
+  const int4v ent = reinterpret_cast<const int4v *>(p.skinny + 4)[t];
+  const int e = ent[0], row0 = ent[1], rows = ent[2], n0 = ent[3] * C::BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = tm * 16 + (lane & 15);
+  if (tm * 16 >= rows) return;
+  const int w_lo = (t * KT) / q, w_hi = ((t + 1) * KT - 1) / q;
+  float4v acc[C::TN];
+#pragma unroll
+  for (int tn = 0; tn < C::TN; ++tn) acc[tn] = float4v{0, 0, 0, 0};
+  for (int w = w_lo; w <= w_hi; ++w) {
+    const int seg = t - (w * q) / KT;
+    const float4v *src = reinterpret_cast<const float4v *>(p.sk_partial) +
+                         static_cast<size_t>(w * kSkTailSegs + seg) * (C::TM * C::TN * 256) + (tm * C::TN) * 256 + tid;
+#pragma unroll
+    for (int tn = 0; tn < C::TN; ++tn) acc[tn] += src[tn * 256];
+  }
+  if (r >= rows) return;
+  const int j = row0 + r;
+  const size_t crow = p.c_rows ? static_cast<size_t>(p.c_rows[j]) : static_cast<size_t>(j);
+  const float sc = p.row_scale ? static_cast<float>(p.row_scale[j]) : 1.0f;
+  const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
+#pragma unroll
+  for (int tn = 0; tn < C::TN; ++tn) {
+    const int col = n0 + wave * 64 + 16 * tn + 4 * (lane >> 4);
+    if (col >= p.N) continue;
+    half4 bv = {0, 0, 0, 0};
+    if (p.bias) bv = *reinterpret_cast<const half4 *>(bias_e + col);
+    half4 o, pre;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float x = acc[tn][c] + static_cast<float>(bv[c]);
+      if (kEpi == kEpiPlain) {
+        x *= sc;
+      } else {
+        pre[c] = static_cast<half_t>(x);
+        x = gelu_erf(x);
+      }
+      o[c] = static_cast<half_t>(x);
+    }
+    *reinterpret_cast<half4 *>(p.C + crow * p.N + col) = o;
+    if (kEpi == kEpiGeluKeep) *reinterpret_cast<half4 *>(p.C2 + static_cast<size_t>(j) * p.N + col) = pre;
+  }
 }
 
 // ---- persistent form -------------------------------------------------------------
@@ -680,10 +787,15 @@ __device__ __forceinline__ void part_range(int k_tiles, int part, int S, int &fi
 }
 
 // One part of one tail tile per workgroup: the main loop over its K range, raw accumulators out.
+// Workgroups from `split_wgs` on run the skinny list as a launch of its own (skinny_tail_role).
 template <class Cfg, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
-grouped_gemm_tail_kernel(GroupedArgs p) {
+grouped_gemm_tail_kernel(GroupedArgs p, int split_wgs) {
   using R = Ring16Mainloop<Cfg, kKN>;
+  if (static_cast<int>(blockIdx.x) >= split_wgs) {
+    if constexpr (!kKN) skinny_tail_role(p, static_cast<int>(blockIdx.x) - split_wgs, R::lds(), R::lds_addr());
+    return;
+  }
   const int bmul = kKN ? p.N : 1;                      // elements between K rows of a [K][N] B
   const int tiles = p.tail[0], S = p.tail[1];
   if (static_cast<int>(blockIdx.x) >= tiles * S) return;
@@ -720,13 +832,23 @@ grouped_gemm_tail_kernel(GroupedArgs p) {
 }
 
 // out tile = sum of its S partial tiles (in part order) + bias, then the epilogue kEpi of the
-// grouped GEMM.  grid (kTailMaxTiles, BM / 16): block (t, q) does tile rows 16q .. 16q+15 of
-// tile slot t, a thread four rows of four columns.  It runs at the speed the partial tiles
+// grouped GEMM.  grid (kTailMaxTiles [+ kSkReduceX], BM / 16): block (t, q) with t < kTailMaxTiles
+// does tile rows 16q .. 16q+15 of tile slot t, a thread four rows of four columns; the blocks past
+// them reduce the skinny tiles that ran as a launch of their own.  It runs at the speed the partial tiles
 // stream back in (config 3, FFN2: 63 MB in 13 us).
 template <class Cfg, int kEpi>
 __global__ void __launch_bounds__(256)
 splitk_reduce_kernel(GroupedArgs p) {
   using R = Ring16Mainloop<Cfg>;
+  if (blockIdx.x >= kTailMaxTiles) {
+    // the skinny tiles of a launch of their own: (tile, row block) pairs over the blocks past the split's
+    if (!p.skinny || p.skinny[3] <= 0) return;
+    const int pairs = p.skinny[0] * SkinnyCfg::TM;
+    const int nblk = (gridDim.x - kTailMaxTiles) * gridDim.y;
+    for (int i = (blockIdx.x - kTailMaxTiles) * gridDim.y + blockIdx.y; i < pairs; i += nblk)
+      skinny_reduce_block<kEpi>(p, i / SkinnyCfg::TM, i % SkinnyCfg::TM);
+    return;
+  }
   const int tiles = p.tail[0], S = p.tail[1];
   const int t = blockIdx.x;
   if (t >= tiles) return;
@@ -792,12 +914,14 @@ int g_split_tail_min_kt = kSplitTailMinKT;
 int g_split_max_parts = 8;
 int g_fused_combine = 0;     // 1: top-2 layers add the gate-weighted expert outputs in the second GEMM's epilogue
 int g_skinny_pct = 70;       // a K step of a skinny tile in percent of a 256-row tile's (plan model); 0: no skinny tiles
+int g_skinny_tail = 1;       // 0: skinny tiles never run as a launch of their own
 
 // The tuning knobs a grouped GEMM's plan and launches depend on, read once per call: the plan
 // and the kernels that consume it must agree even if another thread calls ccf_set_option
 // between the routing stage (which builds the plans of the layer's forward call) and the GEMMs.
 GemmOptions current_options() {
-  return GemmOptions{g_variant, g_split_tail, g_split_tail_min_kt, g_split_max_parts, g_skinny_pct, g_fused_combine};
+  return GemmOptions{g_variant, g_split_tail, g_split_tail_min_kt, g_split_max_parts, g_skinny_pct, g_fused_combine,
+                     g_skinny_tail};
 }
 
 // The kernels of one family of epilogues: `first` and `second` are two epilogue forms, each as
@@ -811,6 +935,7 @@ struct Launch {
   void (*persistent_gelu)(GroupedArgs, int);
 };
 constexpr int kPersistentMinKT = 4;
+constexpr int kSkReduceX = 32;       // x 16 blocks of the reduction launch for the skinny tiles
 
 const Launch kVariants[] = {// forward: "plain" = bias and row scale, "gelu" = bias and GELU
                             {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiPlain>,
@@ -881,7 +1006,7 @@ struct GemmSetup {
   int grid;
   long long wgs;
   int32_t *tail, *plan;
-  float *partial;
+  float *partial, *sk_partial;
   PlanReq req;
 };
 
@@ -890,6 +1015,7 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
   GemmSetup g;
   char *ws = static_cast<char *>(workspace);
   g.partial = reinterpret_cast<float *>(ws + kTailHead);
+  g.sk_partial = reinterpret_cast<float *>(ws + kTailHead + kSplitPartialBytes);
   if (region == 0) {
     g.tail = reinterpret_cast<int32_t *>(ws);                                       // header and entries
     g.plan = reinterpret_cast<int32_t *>(ws + kTailBytes);
@@ -916,7 +1042,7 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
   g.skinny_list = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.plan) + plan_core_bytes(max_rows, E, N > K ? N : K));
   g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, opt.split_max_parts, g.plan,
                   g.split ? g.tail : nullptr, g.skinny ? g.skinny_list : nullptr, g.grid,
-                  gelu ? kEpiCostGelu : kEpiCostPlain, opt.skinny_pct};
+                  gelu ? kEpiCostGelu : kEpiCostPlain, opt.skinny_pct, g.split && g.skinny && opt.skinny_tail};
   return g;
 }
 
@@ -976,6 +1102,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.seg_rows = 0;
   p.tail = tail;
   p.partial = partial;
+  p.sk_partial = gs.sk_partial;
   p.skinny = gs.skinny ? gs.skinny_list : nullptr;
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;                // wgs is a multiple of 8
@@ -983,10 +1110,13 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
                        dim3(v.threads), 0, stream, p, static_cast<int>(wgs / 8));
     if (split) {
       if (int rc = check_launch(what)) return rc;
-      if (b_kn) hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, true>), dim3(grid), dim3(Cfg5::THREADS), 0, stream, p);
-      else hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, false>), dim3(grid), dim3(Cfg5::THREADS), 0, stream, p);
+      // the skinny list may run as a launch of its own: `grid` more workgroups for it, more blocks in the reduction
+      const bool sk = gs.req.sk_tail_ok;
+      if (b_kn) hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, true>), dim3(grid), dim3(Cfg5::THREADS), 0, stream, p, grid);
+      else hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, false>), dim3(sk ? 2 * grid : grid), dim3(Cfg5::THREADS), 0,
+                              stream, p, grid);
       if (int rc = check_launch("grouped_gemm_tail_kernel")) return rc;
-      const dim3 rgrid(kTailMaxTiles, Cfg5::BM / 16);
+      const dim3 rgrid(kTailMaxTiles + (sk ? kSkReduceX : 0), Cfg5::BM / 16);
       if (epi == kEpiPlain) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiPlain>), rgrid, dim3(256), 0, stream, p);
       else if (epi == kEpiGelu) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGelu>), rgrid, dim3(256), 0, stream, p);
       else hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGeluKeep>), rgrid, dim3(256), 0, stream, p);
@@ -1014,7 +1144,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream,
-                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0}, row_off, E);
+                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0, 0}, row_off, E);
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
   p.A = A;
@@ -1035,6 +1165,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.seg_rows = M;
   p.tail = nullptr;
   p.partial = nullptr;
+  p.sk_partial = nullptr;
   p.skinny = nullptr;
   const int grid = persistent_grid();
   if (grid >= 8) {
@@ -1166,10 +1297,15 @@ extern "C" int ccf_set_option(const char *name, int value) {
     return CCF_OK;
   }
   if (!strcmp(name, "skinny")) {             // 0: off; 1: default; n > 1: cost of a skinny K step in percent (plan model);
-                                             // -n: always, with n workgroups per XCD
-    CCF_REQUIRE(value >= -kSkinnyMaxWgs && value <= 400, CCF_ERR_ARG, "set_option: skinny %d outside %d..400", value,
-                -kSkinnyMaxWgs);
+                                             // -n: always, with n workgroups per XCD; -(kSkinnyMaxWgs + 1): always, as a
+                                             // launch of their own
+    CCF_REQUIRE(value >= -kSkinnyMaxWgs - 1 && value <= 400, CCF_ERR_ARG, "set_option: skinny %d outside %d..400", value,
+                -kSkinnyMaxWgs - 1);
     g_skinny_pct = value == 1 ? 70 : value;
+    return CCF_OK;
+  }
+  if (!strcmp(name, "skinny_tail")) {
+    g_skinny_tail = value != 0;
     return CCF_OK;
   }
   if (!strcmp(name, "dgrad_transpose")) {
@@ -1278,6 +1414,28 @@ extern "C" int ccf_ffn2_forward(const void *h, const int32_t *src_row, const int
                                 ccf_stream_t stream) {
   return ccf::ffn2_forward(h, src_row, dst_row, offsets, max_rows, num_expert, d_model, d_ffn, w2, b2,
                            row_scale, y, workspace, workspace_bytes, ccf::as_stream(stream), nullptr);
+}
+
+extern "C" int ccf_ffn_plan_info(const void *workspace, int max_rows, int num_expert, int d_model, int d_ffn,
+                                 int which, int32_t *info, ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(workspace && info, CCF_ERR_ARG, "ffn_plan_info: null pointer");
+  CCF_REQUIRE(which == 1 || which == 2, CCF_ERR_ARG, "ffn_plan_info: which=%d is neither 1 (first GEMM) nor 2", which);
+  CCF_REQUIRE(max_rows > 0 && num_expert > 0 && num_expert <= 1024 && d_model > 0 && d_ffn > 0, CCF_ERR_ARG,
+              "ffn_plan_info: bad size");
+  const int N = which == 1 ? d_ffn : d_model, K = which == 1 ? d_model : d_ffn;
+  const GemmSetup gs = setup_gemm(max_rows, num_expert, N, K, which == 1 ? kEpiGelu : kEpiPlain, false,
+                                  const_cast<void *>(workspace), which == 1 ? 0 : 1, current_options());
+  for (int i = 0; i < 8; ++i) info[i] = 0;
+  hipStream_t st = as_stream(stream);
+  hipError_t e = hipSuccess;
+  if (gs.split) e = hipMemcpyAsync(info, gs.tail, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, st);
+  if (gs.skinny && e == hipSuccess) e = hipMemcpyAsync(info + 2, gs.skinny_list, 4 * sizeof(int32_t), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return fail(CCF_ERR_HIP, "ffn_plan_info: %s", hipGetErrorString(e));
+  info[6] = gs.grid;
+  info[7] = static_cast<int32_t>(gs.wgs < (1ll << 31) ? gs.wgs : -1);
+  return CCF_OK;
 }
 
 extern "C" size_t ccf_ffn_backward_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn) {

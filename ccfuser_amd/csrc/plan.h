@@ -31,7 +31,14 @@ constexpr int kOrderGroupM = 8;
 constexpr int kTailMaxParts = 256;
 constexpr int kTailMaxTiles = kTailMaxParts / 2;     // tile slots: every tile has at least two parts
 constexpr size_t kTailHead = 256 + 16 * kTailMaxParts;
-constexpr size_t kTailBytes = kTailHead + static_cast<size_t>(kTailMaxParts) * 256 * 256 * 4;
+constexpr size_t kSplitPartialBytes = static_cast<size_t>(kTailMaxParts) * 256 * 256 * 4;
+// Behind those partial tiles, the partial tiles of the skinny tiles when they run as a launch of
+// their own (below): kSkTailSegs tiles of 64 x 256 fp32 per workgroup of that launch.
+constexpr int kSkTailMaxWgs = 256;
+constexpr int kSkTailSegs = 4;                       // most skinny tiles the K steps of one workgroup may touch
+constexpr size_t kSkTailTileBytes = 64 * 256 * 4;
+constexpr size_t kSkTailBytes = static_cast<size_t>(kSkTailMaxWgs) * kSkTailSegs * kSkTailTileBytes;
+constexpr size_t kTailBytes = kTailHead + kSplitPartialBytes + kSkTailBytes;
 
 // ---- skinny tiles --------------------------------------------------------------
 // An expert's rows rarely fill its last 256-row M tile, and a tile with a few dozen real rows
@@ -44,9 +51,20 @@ constexpr size_t kTailBytes = kTailHead + static_cast<size_t>(kTailMaxParts) * 2
 // run beside the compute-bound 256-row tiles on bandwidth those leave idle.  Whether that pays
 // depends on the tile counts (a CU taken from the 256-row tiles costs them 1/32 of their
 // rate; whole rounds of tiles matter more than tiles), so build_plan prices both ways with a
-// small model and picks: ns = workgroups per XCD given to skinny tiles, 0 = none (every row
-// stays in 256-row tiles).  Layout of the list (int32):
-//   [0] tiles T   [1] ns   [2] tiles per XCD (XCD x owns entries [x * [2], (x + 1) * [2]))   [3] unused
+// small model and picks: ns = workgroups per XCD given to skinny tiles, 0 = none.
+//
+// The third way: the skinny tiles as a launch of their own behind the persistent kernel, which
+// then keeps every CU for 256-row tiles (a GEMM whose 256-row tiles fill whole rounds exactly
+// loses a round to any CU it gives away).  Alone on the chip the skinny tiles are bound by
+// streaming their experts' weights from HBM once more, so the list is cut stream-K fashion: its
+// T tiles x k_tiles K steps are one sequence that the W workgroups of the launch cut into equal
+// ranges of q = ceil(T k_tiles / W) steps; a workgroup leaves one fp32 partial tile per list
+// entry its range touches, and the reduction that follows adds a tile's partial tiles in K
+// order and applies the epilogue (no atomics: two runs give the same bits).
+//
+// Layout of the list (int32):
+//   [0] tiles T   [1] ns   [2] tiles per XCD (XCD x owns entries [x * [2], (x + 1) * [2]))
+//   [3] q > 0: the tiles run as a launch of their own, q K steps per workgroup; 0 otherwise
 //   [4 + 4 i ...] entry i < T: {expert, first sorted row, rows (1..kSkinnyRows), N tile}
 constexpr int kSkinnyRows = 64;
 constexpr int kSkinnyMaxWgs = 4;                     // per XCD
@@ -113,8 +131,17 @@ struct PlanReq {
   int cus;          // workgroups of the persistent launch (a multiple of 8)
   int epi_cost;     // the epilogue of a 256-row tile, in K steps
   int skinny_pct;   // a K step of a skinny tile in percent of a K step of a 256-row tile; 0 = never use skinny
-                    // tiles; -n = always, with n workgroups per XCD
+                    // tiles; -n (n <= kSkinnyMaxWgs) = always, with n workgroups per XCD; -(kSkinnyMaxWgs + 1) =
+                    // always as a launch of their own (needs `tail`)
+  int sk_tail_ok;   // the skinny tiles may run as a launch of their own (the caller launches the kernels for it)
 };
+
+// A K step of a skinny tile, in percent of a 256-row tile's, when the whole chip runs skinny tiles
+// and HBM bandwidth bounds them; and the fixed cost of that launch and its reduction, in K steps.
+constexpr int kSkTailStepPct = 90, kSkTailFixed = 16;
+
+// Most tiles a range of q consecutive K steps can touch when a tile has k_tiles steps.
+__host__ __device__ inline int sk_tail_segments(int q, int k_tiles) { return (q - 1 + k_tiles - 1) / k_tiles + 1; }
 
 // Built by `nparts` workgroups of any size that is a multiple of 64 (all threads of each call
 // this with the workgroup's `part`).  Every workgroup repeats the small scans and takes a share
@@ -139,11 +166,12 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     s_off[e] = v < max_rows ? v : max_rows;          // never plan past the caller's bound
   }
   __syncthreads();
-  __shared__ int s_ns;             // workgroups per XCD given to skinny tiles (0: every row in 256-row tiles)
+  __shared__ int s_ns;             // workgroups per XCD given to skinny tiles (0: none)
+  __shared__ int s_tail_q;         // > 0: skinny tiles as a launch of their own, K steps per workgroup
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
     // Skinny tiles or not: tile counts both ways, then the cheaper plan by the model above.
-    int ns_wgs = 0;
+    int ns_wgs = 0, tail_q = 0;
     if (skinny && rq.skinny_pct != 0 && rq.cus >= 64) {
       int nl0 = 0, nl1 = 0, nk1 = 0;                // 256-row tiles without / with skinny tiles, skinny M tiles
       for (int e = lane; e < E; e += 64) {
@@ -161,8 +189,19 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
         nl1 += __shfl_xor(nl1, off, 64);
         nk1 += __shfl_xor(nk1, off, 64);
       }
-      if (nk1 > 0 && rq.skinny_pct < 0) {
-        ns_wgs = -rq.skinny_pct < kSkinnyMaxWgs ? -rq.skinny_pct : kSkinnyMaxWgs;   // forced (tests, measurements)
+      // the launch of their own: possible when the caller launches the split kernels and a
+      // workgroup's range stays within kSkTailSegs tiles
+      const int tail_wgs = rq.cus < kSkTailMaxWgs ? rq.cus : kSkTailMaxWgs;
+      int q_c = 0;
+      if (tail && rq.sk_tail_ok && nk1 > 0 && k_tiles > 0) {
+        const long long steps = static_cast<long long>(nk1) * n_tiles_n * k_tiles;
+        const long long q = (steps + tail_wgs - 1) / tail_wgs;
+        if (q < (1 << 20) && sk_tail_segments(static_cast<int>(q), k_tiles) <= kSkTailSegs) q_c = static_cast<int>(q);
+      }
+      if (nk1 > 0 && rq.skinny_pct < -kSkinnyMaxWgs) {
+        tail_q = q_c;                                  // forced (tests, measurements); 0 = not possible: no skinny tiles
+      } else if (nk1 > 0 && rq.skinny_pct < 0) {
+        ns_wgs = -rq.skinny_pct;                       // forced
       } else if (nk1 > 0) {
         const int cus_x = rq.cus / 8;
         const bool may_split = spx > 0;
@@ -175,9 +214,14 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
           const int c = main_c > sk_c ? main_c : sk_c;
           if (c < best) { best = c; ns_wgs = n; }
         }
+        if (q_c > 0) {
+          const int c = rounds_cost(F1, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts) +
+                        (q_c * kSkTailStepPct + 99) / 100 + kSkTailFixed;
+          if (c < best) { best = c; ns_wgs = 0; tail_q = q_c; }
+        }
       }
     }
-    if (lane == 0) s_ns = ns_wgs;
+    if (lane == 0) { s_ns = ns_wgs; s_tail_q = tail_q; }
     int carry_l = 0, carry_s = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
@@ -185,7 +229,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       cnt = cnt > 0 ? cnt : 0;
       const int nt = (cnt + BM - 1) / BM;
       int ns, nl;
-      if (ns_wgs) {
+      if (ns_wgs || tail_q) {
         const int r = cnt % BM;                                   // ns counts skinny M tiles here
         ns = (r > 0 && r <= kSkinnyRows) ? 1 : 0;
         nl = nt - ns;
@@ -218,7 +262,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   // short tile x*per_short + (j - nl).  The used slots of an XCD are a prefix:
   // the first idle entry ends its list.
   const int ns_wgs = s_ns;                                       // published by the barrier above
-  const bool use_skinny = ns_wgs > 0;
+  const bool use_skinny = ns_wgs > 0 || s_tail_q > 0;
   if (spx > 0) spx -= ns_wgs;
   const int total_long = s_long[E] * n_tiles_n;
   const int total_short = use_skinny ? 0 : s_short[E] * n_tiles_n;   // skinny tiles are not in this plan
@@ -227,7 +271,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     skinny[0] = T;
     skinny[1] = ns_wgs;
     skinny[2] = (T + 7) / 8;
-    skinny[3] = 0;
+    skinny[3] = s_tail_q;
   }
   const int per_long = (total_long + 7) / 8;
   const int per_short = (total_short + 7) / 8;
@@ -337,7 +381,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
 // ffn.hip
 // Snapshot of the tuning knobs (ccf_set_option) that a grouped GEMM's plan and launches depend on.
 struct GemmOptions {
-  int variant, split_tail, split_tail_min_kt, split_max_parts, skinny_pct, fused_combine;
+  int variant, split_tail, split_tail_min_kt, split_max_parts, skinny_pct, fused_combine, skinny_tail;
 };
 GemmOptions forward_options();
 bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *workspace, const GemmOptions &opt,

@@ -232,6 +232,23 @@ def combine(y_flat: torch.Tensor, score: torch.Tensor, top_k: int,
 
 
 # ------------------------------------------------------------ expert FFN
+def ffn_workspace(max_rows: int, E: int, d: int, f: int, like: torch.Tensor) -> torch.Tensor:
+    """A workspace for ``ffn1`` / ``ffn2`` (one call at a time per workspace)."""
+    return _workspace(_lib.lib().ccf_ffn_workspace_bytes(int(max_rows), E, d, f), like)
+
+
+def ffn_plan_info(workspace: torch.Tensor, max_rows: int, E: int, d: int, f: int, which: int) -> Dict[str, int]:
+    """What the tile plan left in ``workspace`` by the last ``ffn1`` (which=1) or ``ffn2`` (which=2)
+    call decided (diagnostic; synchronises)."""
+    import ctypes as C
+    info = (C.c_int32 * 8)()
+    with torch.cuda.device(workspace.device):
+        _lib.call("ccf_ffn_plan_info", _ptr(workspace), int(max_rows), E, d, f, int(which), info, _stream(workspace))
+    names = ("split_tiles", "split_parts", "skinny_tiles", "skinny_wgs_per_xcd", "skinny_per_xcd", "skinny_tail_steps",
+             "persistent_wgs", "worst_case_tiles")
+    return dict(zip(names, list(info)))
+
+
 def _check_expert(w: torch.Tensor, b: torch.Tensor, name: str) -> None:
     _check(w, f"{name} weight", dtype=torch.float16, ndim=3)
     _check(b, f"{name} bias", dtype=torch.float16, ndim=2)
@@ -241,7 +258,8 @@ def _check_expert(w: torch.Tensor, b: torch.Tensor, name: str) -> None:
 
 def ffn1(x: torch.Tensor, src_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
          w1: torch.Tensor, b1: torch.Tensor, gelu: bool = True,
-         out: Optional[torch.Tensor] = None, dst_row: Optional[torch.Tensor] = None) -> torch.Tensor:
+         out: Optional[torch.Tensor] = None, dst_row: Optional[torch.Tensor] = None,
+         workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """h [max_rows, f] (or ``out``); rows nothing maps to are left as they were."""
     if x.dtype != torch.float16:
         raise TypeError("moe input data type must be float 16")
@@ -266,7 +284,7 @@ def ffn1(x: torch.Tensor, src_row: Optional[torch.Tensor], offsets: torch.Tensor
     if h.shape[1] != f or (dst_row is None and h.shape[0] < max_rows):
         raise ValueError("ffn1: output buffer too small")
     with torch.cuda.device(x.device):
-        ws = _workspace(_lib.lib().ccf_ffn_workspace_bytes(max_rows, E, d, f), x)
+        ws = workspace if workspace is not None else ffn_workspace(max_rows, E, d, f, x)
         _lib.call("ccf_ffn1_forward", _ptr(x), _ptr(src_row), _ptr(dst_row), _ptr(offsets), int(max_rows), E, d, f,
                   _ptr(w1), _ptr(b1), int(bool(gelu)), _ptr(h), _ptr(ws), ws.numel(), _stream(x))
     return h
@@ -300,7 +318,7 @@ def ffn1_keep(x: torch.Tensor, src_row: Optional[torch.Tensor], offsets: torch.T
 def ffn2(h: torch.Tensor, dst_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
          w2: torch.Tensor, b2: torch.Tensor, y: torch.Tensor,
          row_scale: Optional[torch.Tensor] = None,
-         src_row: Optional[torch.Tensor] = None) -> torch.Tensor:
+         src_row: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Writes ``y[dst_row[j]]`` for the routed rows and returns ``y``."""
     _check(h, "h", dtype=torch.float16, ndim=2)
     _check_expert(w2, b2, "ffn2")
@@ -324,7 +342,7 @@ def ffn2(h: torch.Tensor, dst_row: Optional[torch.Tensor], offsets: torch.Tensor
     if row_scale is not None:
         _check(row_scale, "row_scale", dtype=torch.float16, ndim=1)
     with torch.cuda.device(h.device):
-        ws = _workspace(_lib.lib().ccf_ffn_workspace_bytes(max_rows, E, d, f), h)
+        ws = workspace if workspace is not None else ffn_workspace(max_rows, E, d, f, h)
         _lib.call("ccf_ffn2_forward", _ptr(h), _ptr(src_row), _ptr(dst_row), _ptr(offsets), int(max_rows), E, d, f,
                   _ptr(w2), _ptr(b2), _ptr(row_scale), _ptr(y), _ptr(ws), ws.numel(), _stream(h))
     return y

@@ -64,7 +64,9 @@ const char *ccf_last_error(void);
  *                     may run as 64-row tiles in a few workgroups set aside for them, when the tile plan's
  *                     cost model says that beats a padded 256-row tile; n > 1 sets the model's cost of
  *                     such a tile's K step in percent of a 256-row tile's (default 70); -n (1..4) forces
- *                     them with n workgroups per XCD
+ *                     them with n workgroups per XCD; -5 forces them as a launch of their own behind the
+ *                     persistent kernel, cut along K over all workgroups (the model's third choice)
+ *   "skinny_tail"     0/1 (default 1): the plan may choose that third way
  *   "fused_combine"   0/1 (default 0): ccf_moe_forward with top_k = 2 adds the gate-weighted expert outputs
  *                     into the output in the second GEMM's epilogue (packed fp16 atomic adds onto zeros)
  *                     instead of running the combine pass; measured slower, kept for comparison
@@ -232,6 +234,19 @@ int ccf_combine(const void *y_flat, const void *score, const int32_t *inv_pos,
 
 /* Bytes of workspace the FFN entry points need (the device-built tile plan). */
 size_t ccf_ffn_workspace_bytes(int max_rows, int num_expert, int d_model, int d_ffn);
+
+/*
+ * Diagnostic (no counterpart in the reference): what the tile plan that the last call left in
+ * `workspace` decided, for which = 1 (the first GEMM: ccf_ffn1_forward, ccf_ffn1_forward_keep) or 2
+ * (ccf_ffn2_forward); for ccf_moe_forward's plans pass the FFN part of its workspace.  Copies a few
+ * integers to the host and synchronises the stream.  info (host, 8 ints):
+ *   [0] tiles of the split last round, [1] parts each is cut into (0 = not split)
+ *   [2] skinny tiles, [3] workgroups per XCD that run them beside the 256-row tiles,
+ *   [4] skinny tiles per XCD, [5] K steps per workgroup when they run as a launch of their own (0 = not)
+ *   [6] workgroups of the persistent launch (0 = one workgroup per tile), [7] worst-case tile count
+ */
+int ccf_ffn_plan_info(const void *workspace, int max_rows, int num_expert, int d_model, int d_ffn,
+                      int which, int32_t *info, ccf_stream_t stream);
 
 /*
  * FFN1 as a grouped GEMM with the scatter fused into the A-tile loads:

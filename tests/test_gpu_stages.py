@@ -519,41 +519,71 @@ def test_split_k_tail_all_epilogues():
     assert not torch.equal(results[4][3], results[0][3]) and not torch.equal(results[4][0], results[0][0])
 
 
-@pytest.mark.parametrize("R,d,f,E,skew,seed,mode", [
-    (8192, 4096, 4096, 6, False, 31, 1),       # remainders of ~80 rows: above 64, stay in 256-row tiles
-    (8192 + 6 * 200, 4096, 4096, 6, False, 35, 1),   # remainders of ~25 rows, long K: the plan's own choice
-    (3000, 256, 512, 5, False, 32, -2),        # short K
-    (2100, 1024, 2048, 40, True, 33, -1),      # most experts are nothing but a skinny tile, some are empty
-    (1150, 512, 768, 3, False, 34, -3),        # remainders of 127, 130 and 125 rows: none is skinny, nothing to do
-    (2000, 512, 768, 7, False, 36, -4),        # remainders around 30 rows, N no multiple of 256
+# Forced cases are sized so that both GEMMs have at least as many worst-case tiles as the chip has
+# CUs ((ceil(R / 256) + E) * ceil(N / 256) >= 256): only then does the persistent launch set
+# workgroups aside for skinny tiles.  `expect`: which GEMMs must report skinny tiles actually run.
+@pytest.mark.parametrize("R,d,f,E,skew,seed,mode,expect", [
+    (8192, 4096, 4096, 6, False, 31, 1, ""),          # remainders of ~80 rows: above 64, stay in 256-row tiles
+    (8192 + 6 * 200, 4096, 4096, 6, False, 35, 1, ""),   # remainders of ~25 rows, long K: the plan's own choice
+    (0, 256, 1024, 60, False, 32, -2, "1"),           # first GEMM with K = 256: four K tiles, the shortest the loop takes
+    (2100, 1024, 2048, 70, True, 33, -1, "12"),       # most experts are nothing but a skinny tile, some are empty
+    (1150, 512, 768, 3, False, 34, -3, ""),           # remainders of 127, 130 and 125 rows: none is skinny, nothing to do
+    (15360, 1088, 832, 60, False, 36, -4, "12"),      # N no multiple of 256 in either GEMM (832, 1088)
+    (8192, 4096, 4096, 6, False, 37, -5, "12"),       # as a launch of their own, cut along K: a workgroup's range inside one tile
+    (0, 1536, 4160, 40, False, 38, -5, "12"),         # experts of 17..64 rows only: ranges of four tiles, N = 4160
 ])
-def test_skinny_tiles(R, d, f, E, skew, seed, mode):
-    """Rows beyond an expert's full 256-row tiles (at most 64) run as 64-row tiles in workgroups
-    the plan sets aside (mode 1: when its cost model says so; -n: forced, n workgroups per XCD).
-    All three forward epilogues with that path on and off, each against fp32; both paths add
-    over K in the same order and must agree bit for bit."""
+def test_skinny_tiles(R, d, f, E, skew, seed, mode, expect):
+    """Rows beyond an expert's full 256-row tiles (at most 64) run as 64-row tiles: in workgroups
+    the plan sets aside beside the 256-row tiles (mode -n: forced, n workgroups per XCD) or as a
+    launch of their own cut along K (mode -5: forced); mode 1 leaves the choice to the plan's
+    cost model.  All three forward epilogues with that path on and off, each against fp32.
+    Beside the 256-row tiles the path adds over K in the same order as they do and must agree
+    bit for bit; cut along K it agrees within rounding.  The plan must report that skinny tiles
+    really ran where the case is built for them."""
     from ccfuser_amd import ops
+    counts = None
+    if expect and not skew:
+        # every expert: whole 256-row tiles (R / E rounded down to them) plus a remainder of 17..64 rows
+        counts = torch.tensor([(R // E) // 256 * 256 + 17 + (e * 11) % 48 for e in range(E)])
+        R = int(counts.sum())
     x, w1, b1, w2, b2, e_of_row = _ffn_case(R, d, f, E, seed, skew)
     g = torch.Generator().manual_seed(seed)
+    if counts is not None:
+        e_of_row = torch.repeat_interleave(torch.arange(E), counts)[torch.randperm(R, generator=g)]
     scale = (torch.rand(R, generator=g) + 0.5).half()
     r = ops.route(dev(e_of_row), E, 1)
     off, pos = r["offsets"].cpu().tolist(), r["pos"].cpu()
     rem = r["counts"].cpu() % 256
     _say(f"skinny mode={mode} R={R} d={d} f={f} E={E} remainders={rem.tolist()[:12]}")
-    res = {}
+    ws = ops.ffn_workspace(R, E, d, f, dev(x))
+    res, info = {}, {}
     for m in (mode, 0):
         ops.set_option("skinny", m)
-        ops.set_option("split_tail", 0)           # keep the 256-row path unsplit: the comparison is about the skinny path
+        # beside the 256-row tiles: keep those unsplit, the comparison is about the skinny path;
+        # a launch of their own needs the split kernels launched (every K tile count allowed)
+        ops.set_option("split_tail", 2 if mode == -5 else 0)
         try:
-            h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True)
+            h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True, workspace=ws)
+            info[m, 1] = ops.ffn_plan_info(ws, R, E, d, f, 1)
             act, pre = ops.ffn1_keep(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1))
             y = torch.zeros(R, d, dtype=torch.float16, device="cuda")
-            ops.ffn2(h, r["dst_row"], r["offsets"], R, dev(w2), dev(b2), y, row_scale=dev(scale))
+            ops.ffn2(h, r["dst_row"], r["offsets"], R, dev(w2), dev(b2), y, row_scale=dev(scale), workspace=ws)
+            info[m, 2] = ops.ffn_plan_info(ws, R, E, d, f, 2)
             torch.cuda.synchronize()
             res[m] = [t.cpu() for t in (h, act, pre, y)]
         finally:
             ops.set_option("skinny", 1)
             ops.set_option("split_tail", 1)
+    _say(f"  plan, first GEMM: {info[mode, 1]}")
+    _say(f"  plan, second GEMM: {info[mode, 2]}")
+    for which in (1, 2):
+        i = info[mode, which]
+        ran = i["skinny_tiles"] > 0 and (i["skinny_wgs_per_xcd"] > 0 or i["skinny_tail_steps"] > 0)
+        if str(which) in expect:
+            assert ran, (which, i)
+            assert (i["skinny_tail_steps"] > 0) == (mode == -5) and (i["skinny_wgs_per_xcd"] == -mode or mode == -5), i
+        if mode < 0:
+            assert info[0, which]["skinny_tiles"] == 0
     buf = x[pos].float()
     pre_ref = torch.zeros(R, f)
     for e in range(E):
@@ -574,7 +604,13 @@ def test_skinny_tiles(R, d, f, E, skew, seed, mode):
         assert O.max_abs_err(y, y_ref) <= MAX_ABS and O.mean_rel_err(y, y_ref) <= MEAN_REL, m
     same = [torch.equal(a, b) for a, b in zip(res[mode], res[0])]
     _say(f"  skinny on/off bitwise equal (h, act, pre, y): {same}")
-    assert all(same)
+    if mode == -5:
+        # another summation order: close, and not identical where skinny tiles ran
+        for a, b in zip(res[mode], res[0]):
+            assert O.max_abs_err(a, b.float()) <= MAX_ABS
+        assert not all(same)
+    else:
+        assert all(same)
 
 
 def test_mfma_probe_runs_and_counts_its_flop():
