@@ -22,6 +22,11 @@
 namespace ccf {
 namespace {
 
+// The main loop of a tile shape: eight wavefronts (two per SIMD, half the registers each) keep one
+// register buffer of token fragments, four wavefronts two.
+template <class Cfg, bool kKN>
+using RingFor = Ring16Mainloop<Cfg, kKN, Cfg::NW == 8>;
+
 // ---- tile plan ---------------------------------------------------------------
 // build_plan() (plan.h) in a launch of its own; the layer's forward call lets the routing
 // stage build both of its plans instead.
@@ -115,7 +120,7 @@ constexpr int kEpiPlain = 0, kEpiGelu = 1, kEpiGeluKeep = 2, kEpiGeluGrad = 3, k
 // skips MFMAs in both.
 template <class Cfg>
 __device__ __forceinline__ int tile_row_to_local(int r, int rows) {
-  return Ring16Mainloop<Cfg>::local_row(r, rows);
+  return RingFor<Cfg, false>::local_row(r, rows);
 }
 
 // Global source of every tile load of this lane for the tile of plan entry
@@ -151,7 +156,7 @@ __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v e
   }
   if constexpr (kKN) {
     // B is [E, K, N]: K row r of the tile, the columns LDS unit u of that row holds (N % BN == 0)
-    using R = Ring16Mainloop<Cfg, true>;
+    using R = RingFor<Cfg, true>;
     const int tid = threadIdx.x;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {                          // loads 0 and 1; load i >= 2 is 16 rows below load i - 2
@@ -218,7 +223,7 @@ __device__ __forceinline__ half8 pair_exchange(half4 x, half4 y) {
 // fp16, 8-byte stores through the row index.
 template <class Cfg, int kEpi, bool kPlainRows = false>     // kPlainRows: no row index, no row scale, no bias
 __device__ __forceinline__ void epilogue16(const GroupedArgs &p, int e, int row0, int rows, int n0) {
-  using R = Ring16Mainloop<Cfg>;
+  using R = RingFor<Cfg, false>;
   constexpr int TM = R::TM, TN = R::TN;
   const int tid = fresh_tid();
   const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
@@ -331,7 +336,7 @@ grouped_gemm_kernel(GroupedArgs p) {
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
   tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
-  Ring16Mainloop<Cfg, kKN>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, ent[2], p.N);
+  RingFor<Cfg, kKN>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, ent[2], p.N);
   epilogue16<Cfg, kEpi, kSeg>(p, e, ent[1], ent[2], ent[3] * Cfg::BN);
 }
 
@@ -622,14 +627,14 @@ template <class Cfg, int kEpi, bool kSeg = false, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   using ML = GemmMainloop<Cfg>;
-  using R = Ring16Mainloop<Cfg, kKN>;
+  using R = RingFor<Cfg, kKN>;
   const int bmul = kKN ? p.N : 1;                     // elements between K rows of a [K][N] B
   constexpr int TM = R::TM, TN = R::TN;
   const int4v *plan = reinterpret_cast<const int4v *>(p.plan);
   const int xcd = blockIdx.x & 7;
   int stride = gridDim.x >> 3;
   int slot_j = blockIdx.x >> 3;
-  if constexpr (!kSeg && !kKN && kEpi <= kEpiGeluKeep) {
+  if constexpr (!kSeg && !kKN && kEpi <= kEpiGeluKeep && Cfg::NW == 4) {
     // the last ns workgroups of each XCD do the skinny tiles (if the plan has any), the others the 256-row tiles
     if (p.skinny) {
       const int ns = __builtin_amdgcn_readfirstlane(p.skinny[1]);
@@ -657,7 +662,7 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
   int a_off[2], b_off[2];
   R::frag_offsets(a_off, b_off);
-  half8 fa[2][TM], fb[2][TN];
+  half8 fa[R::AB][TM], fb[2][TN];
   R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg>(p, ent[0]), a_off, b_off, wave, bmul);
   R::reserve();
   int phase = 0;
@@ -690,7 +695,10 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       }
     }
 
-    const int live_m = R::live_blocks(ent[2]);
+    // The eight-wavefront form runs the MFMAs of padded row blocks too (they repeat real rows and are not
+    // stored): with half the registers, the branch around each row block makes the compiler park values in
+    // accumulation registers, which this kernel owns.
+    const int live_m = Cfg::NW == 8 ? TM : R::live_blocks(ent[2]);
     R::acc_settle();
     if (live_m == TM) {
       R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m, bmul);
@@ -791,7 +799,7 @@ __device__ __forceinline__ void part_range(int k_tiles, int part, int S, int &fi
 template <class Cfg, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_tail_kernel(GroupedArgs p, int split_wgs) {
-  using R = Ring16Mainloop<Cfg, kKN>;
+  using R = RingFor<Cfg, kKN>;
   if (static_cast<int>(blockIdx.x) >= split_wgs) {
     if constexpr (!kKN) skinny_tail_role(p, static_cast<int>(blockIdx.x) - split_wgs, R::lds(), R::lds_addr());
     return;
@@ -839,7 +847,7 @@ grouped_gemm_tail_kernel(GroupedArgs p, int split_wgs) {
 template <class Cfg, int kEpi>
 __global__ void __launch_bounds__(256)
 splitk_reduce_kernel(GroupedArgs p) {
-  using R = Ring16Mainloop<Cfg>;
+  using R = RingFor<Cfg, false>;
   if (blockIdx.x >= kTailMaxTiles) {
     // the skinny tiles of a launch of their own: (tile, row block) pairs over the blocks past the split's
     if (!p.skinny || p.skinny[3] <= 0) return;
@@ -904,6 +912,13 @@ splitk_reduce_kernel(GroupedArgs p) {
 // wavefronts of 128x128.  ccf_set_option("gemm_variant", n): 0 = persistent workgroups (default),
 // 1 = one workgroup per tile for every K (otherwise only K below four K tiles runs that way).
 using Cfg5 = GemmCfg<256, 256, 64, 2, 2, 8>;
+// The same tile with eight wavefronts of 128x64, two per SIMD, half the registers each (gemm_variant 3; the
+// forward epilogues only).  Built for GEMMs with few K steps in front of a GELU epilogue; measured, it gives
+// the four-wavefront form's bits and is no faster: what two wavefronts per SIMD gain in the epilogue, the main
+// loop loses, because a K step then reads 192 KB of fragments from LDS instead of 128 KB next to the 64 KB the
+// tile loads write, and the LDS pipe is busy for as long as the MFMAs are.  It is not chosen by default.
+using Cfg8 = GemmCfg<256, 256, 64, 2, 4, 8>;
+constexpr int kWideMaxKT = 0;        // forward GEMMs with at most this many K tiles take the eight-wavefront form by default
 
 constexpr int kDefaultVariant = 0;
 int g_variant = kDefaultVariant;
@@ -953,8 +968,11 @@ const Launch kVariants[] = {// forward: "plain" = bias and row scale, "gelu" = b
                              grouped_gemm_persistent_kernel<Cfg5, kEpiGeluGrad>},
                             // the combine epilogue ("plain" slot)
                             {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiCombine>, nullptr,
-                             grouped_gemm_persistent_kernel<Cfg5, kEpiCombine>, nullptr}};
-constexpr int kFwdVariant = 0, kKnVariant = 1, kTrainVariant = 2, kCombineVariant = 3;
+                             grouped_gemm_persistent_kernel<Cfg5, kEpiCombine>, nullptr},
+                            // forward, eight wavefronts (persistent only)
+                            {Cfg8::BM, Cfg8::BN, Cfg8::THREADS, nullptr, nullptr, grouped_gemm_persistent_kernel<Cfg8, kEpiPlain>,
+                             grouped_gemm_persistent_kernel<Cfg8, kEpiGelu>}};
+constexpr int kFwdVariant = 0, kKnVariant = 1, kTrainVariant = 2, kCombineVariant = 3, kFwd8Variant = 4;
 
 // Compute units of the current device, rounded down to whole XCD rounds of 8.
 int persistent_grid() {
@@ -969,7 +987,7 @@ int persistent_grid() {
   }
   return cached;
 }
-constexpr int kNumVariants = 2;                      // what ccf_set_option accepts
+constexpr int kNumVariants = 4;                      // what ccf_set_option accepts
 constexpr int kMinBM = 256;
 
 int max_tiles_for(int max_rows, int E, int bm) { return (max_rows + bm - 1) / bm + E; }
@@ -1024,25 +1042,31 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
     g.plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.tail) + kTailHead);
   }
   const bool gelu = epi != kEpiPlain && epi != kEpiCombine;
-  g.v = &kVariants[b_kn ? kKnVariant : (epi == kEpiCombine ? kCombineVariant : (epi >= kEpiGeluKeep ? kTrainVariant : kFwdVariant))];
+  const int kt_all = K / 64;
+  const int cus = persistent_grid();
+  const bool persistent = opt.variant != 1 && kt_all >= kPersistentMinKT && cus >= 8;
+  // eight wavefronts: the two plain forward epilogues, short K (or forced)
+  const bool wide = persistent && !b_kn && epi <= kEpiGelu && (opt.variant == 3 || (opt.variant == 0 && kt_all <= kWideMaxKT));
+  g.v = &kVariants[b_kn ? kKnVariant : (epi == kEpiCombine ? kCombineVariant : (epi >= kEpiGeluKeep ? kTrainVariant :
+                                                                                   (wide ? kFwd8Variant : kFwdVariant)))];
   const Launch &v = *g.v;
   // which of the entry's two kernels: the K-N and training entries hold the GELU-gradient form in the second slot
   g.second = b_kn ? epi == kEpiGeluGrad : (epi == kEpiCombine ? false : (epi >= kEpiGeluKeep ? epi == kEpiGeluGrad : gelu));
   const int max_tiles = max_tiles_for(max_rows, E, v.bm);
   const int n_tiles_n = (N + v.bn - 1) / v.bn;
   g.wgs = launched_wgs(max_tiles, n_tiles_n);                   // worst-case tile count
-  g.grid = opt.variant == 0 && K / 64 >= kPersistentMinKT ? persistent_grid() : 0;
+  g.grid = persistent ? cus : 0;
   // the last, partly filled round is cut along K and spread over all workgroups (forward forms;
   // worth its two small launches only where a tile is long: K of 4096 and more)
   g.split = opt.split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && g.grid >= 8 && g.grid <= g.wgs &&
             g.grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= opt.split_tail_min_kt;
   // remainder rows as skinny tiles: forward epilogues of the persistent 256 x 256 kernel with the [N][K] weight
   g.skinny = opt.skinny_pct != 0 && !b_kn && epi <= kEpiGeluKeep && g.grid >= 64 && g.grid <= g.wgs &&
-             v.bm == Cfg5::BM && v.bn == Cfg5::BN && v.persistent_plain;
+             v.bm == Cfg5::BM && v.bn == Cfg5::BN && v.persistent_plain && (!wide || g.split);
   g.skinny_list = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.plan) + plan_core_bytes(max_rows, E, N > K ? N : K));
   g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, opt.split_max_parts, g.plan,
                   g.split ? g.tail : nullptr, g.skinny ? g.skinny_list : nullptr, g.grid,
-                  gelu ? kEpiCostGelu : kEpiCostPlain, opt.skinny_pct, g.split && g.skinny && opt.skinny_tail};
+                  gelu ? kEpiCostGelu : kEpiCostPlain, opt.skinny_pct, g.split && g.skinny && opt.skinny_tail, !wide};
   return g;
 }
 
@@ -1144,7 +1168,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream,
-                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0, 0}, row_off, E);
+                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0, 0, 0}, row_off, E);
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
   p.A = A;
@@ -1283,7 +1307,7 @@ extern "C" int ccf_set_option(const char *name, int value) {
   if (!strcmp(name, "gemm_variant")) {
     CCF_REQUIRE(value >= -1 && value < kNumVariants, CCF_ERR_ARG, "set_option: gemm_variant %d outside -1..%d",
                 value, kNumVariants - 1);
-    g_variant = value < 0 ? kDefaultVariant : value;     // -1: back to the default
+    g_variant = value < 0 ? kDefaultVariant : value;     // -1: back to the default (0: the library chooses by K)
     return CCF_OK;
   }
   if (!strcmp(name, "split_tail")) {         // 0 = off, 1 = default, n > 1: for K of n K tiles and more

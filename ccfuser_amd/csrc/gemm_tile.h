@@ -213,9 +213,18 @@ struct GemmMainloop {
 // XORed with f(row) = row%4 + 4*((row/8)%2): two cycles per read, the minimum
 // for 512 bytes.  The XOR sits in address bits 5..7, the column block tn in the
 // same bits, so a fragment's address is the lane's base address XOR 32*tn.
-template <class Cfg, bool B_KN = false>
+//
+// ROLL_A (the eight-wavefront form: two wavefronts per SIMD, 128 vector and 128 accumulation
+// registers each): the token fragments have ONE register buffer instead of two.  The MFMAs
+// of a substep run row block by row block, and as soon as a row block's last MFMA has issued,
+// its fragment registers take the NEXT substep's fragment of that row block.  The reads still
+// leave during the substep before their use, so the ring schedule above is unchanged; what
+// changes is that a row block's new fragment has one substep less one row block of lead
+// instead of a whole substep, which the second wavefront of the SIMD covers.
+template <class Cfg, bool B_KN = false, bool ROLL_A = false>
 struct Ring16Mainloop {
   using acc_t = float4v;
+  static constexpr int AB = ROLL_A ? 1 : 2;                      // register buffers of the token fragments
   static constexpr int KN_PITCH = Cfg::BN * 2;                   // bytes per K row of a [K][N] half tile
   // Source pointers a lane holds for its B tile loads.  [N][K]: one per load.  [K][N]: load i
   // fetches K row 8*i + r0 (r0 < 8 fixed per lane), whose chunk XOR depends on i%2 only, so
@@ -317,7 +326,11 @@ struct Ring16Mainloop {
   // MFMAs get no hazard padding from the compiler: callers keep the required
   // distance to any other instruction that touches an accumulator (settle()).
   static_assert(TM * TN * 4 <= 256, "accumulation registers");
-  static __device__ __forceinline__ void reserve() { asm volatile("" ::: "a255"); }
+  static __device__ __forceinline__ void reserve() {
+    static_assert(TM * TN * 4 == 256 || TM * TN * 4 == 128, "accumulation registers owned by the kernel");
+    if constexpr (TM * TN * 4 == 256) asm volatile("" ::: "a255");
+    else asm volatile("" ::: "a127");
+  }
   // acc(tm, tn) += w (16 weight rows) x t (16 token rows), K = 32
   template <int BLK>
   static __device__ __forceinline__ void mfma16(const half8 &w, const half8 &t) {
@@ -344,14 +357,20 @@ struct Ring16Mainloop {
   // reads of the NEXT substep's fragments (LDS addresses ra, rb) into the other
   // buffer and the tile loads into the slot at byte offset ws.
   template <int SUB, int NLOAD, bool FULL, bool KN2 = false, int NSRC>
-  static __device__ __forceinline__ void substep(half8 (&a)[2][TM], half8 (&b)[2][TN],
+  static __device__ __forceinline__ void substep(half8 (&a)[AB][TM], half8 (&b)[2][TN],
                                                  const half_t *const (&src)[NSRC], int k_elem, uint32_t ra,
                                                  uint32_t rb, int ws, int wave, int live_m, int bmul = 1) {
+    constexpr int AS = ROLL_A ? 0 : SUB, AN = ROLL_A ? 0 : SUB ^ 1;     // token fragment buffer in use / being filled
     // what goes out behind MFMA i
     auto behind = [&](auto II) {
       constexpr int i = II.value;
-      if constexpr (i % READ_EVERY == 0 && i / READ_EVERY < FRAGS)
-        read_frag<i / READ_EVERY>(a[SUB ^ 1], b[SUB ^ 1], ra, rb);
+      if constexpr (ROLL_A) {
+        // weight fragments early; a row block's token fragment when its last MFMA of this substep has issued
+        if constexpr (i % READ_EVERY == 0 && i / READ_EVERY < TN) read_frag<i / READ_EVERY>(a[AN], b[SUB ^ 1], ra, rb);
+        if constexpr (i % TN == TN - 1) read_frag<TN + i / TN>(a[AN], b[SUB ^ 1], ra, rb);
+      } else if constexpr (i % READ_EVERY == 0 && i / READ_EVERY < FRAGS) {
+        read_frag<i / READ_EVERY>(a[AN], b[SUB ^ 1], ra, rb);
+      }
       if constexpr (i % Cfg::DMA_EVERY == 1 && i / Cfg::DMA_EVERY < NLOAD) {
         constexpr int l = i / Cfg::DMA_EVERY;
         lds_dma16(load_src<KN2>(src, l, k_elem, bmul), lds() + ws + (l * Cfg::NW + wave) * 1024);
@@ -364,7 +383,7 @@ struct Ring16Mainloop {
       if (FULL || tm < live_m) {
         static_for<0, TN>([&](auto J) {
           constexpr int tn = J.value;
-          mfma16<tm * TN + tn>(b[SUB][tn], a[SUB][tm]);
+          mfma16<tm * TN + tn>(b[SUB][tn], a[AS][tm]);
           behind(std::integral_constant<int, tm * TN + tn>{});
         });
       } else {
@@ -376,7 +395,7 @@ struct Ring16Mainloop {
   // K tile kt in ring phase ph; k2 / kb2: element offset from the A / B sources of the K
   // tile that the loads of this step fetch (A into the fifth slot, B into the slot A(kt) leaves).
   template <bool FULL>
-  static __device__ __forceinline__ void step(half8 (&a)[2][TM], half8 (&b)[2][TN],
+  static __device__ __forceinline__ void step(half8 (&a)[AB][TM], half8 (&b)[2][TN],
                                               const half_t *const (&a_src)[Cfg::A_DMA],
                                               const half_t *const (&b_src)[B_SRCS], const int (&a_off)[2],
                                               const int (&b_off)[2], int k2, int kb2, int ph, int wave, int live_m, int bmul) {
@@ -390,7 +409,7 @@ struct Ring16Mainloop {
     // B(kt+1) and everything older have landed; A(kt+2) may stay in flight
     wait_vmcnt<Cfg::A_DMA>();
     block_barrier();
-    frags_ready(a[1], b[1]);
+    frags_ready(a[AB - 1], b[1]);
     __builtin_amdgcn_sched_barrier(0);
     // K half 1; fetch the fragments of K half 0 of tile kt+1; load B(kt+2) into A(kt)'s slot
     substep<1, Cfg::B_DMA, FULL, B_KN>(a, b, b_src, kb2, base + s.na + a_off[0], base + s.nb + b_off[0], s.a, wave,
@@ -401,7 +420,7 @@ struct Ring16Mainloop {
   // Step i loads the K tile at element offset min(k2_first + i*BK, k2_max); bmul: elements
   // between consecutive K rows of a [K][N] B operand.
   template <bool FULL>
-  static __device__ __forceinline__ void k_range(half8 (&a)[2][TM], half8 (&b)[2][TN],
+  static __device__ __forceinline__ void k_range(half8 (&a)[AB][TM], half8 (&b)[2][TN],
                                                  const half_t *const (&a_src)[Cfg::A_DMA],
                                                  const half_t *const (&b_src)[B_SRCS], const int (&a_off)[2],
                                                  const int (&b_off)[2], int steps, int k2_first, int k2_max,
@@ -474,7 +493,7 @@ struct Ring16Mainloop {
 
   // Phase 0: A(0) -> slot 0, B(0) -> slot 1, A(1) -> slot 2, B(1) -> slot 3, then
   // the fragments of K half 0 of tile 0 into a[0], b[0].
-  static __device__ __forceinline__ void prologue(half8 (&a)[2][TM], half8 (&b)[2][TN],
+  static __device__ __forceinline__ void prologue(half8 (&a)[AB][TM], half8 (&b)[2][TN],
                                                   const half_t *const (&a_src)[Cfg::A_DMA],
                                                   const half_t *const (&b_src)[B_SRCS], int KT,
                                                   const int (&a_off)[2], const int (&b_off)[2], int wave,
@@ -499,7 +518,7 @@ struct Ring16Mainloop {
     const int live_m = live_blocks(rows);
     int a_off[2], b_off[2];
     frag_offsets(a_off, b_off);
-    half8 a[2][TM], b[2][TN];
+    half8 a[AB][TM], b[2][TN];
     prologue(a, b, a_src, b_src, KT, a_off, b_off, wave, bmul);
     int phase = 0;
     reserve();

@@ -134,6 +134,7 @@ struct PlanReq {
                     // tiles; -n (n <= kSkinnyMaxWgs) = always, with n workgroups per XCD; -(kSkinnyMaxWgs + 1) =
                     // always as a launch of their own (needs `tail`)
   int sk_tail_ok;   // the skinny tiles may run as a launch of their own (the caller launches the kernels for it)
+  int sk_beside_ok; // they may run in workgroups of the persistent launch (its four-wavefront form only)
 };
 
 // A K step of a skinny tile, in percent of a 256-row tile's, when the whole chip runs skinny tiles
@@ -201,14 +202,14 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       if (nk1 > 0 && rq.skinny_pct < -kSkinnyMaxWgs) {
         tail_q = q_c;                                  // forced (tests, measurements); 0 = not possible: no skinny tiles
       } else if (nk1 > 0 && rq.skinny_pct < 0) {
-        ns_wgs = -rq.skinny_pct;                       // forced
+        ns_wgs = rq.sk_beside_ok ? -rq.skinny_pct : 0; // forced
       } else if (nk1 > 0) {
         const int cus_x = rq.cus / 8;
         const bool may_split = spx > 0;
         const int F0 = (nl0 * n_tiles_n + 7) / 8, F1 = (nl1 * n_tiles_n + 7) / 8, T_x = (nk1 * n_tiles_n + 7) / 8;
         int best = rounds_cost(F0, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts);
         const int sk_tile = (k_tiles * rq.skinny_pct + 99) / 100 + 3;         // one skinny tile, in K steps
-        for (int n = 1; n <= kSkinnyMaxWgs && n * 4 <= cus_x; ++n) {
+        for (int n = 1; n <= kSkinnyMaxWgs && n * 4 <= cus_x && rq.sk_beside_ok; ++n) {
           const int main_c = rounds_cost(F1, cus_x - n, k_tiles, rq.epi_cost, may_split, rq.max_parts);
           const int sk_c = (T_x + n - 1) / n * sk_tile;
           const int c = main_c > sk_c ? main_c : sk_c;

@@ -292,7 +292,7 @@ int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capaci
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, chunk_cnt, nchunk, E, capacity,
                      counts, offsets, cum_inout);
   if (int rc = check_launch("scan_kernel")) return rc;
-  const PlanReq none{0, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, 0, 0, 0, 0};
+  const PlanReq none{0, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
   const size_t pos_lds = sizeof(int) * kSub * E;
   if (pos_lds > 32768) {
     // with the plan builder's static arrays the kernel passes 64 KB of LDS for many experts

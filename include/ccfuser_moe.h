@@ -55,8 +55,10 @@ const char *ccf_last_error(void);
 /*
  * Tuning knobs (no counterpart in the reference).  Process-wide; not meant to
  * be changed while work is in flight.
- *   "gemm_variant"    0 (default, also -1) = the grouped GEMMs run as persistent workgroups, one per CU;
- *                     1 = one workgroup per tile for every K (otherwise only K < 256 runs that way)
+ *   "gemm_variant"    0 (default, also -1) = the grouped GEMMs run as persistent workgroups of four wavefronts,
+ *                     one per CU; 1 = one workgroup per tile for every K (otherwise only K < 256 runs that
+ *                     way); 2 = as 0; 3 = the forward GEMMs as persistent workgroups of eight wavefronts
+ *                     (same bits, measured no faster)
  *   "split_tail"      0 = off, 1 = default, n > 1 = for K of n*64 and more: the tiles of a launch's
  *                     last, partly filled round are cut along K and reduced by a second kernel
  *   "split_parts"     2..8 (default 8): most parts such a tile is cut into

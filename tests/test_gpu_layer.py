@@ -460,12 +460,13 @@ def _staged_forward(ops, args, E, k, capacity):
 
 
 @pytest.mark.parametrize("name,rows,variant", [("c3_mixtral", None, -1)] +
-                         [("c2_gshard", 1024, v) for v in (0, 1)])
+                         [("c2_gshard", 1024, v) for v in (0, 1, 2, 3)] + [("c5_skewed", None, 3), ("c3_mixtral", None, 3)])
 def test_fused_call_equals_stage_by_stage_calls(workloads, name, rows, variant):
     """In the fused call the routing stage builds the tile plans of both GEMMs; stand-alone
     GEMM calls build their own.  Same plans, same kernels, so the same bits: at full size on the
     benchmark shape (last round of tiles split along K in both GEMMs) and, on a small batch, for
-    both launch forms (persistent workgroups, one workgroup per tile)."""
+    every launch form (chosen by K, one workgroup per tile, persistent with four and with eight
+    wavefronts), the eight-wavefront form also at full size."""
     from ccfuser_amd import ops
     wl = workloads(name, rows) if rows else workloads(name)
     t = wl.tensors

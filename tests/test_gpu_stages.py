@@ -348,7 +348,7 @@ def _ffn_case(R, d, f, E, seed, skew=False):
     return x, w1, b1, w2, b2, e_of_row
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
 @pytest.mark.parametrize("R,d,f,E,skew,seed", [
     (512, 256, 1024, 4, False, 0),
     (700, 768, 3072, 32, True, 1),
@@ -387,6 +387,37 @@ def test_ffn_stages(variant, R, d, f, E, skew, seed):
         assert O.mean_rel_err(y.cpu(), y_ref) <= MEAN_REL
     finally:
         ops.set_option("gemm_variant", -1)
+
+
+@pytest.mark.parametrize("R,d,f,E,skew,seed", [
+    (9000, 1024, 2048, 8, False, 50),          # several rounds of tiles per workgroup, ragged last tiles
+    (3000, 768, 1536, 32, True, 51),           # many partly filled tiles (the eight-wavefront form computes their padding)
+    (700, 256, 320, 5, False, 52),             # four K tiles, N no multiple of 256
+])
+def test_eight_wavefront_kernel_gives_the_four_wavefront_bits(R, d, f, E, skew, seed):
+    """The persistent kernel with eight wavefronts per workgroup (one register buffer of token
+    fragments, refilled row block by row block) adds over K in the same order with the same
+    instruction as the four-wavefront form: both GEMMs must agree bit for bit."""
+    from ccfuser_amd import ops
+    x, w1, b1, w2, b2, e_of_row = _ffn_case(R, d, f, E, seed, skew)
+    r = ops.route(dev(e_of_row), E, 1)
+    _say(f"8 vs 4 wavefronts R={R} d={d} f={f} E={E} counts={r['counts'].tolist()[:10]}")
+    res = {}
+    ops.set_option("split_tail", 0)
+    try:
+        for variant in (2, 3):
+            ops.set_option("gemm_variant", variant)
+            h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True)
+            y = torch.zeros(R, d, dtype=torch.float16, device="cuda")
+            ops.ffn2(h, r["dst_row"], r["offsets"], R, dev(w2), dev(b2), y)
+            torch.cuda.synchronize()
+            res[variant] = (h.cpu(), y.cpu())
+    finally:
+        ops.set_option("gemm_variant", -1)
+        ops.set_option("split_tail", 1)
+    assert torch.isfinite(res[3][0].float()).all() and res[3][0].abs().sum() > 0
+    assert torch.equal(res[2][0], res[3][0]), "first GEMM"
+    assert torch.equal(res[2][1], res[3][1]), "second GEMM"
 
 
 def test_ffn_special_cases():
