@@ -54,7 +54,7 @@ SIGNATURES = {
 
 
 # libccfuser_probe.so (include/ccfuser_probe.h): measurement probes, not part of the product ABI
-PROBE_LIB_PATH = LIB_PATH.with_name("libccfuser_probe.so")
+PROBE_LIB_PATH = Path(__file__).resolve().parent / "libccfuser_probe.so"
 PROBE_SIGNATURES = {
     "ccf_probe_mfma": (_i, [_i, _i, _i, _p, C.POINTER(C.c_double), _p]),
     "ccf_probe_mfma_chain": (_i, [_p, _p, _i, _i, _p, _p]),

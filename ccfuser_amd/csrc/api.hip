@@ -164,8 +164,13 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
   hipStream_t st = as_stream(stream);
   int rc;
   mark_stage(0, st);
-  if ((rc = ccf_gate_topk_softmax(x, wg, bg, tokens, d_model, num_expert, top_k, CCF_F16, w.idx,
-                                  w.score, nullptr, stream)))
+  // the gate's selection threads also leave per-workgroup expert counts in the routing workspace when that
+  // table is small and a workgroup's flat indices tile the routing chunks (top_k a power of two): the
+  // routing stage is then one launch
+  int gate_tokens = 0;
+  const bool pow2_k = (top_k & (top_k - 1)) == 0;
+  if ((rc = gate_forward(x, wg, bg, tokens, d_model, num_expert, top_k, CCF_F16, w.idx, w.score, nullptr, stream,
+                         pow2_k ? reinterpret_cast<int32_t *>(w.route_ws) : nullptr, route_rows_max_ints(), &gate_tokens)))
     return rc;
   mark_stage(1, st);
   // the tile plans of both GEMMs are built by two more workgroups of the routing stage's last
@@ -181,7 +186,7 @@ extern "C" int ccf_moe_forward(const void *x, const void *wg, const void *bg, co
                        forward_plan_request(fuse ? 3 : 2, n, num_expert, d_model, d_ffn, w.ffn_ws, opt, &plans[1]);
   if ((rc = route_with_plans(w.idx, n, num_expert, top_k, capacity, w.counts, w.offsets, w.pos, w.src_row,
                              w.dst_row, w.inv_pos, w.idx_kept, w.route_ws, w.route_bytes, st, plans,
-                             planned ? 2 : 0)))
+                             planned ? 2 : 0, gate_tokens * top_k)))
     return rc;
   mark_stage(2, st);
   if ((rc = ffn1_forward(x, w.src_row, nullptr, w.offsets, n, num_expert, d_model, d_ffn, w1, b1, 1, w.h,

@@ -51,8 +51,14 @@ int launch_transpose_rows(const half_t *in, const int32_t *rows, const int32_t *
 int launch_bias_reduce(const float *partial, const int32_t *k_seg, int E, int C, half_t *grad_bias,
                        hipStream_t stream);
 
+// gate.hip
+int gate_forward(const void *x, const void *wg, const void *bg, int tokens, int d_model, int tot_expert, int top_k,
+                 int dtype, int64_t *idx_out, void *score_out, void *logits_out, ccf_stream_t stream,
+                 int32_t *wg_cnt, long long max_cnt, int *tokens_per_wg);
+
 // tuning knobs set through ccf_set_option()
 extern int g_gate_waves, g_gate_slots;   // gate.hip
+extern int g_route_rows_max;             // route.hip
 
 }  // namespace ccf
 

@@ -1345,6 +1345,11 @@ extern "C" int ccf_set_option(const char *name, int value) {
     g_fused_combine = value != 0;
     return CCF_OK;
   }
+  if (!strcmp(name, "route_rows_max")) {
+    CCF_REQUIRE(value >= 0 && value <= 32768, CCF_ERR_ARG, "set_option: route_rows_max %d outside 0..32768", value);
+    g_route_rows_max = value;
+    return CCF_OK;
+  }
   if (!strcmp(name, "gate_slots")) {
     CCF_REQUIRE(value == 0 || value == 1 || value == 2 || value == 4, CCF_ERR_ARG,
                 "set_option: gate_slots %d is none of 0, 1, 2, 4", value);

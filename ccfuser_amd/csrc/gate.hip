@@ -129,7 +129,7 @@ template <int N, int LS, int KS>
 __global__ void __launch_bounds__(kMaxWaves * 64)
 gate_mfma_kernel(const half_t *__restrict__ x, const half_t *__restrict__ wg, const half_t *__restrict__ bg,
                  int tokens, int d, int E, int k, int64_t *__restrict__ idx_out,
-                 half_t *__restrict__ score_out, half_t *__restrict__ logits_out) {
+                 half_t *__restrict__ score_out, half_t *__restrict__ logits_out, int32_t *__restrict__ wg_cnt) {
   using M = Mfma<N>;
   constexpr int kBlocks = 64 / N;
   constexpr int S = 1 << LS;
@@ -315,6 +315,21 @@ gate_mfma_kernel(const half_t *__restrict__ x, const half_t *__restrict__ wg, co
   }
   if (threadIdx.x < TW && t0 + threadIdx.x < tokens)
     best.template write<half_t>(t0 + threadIdx.x, k, idx_out, score_out);
+  if (wg_cnt) {
+    // How many of this workgroup's token slots chose each expert, for the routing stage: the
+    // selection threads hold the ids, so the routing needs no pass of its own over idx to count
+    // them.  The wavefronts' regions are free since the last barrier.
+    int *row = reinterpret_cast<int *>(s_mem);
+    for (int e = threadIdx.x; e < E; e += blockDim.x) row[e] = 0;
+    __syncthreads();
+    if (threadIdx.x < TW && t0 + threadIdx.x < tokens) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        if (s < k) atomicAdd(&row[best.id[s]], 1);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) wg_cnt[static_cast<size_t>(blockIdx.x) * E + e] = row[e];
+  }
 }
 
 // fp32 gate on the vector unit, one wavefront per token: a lane takes one (expert, part)
@@ -372,11 +387,14 @@ gate_f32_kernel(const float *__restrict__ x, const float *__restrict__ wg, const
 }  // namespace
 }  // namespace ccf
 
-extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *bg, int tokens,
-                                     int d_model, int tot_expert, int top_k, int dtype,
-                                     int64_t *idx_out, void *score_out, void *logits_out,
-                                     ccf_stream_t stream) {
-  using namespace ccf;
+namespace ccf {
+// The gate; with wg_cnt (room for max_cnt ints) the fp16 kernel also leaves, per workgroup, how many of
+// its token slots chose each expert ([workgroups][tot_expert], a workgroup covering *tokens_per_wg
+// consecutive tokens), when that table fits; *tokens_per_wg = 0 says it was not written.
+int gate_forward(const void *x, const void *wg, const void *bg, int tokens, int d_model, int tot_expert, int top_k,
+                 int dtype, int64_t *idx_out, void *score_out, void *logits_out, ccf_stream_t stream,
+                 int32_t *wg_cnt, long long max_cnt, int *tokens_per_wg) {
+  if (tokens_per_wg) *tokens_per_wg = 0;
   CCF_REQUIRE(x && wg && idx_out && score_out, CCF_ERR_ARG, "gate: null pointer");
   CCF_REQUIRE(tokens >= 0 && d_model > 0 && tot_expert > 0, CCF_ERR_ARG, "gate: bad size");
   CCF_REQUIRE(d_model % 8 == 0, CCF_ERR_SHAPE, "gate: d_model=%d is not a multiple of 8", d_model);
@@ -420,6 +438,11 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
   const size_t lds = sizeof(float) * (static_cast<size_t>(waves) * kRegionFloats + static_cast<size_t>(tw) * (n + 1));
   CCF_REQUIRE(lds <= 160 * 1024, CCF_ERR_SHAPE, "gate: %zu bytes of LDS needed", lds);
   dim3 grid((tokens + tw - 1) / tw), block(waves * 64);
+  if (wg_cnt && static_cast<long long>(grid.x) * tot_expert <= max_cnt) {
+    if (tokens_per_wg) *tokens_per_wg = tw;
+  } else {
+    wg_cnt = nullptr;
+  }
 #define CCF_GATE_LAUNCH(NN, LSV, KSV)                                                              \
   do {                                                                                             \
     auto kern = gate_mfma_kernel<NN, LSV, KSV>;                                                    \
@@ -432,7 +455,7 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
     hipLaunchKernelGGL(kern, grid, block, lds, as_stream(stream), static_cast<const half_t *>(x),  \
                        static_cast<const half_t *>(wg), static_cast<const half_t *>(bg), tokens,   \
                        d_model, tot_expert, top_k, idx_out, static_cast<half_t *>(score_out),      \
-                       static_cast<half_t *>(logits_out));                                         \
+                       static_cast<half_t *>(logits_out), wg_cnt);                                 \
   } while (0)
 #define CCF_GATE_K(NN, LSV)                                                  \
   do {                                                                       \
@@ -446,4 +469,13 @@ extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *
 #undef CCF_GATE_K
 #undef CCF_GATE_LAUNCH
   return check_launch("gate_mfma_kernel");
+}
+}  // namespace ccf
+
+extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *bg, int tokens,
+                                     int d_model, int tot_expert, int top_k, int dtype,
+                                     int64_t *idx_out, void *score_out, void *logits_out,
+                                     ccf_stream_t stream) {
+  return ccf::gate_forward(x, wg, bg, tokens, d_model, tot_expert, top_k, dtype, idx_out, score_out, logits_out, stream,
+                           nullptr, 0, nullptr);
 }

@@ -399,10 +399,13 @@ int ffn2_forward_combine(const void *h, const int32_t *token_row, const int32_t 
                          int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
                          const void *score, void *out, void *workspace, size_t workspace_bytes, hipStream_t stream,
                          const GemmOptions *planned);
-// route.hip: ccf_route(), whose last launch also builds n_plans (0..2) tile plans from the offsets
+// route.hip: ccf_route(), whose last launch also builds n_plans (0..2) tile plans from the offsets.  gate_row_len > 0:
+// the head of the workspace already holds the gate kernel's counts, one row per gate_row_len flat indices.
 int route_with_plans(const int64_t *gate_idx, int n_flat, int num_expert, int top_k, int capacity,
                      int32_t *counts, int32_t *offsets, int64_t *pos, int32_t *src_row, int32_t *dst_row,
                      int32_t *inv_pos, int64_t *idx_kept, void *workspace, size_t workspace_bytes,
-                     hipStream_t stream, const PlanReq *plans, int n_plans);
+                     hipStream_t stream, const PlanReq *plans, int n_plans, int gate_row_len);
+// most entries of a table of per-run expert counts that the routing stage takes from the gate kernel
+long long route_rows_max_ints();
 
 }  // namespace ccf

@@ -7,7 +7,7 @@
 // here the flat indices inside a segment ascend, which is one of the orders
 // that race can produce, and everything stays on the device.
 //
-// Three small launches over chunks of kChunk flat indices:
+// Small launches over chunks of kChunk flat indices:
 //   hist   per chunk, per expert counts (wavefront match + LDS integer adds)
 //   scan   one workgroup: per expert running sums over chunks, capacity clamp,
 //          exclusive scan over experts
@@ -15,6 +15,13 @@
 //          earlier wavefront passes in the chunk + lanes before it in the
 //          wavefront (ballot / popcount), then the scatter of pos and friends
 // Integer adds commute, so the results do not depend on scheduling.
+//
+// When the table of counts is small (at most kRowsMaxInts entries) there is no scan launch:
+// every workgroup of the pos launch adds up the rows in front of its chunk and all rows
+// itself (a few thousand integers out of L2), which is cheaper than a launch.  The rows are
+// then the hist launch's, one per chunk, or, in the layer's forward call, rows the gate
+// kernel left, one per gate workgroup (its selection threads hold the expert ids), and the
+// routing stage is the pos launch alone.
 #include "ccf_common.h"
 #include "plan.h"
 
@@ -28,6 +35,7 @@ constexpr int kStaticScratchInts = 1 << 18;
 static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
 
 namespace ccf {
+int g_route_rows_max = 16384;   // largest table of counts (entries) that the pos launch sums itself; 0: always a scan launch
 namespace {
 
 constexpr int kThreads = 256;
@@ -35,6 +43,7 @@ constexpr int kPasses = 4;                       // indices per thread
 constexpr int kChunk = kThreads * kPasses;       // flat indices per workgroup
 constexpr int kSub = kPasses * (kThreads / 64);  // wavefront passes per chunk
 constexpr int kMaxExpert = 1024;
+constexpr int kRowsMaxInts = 32768;              // largest table of counts that the pos launch sums itself
 
 __device__ inline uint64_t lanes_below() {
   const int lane = threadIdx.x & 63;
@@ -147,18 +156,86 @@ scan_kernel(int32_t *__restrict__ chunk_cnt, int nchunk, int E, int capacity,
 
 __global__ void __launch_bounds__(kThreads)
 pos_kernel(const int64_t *__restrict__ idx, int n, int E, int nbits, int top_k, int capacity,
-           const int32_t *__restrict__ chunk_base, const int32_t *__restrict__ offsets,
+           const int32_t *chunk_base, const int32_t *offsets,
            int64_t *__restrict__ pos, int32_t *__restrict__ src_row,
            int32_t *__restrict__ dst_row, int32_t *__restrict__ inv_pos,
-           int64_t *__restrict__ idx_kept, int nchunk, int plan_wgs, PlanReq plan0, PlanReq plan1) {
+           int64_t *__restrict__ idx_kept, int nchunk, int plan_wgs, PlanReq plan0, PlanReq plan1,
+           const int32_t *__restrict__ rows, int nrows, int rows_per_chunk, int32_t *__restrict__ counts_out,
+           int32_t *__restrict__ offsets_out) {
+  extern __shared__ int s_sub[];                 // [kSub][E], then with `rows`: [E] chunk base, [E] totals, [E + 1] offsets
+  const bool is_plan = static_cast<int>(blockIdx.x) >= nchunk;
+  if (rows) {
+    // No scan launch: rows [nrows][E] hold counts of consecutive, equally long runs of flat
+    // indices, rows_per_chunk of them per chunk.  Every workgroup adds up the rows in front of
+    // its chunk (its rank base) and all rows (the experts' totals, hence the offsets).
+    int *s_base = s_sub + kSub * E, *s_tot = s_base + E, *s_off = s_tot + E;
+    for (int e = threadIdx.x; e < E; e += kThreads) { s_base[e] = 0; s_tot[e] = 0; }
+    __syncthreads();
+    const int first = is_plan ? 0 : static_cast<int>(blockIdx.x) * rows_per_chunk;   // rows in front of this chunk
+    if (E <= kThreads) {
+      // thread t: expert t % E, rows t / E, t / E + G, ...; sums in registers, one LDS add per thread at the end
+      const int G = kThreads / E, e = threadIdx.x % E, grp = threadIdx.x / E;
+      if (grp < G) {
+        int tot = 0, base = 0;
+        const int32_t *col = rows + e;
+#pragma unroll 8
+        for (int g = grp; g < nrows; g += G) {
+          const int v = col[static_cast<size_t>(g) * E];
+          tot += v;
+          base += g < first ? v : 0;
+        }
+        atomicAdd(&s_tot[e], tot);
+        atomicAdd(&s_base[e], base);
+      }
+    } else {
+      for (int e = threadIdx.x; e < E; e += kThreads) {
+        int tot = 0, base = 0;
+#pragma unroll 8
+        for (int g = 0; g < nrows; ++g) {
+          const int v = rows[static_cast<size_t>(g) * E + e];
+          tot += v;
+          base += g < first ? v : 0;
+        }
+        s_tot[e] = tot;
+        s_base[e] = base;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+      // capacity clamp and exclusive scan over experts by one wavefront, 64 at a time
+      int carry = 0;
+      const int lane = threadIdx.x;
+      for (int e0 = 0; e0 < E; e0 += 64) {
+        int v = 0;
+        if (e0 + lane < E) {
+          v = s_tot[e0 + lane];
+          v = (capacity >= 0 && v > capacity) ? capacity : v;
+          if (blockIdx.x == 0 && counts_out) counts_out[e0 + lane] = v;
+        }
+        int inc = v;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          int o = __shfl_up(inc, off, 64);
+          if (lane >= off) inc += o;
+        }
+        if (e0 + lane < E) s_off[e0 + lane] = carry + inc - v;
+        carry += __shfl(inc, 63, 64);
+      }
+      if (lane == 0) s_off[E] = carry;
+    }
+    __syncthreads();
+    if (blockIdx.x == 0)
+      for (int e = threadIdx.x; e <= E; e += kThreads) offsets_out[e] = s_off[e];
+    chunk_base = nullptr;
+    offsets = s_off;
+  }
   // Workgroups past the chunks build the tile plans of the GEMMs that follow: the offsets are
-  // final since the scan, and the plans then cost no launch of their own.
-  if (static_cast<int>(blockIdx.x) >= nchunk) {
+  // final, and the plans then cost no launch of their own.
+  if (is_plan) {
     const int r = static_cast<int>(blockIdx.x) - nchunk;        // plan_wgs workgroups per plan
     build_plan(r < plan_wgs ? plan0 : plan1, offsets, E, r % plan_wgs, plan_wgs);
     return;
   }
-  extern __shared__ int s_sub[];                 // [kSub][E]
   for (int i = threadIdx.x; i < kSub * E; i += kThreads) s_sub[i] = 0;
   __syncthreads();
   const int base = blockIdx.x * kChunk;
@@ -178,7 +255,7 @@ pos_kernel(const int64_t *__restrict__ idx, int n, int E, int nbits, int top_k, 
   __syncthreads();
   // exclusive running sum over the kSub wavefront passes, per expert
   for (int e = threadIdx.x; e < E; e += kThreads) {
-    int run = chunk_base[static_cast<size_t>(blockIdx.x) * E + e];
+    int run = chunk_base ? chunk_base[static_cast<size_t>(blockIdx.x) * E + e] : s_sub[kSub * E + e];
 #pragma unroll
     for (int s = 0; s < kSub; ++s) {
       int v = s_sub[s * E + e];
@@ -261,22 +338,21 @@ int ceil_log2(int v) {
   return b;
 }
 
-struct RouteWs {
-  int32_t *chunk_cnt;   // [nchunk][E]
-  int nchunk;
-};
-
 size_t route_ws_bytes(int n_flat, int E) {
   int nchunk = (n_flat + kChunk - 1) / kChunk;
   if (nchunk < 1) nchunk = 1;
-  return round_up(sizeof(int32_t) * static_cast<size_t>(nchunk) * E, 256);
+  size_t ints = static_cast<size_t>(nchunk) * E;
+  ints = ints < kRowsMaxInts ? kRowsMaxInts : ints;   // room for the gate's rows (finer than chunks) when the table is small
+  return round_up(sizeof(int32_t) * ints, 256);
 }
 
+// gate_rows: the table of counts is already in the workspace, one row per gate_row_len flat indices
+// (left there by the gate kernel); 0: the hist launch makes it, one row per chunk.
 int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capacity,
                int32_t *counts, int32_t *offsets, int32_t *cum_inout, int64_t *pos,
                int32_t *src_row, int32_t *dst_row, int32_t *inv_pos, int64_t *idx_kept,
                void *ws, size_t ws_bytes, hipStream_t stream, const PlanReq *plans = nullptr,
-               int n_plans = 0) {
+               int n_plans = 0, int gate_row_len = 0) {
   CCF_REQUIRE(gate_idx && pos, CCF_ERR_ARG, "route: null pointer");
   CCF_REQUIRE(n_plans >= 0 && n_plans <= 2 && (n_plans == 0 || plans), CCF_ERR_ARG, "route: bad plan requests");
   CCF_REQUIRE(n_flat >= 0 && E > 0 && top_k >= 1, CCF_ERR_ARG, "route: bad size");
@@ -286,14 +362,27 @@ int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capaci
   const int nchunk = n_flat > 0 ? (n_flat + kChunk - 1) / kChunk : 1;
   const int nbits = ceil_log2(E);
   int32_t *chunk_cnt = static_cast<int32_t *>(ws);
-  hipLaunchKernelGGL(hist_kernel, dim3(nchunk), dim3(kThreads), sizeof(int) * E, stream, gate_idx,
-                     n_flat, E, nbits, chunk_cnt, static_cast<int32_t *>(nullptr));
-  if (int rc = check_launch("hist_kernel")) return rc;
-  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, chunk_cnt, nchunk, E, capacity,
-                     counts, offsets, cum_inout);
-  if (int rc = check_launch("scan_kernel")) return rc;
+  // the table of counts: the gate's rows, or one row per chunk from the hist launch
+  int nrows = nchunk, rows_per_chunk = 1;
+  if (gate_row_len > 0) {
+    CCF_REQUIRE(kChunk % gate_row_len == 0 && !cum_inout, CCF_ERR_ARG, "route: rows of %d indices do not tile a chunk", gate_row_len);
+    nrows = (n_flat + gate_row_len - 1) / gate_row_len;
+    rows_per_chunk = kChunk / gate_row_len;
+    CCF_REQUIRE(static_cast<long long>(nrows) * E <= kRowsMaxInts, CCF_ERR_ARG, "route: table of counts too large");
+  } else {
+    hipLaunchKernelGGL(hist_kernel, dim3(nchunk), dim3(kThreads), sizeof(int) * E, stream, gate_idx,
+                       n_flat, E, nbits, chunk_cnt, static_cast<int32_t *>(nullptr));
+    if (int rc = check_launch("hist_kernel")) return rc;
+  }
+  // small table: the pos launch sums the rows itself; otherwise (or with caller-given segment ends) a scan launch
+  const bool sum_rows = !cum_inout && (gate_row_len > 0 || static_cast<long long>(nrows) * E <= g_route_rows_max);
+  if (!sum_rows) {
+    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, chunk_cnt, nchunk, E, capacity,
+                       counts, offsets, cum_inout);
+    if (int rc = check_launch("scan_kernel")) return rc;
+  }
   const PlanReq none{0, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
-  const size_t pos_lds = sizeof(int) * kSub * E;
+  const size_t pos_lds = sizeof(int) * (static_cast<size_t>(kSub + (sum_rows ? 3 : 0)) * E + 1);
   if (pos_lds > 32768) {
     // with the plan builder's static arrays the kernel passes 64 KB of LDS for many experts
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(pos_kernel),
@@ -306,7 +395,8 @@ int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capaci
   hipLaunchKernelGGL(pos_kernel, dim3(nchunk + n_plans * plan_wgs), dim3(kThreads), pos_lds, stream,
                      gate_idx, n_flat, E, nbits, top_k, capacity, chunk_cnt, offsets, pos, src_row,
                      dst_row, inv_pos, idx_kept, nchunk, plan_wgs, n_plans > 0 ? plans[0] : none,
-                     n_plans > 1 ? plans[1] : none);
+                     n_plans > 1 ? plans[1] : none, sum_rows ? chunk_cnt : static_cast<int32_t *>(nullptr), nrows,
+                     rows_per_chunk, counts, offsets);
   return check_launch("pos_kernel");
 }
 
@@ -437,11 +527,12 @@ namespace ccf {
 int route_with_plans(const int64_t *gate_idx, int n_flat, int num_expert, int top_k, int capacity,
                      int32_t *counts, int32_t *offsets, int64_t *pos, int32_t *src_row, int32_t *dst_row,
                      int32_t *inv_pos, int64_t *idx_kept, void *workspace, size_t workspace_bytes,
-                     hipStream_t stream, const PlanReq *plans, int n_plans) {
+                     hipStream_t stream, const PlanReq *plans, int n_plans, int gate_row_len) {
   CCF_REQUIRE(counts && offsets, CCF_ERR_ARG, "route: null counts/offsets");
   return route_impl(gate_idx, n_flat, num_expert, top_k, capacity, counts, offsets, nullptr, pos, src_row,
-                    dst_row, inv_pos, idx_kept, workspace, workspace_bytes, stream, plans, n_plans);
+                    dst_row, inv_pos, idx_kept, workspace, workspace_bytes, stream, plans, n_plans, gate_row_len);
 }
+long long route_rows_max_ints() { return g_route_rows_max < kRowsMaxInts ? g_route_rows_max : kRowsMaxInts; }
 }  // namespace ccf
 
 extern "C" int ccf_route(const int64_t *gate_idx, int n_flat, int num_expert, int top_k,

@@ -72,6 +72,10 @@ const char *ccf_last_error(void);
  *   "fused_combine"   0/1 (default 0): ccf_moe_forward with top_k = 2 adds the gate-weighted expert outputs
  *                     into the output in the second GEMM's epilogue (packed fp16 atomic adds onto zeros)
  *                     instead of running the combine pass; measured slower, kept for comparison
+ *   "route_rows_max"  0..32768 (default 16384): the largest table of per-run expert counts (entries) that the
+ *                     routing stage's last launch sums itself instead of running a scan launch; in
+ *                     ccf_moe_forward the gate kernel leaves such a table when it fits (and top_k is a power
+ *                     of two), and the routing stage is then one launch.  0 = always histogram, scan, pos
  *   "gate_slots"      0, 1, 2 or 4: parts of K a gate wavefront works on at a time, which divides the tokens
  *                     of a workgroup by the same number (0 = chosen by the token count)
  *   "dgrad_transpose" 0/1: the backward's input-gradient GEMM runs on a transposed copy of the

@@ -481,10 +481,13 @@ def test_fused_call_equals_stage_by_stage_calls(workloads, name, rows, variant):
         ops.set_option("gemm_variant", -1)
 
 
-@pytest.mark.parametrize("T,d,f,E,k", [(2048, 64, 128, 600, 2), (4096, 128, 64, 1024, 1), (300, 64, 64, 37, 4)])
+@pytest.mark.parametrize("T,d,f,E,k", [(2048, 64, 128, 600, 2), (4096, 128, 64, 1024, 1), (300, 64, 64, 37, 4),
+                                       (1000, 128, 64, 20, 3), (5000, 256, 64, 8, 8)])
 def test_fused_layer_with_many_experts(T, d, f, E, k):
     """Most experts get a handful of rows or none; the routing launch builds the tile plans with
-    eight workgroups per plan and needs more than 64 KB of LDS past 512 experts."""
+    eight workgroups per plan and needs more than 64 KB of LDS past 512 experts.  The cases also
+    cover the ways the routing stage gets its counts: from the gate kernel's workgroups (top-k
+    a power of two, small table), from its own histogram launch (1024 experts; top-3)."""
     from ccfuser_amd import ops
     g = torch.Generator().manual_seed(E)
     r = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).half()

@@ -216,6 +216,8 @@ def test_gate_ties_go_to_lower_expert():
     (1, 4, 1, -1, 0), (63, 4, 1, -1, 1), (1024, 8, 2, -1, 2), (1025, 8, 1, -1, 3),
     (16384, 8, 2, 2560, 4), (32768, 32, 1, -1, 5), (5000, 70, 2, 40, 6), (4096, 1000, 2, -1, 7),
     (3000, 3, 1, 0, 8),
+    (70000, 600, 2, -1, 9),        # a table of counts too large for the pos launch to sum: the scan launch runs
+    (40000, 900, 1, 30, 10),       # the same with a capacity
 ])
 def test_route_bit_exact(n, E, k, cap, seed):
     from ccfuser_amd import ops
