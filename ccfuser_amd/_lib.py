@@ -45,6 +45,7 @@ SIGNATURES = {
     "ccf_ffn1_forward_keep": (_i, [_p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
     "ccf_ffn2_backward": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
     "ccf_ffn1_backward": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
+    "ccf_ffn1_backward_gelu": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _sz, _p]),
     "ccf_moe_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "ccf_moe_forward": (_i, [_p] * 7 + [_i] * 6 + [_p] * 6 + [_p, _sz, _p]),
     "ccf_moe_forward_set_events": (_i, [C.POINTER(_p), _i]),

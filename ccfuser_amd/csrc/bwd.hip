@@ -21,6 +21,7 @@
 //     the result does not depend on scheduling.
 // The reference leaves grad_bias uninitialised (mix_moe.h:342, 488).
 #include "ccf_common.h"
+#include "gelu.h"
 
 namespace ccf {
 namespace {
@@ -107,10 +108,14 @@ transpose_weights_kernel(const half_t *__restrict__ in, half_t *__restrict__ out
 // out_t[c][64 * b + i] = in[rows[row0_b + i]][c] for i < cnt_b, else 0; one
 // workgroup per (64-row block b, 64-column tile).  partial[b][c] (optional) =
 // sum over the block's rows of column c, in row order, fp32.
+// kGelu: the rows are gradients of gelu(pre) (same layout, no row index): they are multiplied by
+// gelu'(pre), written back in place, and what is transposed and summed is the product.
+template <bool kGelu>
 __global__ void __launch_bounds__(256)
-transpose_rows_kernel(const half_t *__restrict__ in, const int32_t *__restrict__ rows,
+transpose_rows_kernel(half_t *in, const int32_t *__restrict__ rows,
                       const int32_t *__restrict__ blk_row0, const int32_t *__restrict__ blk_cnt,
-                      int C, int ld_t, half_t *__restrict__ out_t, float *__restrict__ partial) {
+                      int C, int ld_t, half_t *__restrict__ out_t, float *__restrict__ partial,
+                      const half_t *__restrict__ pre) {
   __shared__ half_t tile[kTile][kTile + 8];
   const int b = blockIdx.x, c0 = blockIdx.y * kTile;
   const int cnt = blk_cnt[b];
@@ -122,8 +127,15 @@ transpose_rows_kernel(const half_t *__restrict__ in, const int32_t *__restrict__
     const int i = q >> 3, ch = q & 7;
     half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
     if (i < cnt) {
-      const size_t r = rows ? static_cast<size_t>(rows[row0 + i]) : static_cast<size_t>(row0 + i);
+      const size_t r = (!kGelu && rows) ? static_cast<size_t>(rows[row0 + i]) : static_cast<size_t>(row0 + i);
       v = *reinterpret_cast<const half8 *>(in + r * C + c0 + ch * 8);
+      if constexpr (kGelu) {
+        const half8 p = *reinterpret_cast<const half8 *>(pre + r * C + c0 + ch * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          v[j] = static_cast<half_t>(static_cast<float>(v[j]) * gelu_erf_grad(static_cast<float>(p[j])));
+        *reinterpret_cast<half8 *>(in + r * C + c0 + ch * 8) = v;
+      }
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) tile[i][ch * 8 + j] = v[j];
@@ -231,9 +243,14 @@ int launch_transpose_weights(const half_t *in, half_t *out, int E, int R, int C,
 
 int launch_transpose_rows(const half_t *in, const int32_t *rows, const int32_t *blk_row0,
                           const int32_t *blk_cnt, int n_blk, int C, int ld_t, half_t *out_t,
-                          float *partial, hipStream_t stream) {
-  hipLaunchKernelGGL(transpose_rows_kernel, dim3(n_blk, C / kTile), dim3(256), 0, stream, in, rows,
-                     blk_row0, blk_cnt, C, ld_t, out_t, partial);
+                          float *partial, hipStream_t stream, const half_t *gelu_pre_inplace) {
+  half_t *src = const_cast<half_t *>(in);             // written only in the GELU form
+  if (gelu_pre_inplace)
+    hipLaunchKernelGGL(transpose_rows_kernel<true>, dim3(n_blk, C / kTile), dim3(256), 0, stream, src, rows,
+                       blk_row0, blk_cnt, C, ld_t, out_t, partial, gelu_pre_inplace);
+  else
+    hipLaunchKernelGGL(transpose_rows_kernel<false>, dim3(n_blk, C / kTile), dim3(256), 0, stream, src, rows,
+                       blk_row0, blk_cnt, C, ld_t, out_t, partial, static_cast<const half_t *>(nullptr));
   return check_launch("transpose_rows_kernel");
 }
 

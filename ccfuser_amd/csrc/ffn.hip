@@ -17,6 +17,7 @@
 // derives the tile list from the offsets on the device.
 #include "ccf_common.h"
 #include "gemm_tile.h"
+#include "gelu.h"
 #include "plan.h"
 
 namespace ccf {
@@ -61,49 +62,6 @@ struct GroupedArgs {
   const int32_t *skinny;
   float *sk_partial;        // partial tiles of the skinny tiles when they run as a launch of their own
 };
-
-// erf-form GELU, v * Phi(v) with Phi(v) = 0.5 + 0.5*erf(v/sqrt2) = 0.5 + u*Q(u^2), u = v
-// clamped to +-3*sqrt2 (beyond it 1 - erf < 2.3e-5).  0.5*erf(u/sqrt2) is an odd minimax
-// polynomial u*Q(u^2) of degree 8 in u^2, fitted on [0, 3] in z = u/sqrt2 with the 1/sqrt2
-// and the 0.5 folded into the coefficients.  Measured in fp32 against the exact function:
-// within 1.4e-5 for |v| <= 2, 5.9e-5 for |v| <= 8 (at -8 the result is -2e-5 instead of -0),
-// an eighth of the fp16 rounding step of a result of magnitude 1.  12 full-rate instructions
-// with the fp16 conversion and no transcendental (the library erff is ~40, the exp-based form
-// 15 plus rcp and exp at quarter rate); the FFN1 epilogue applies it to 256 values per lane
-// and tile and is bound by this arithmetic.
-__device__ __forceinline__ float gelu_erf(float v) {
-  const float u = __builtin_amdgcn_fmed3f(v, -4.2426406871192851464f, 4.2426406871192851464f);
-  const float t = u * u;
-  float q = 1.1253530e-10f * 0.5f;
-  q = fmaf(q, t, -1.0743734e-08f * 0.5f);
-  q = fmaf(q, t, 4.5365911e-07f * 0.5f);
-  q = fmaf(q, t, -1.1292428e-05f * 0.5f);
-  q = fmaf(q, t, 1.8718123e-04f * 0.5f);
-  q = fmaf(q, t, -2.2188006e-03f * 0.5f);
-  q = fmaf(q, t, 1.9636238e-02f * 0.5f);
-  q = fmaf(q, t, -1.3269384e-01f * 0.5f);
-  q = fmaf(q, t, 7.9780629e-01f * 0.5f);
-  return v * fmaf(u, q, 0.5f);
-}
-
-// Derivative of the erf GELU, Phi(v) + v*phi(v), with the same erf polynomial.
-__device__ __forceinline__ float gelu_erf_grad(float v) {
-  const float u = fminf(fabsf(v), 4.2426406871192851464f);
-  const float t = u * u;
-  float q = 1.1253530e-10f * 0.5f;
-  q = fmaf(q, t, -1.0743734e-08f * 0.5f);
-  q = fmaf(q, t, 4.5365911e-07f * 0.5f);
-  q = fmaf(q, t, -1.1292428e-05f * 0.5f);
-  q = fmaf(q, t, 1.8718123e-04f * 0.5f);
-  q = fmaf(q, t, -2.2188006e-03f * 0.5f);
-  q = fmaf(q, t, 1.9636238e-02f * 0.5f);
-  q = fmaf(q, t, -1.3269384e-01f * 0.5f);
-  q = fmaf(q, t, 7.9780629e-01f * 0.5f);
-  const float half_erf = copysignf(fminf(q * u, 0.5f), v);        // 0.5 * erf(v / sqrt2)
-  // phi(v) = exp(-v^2/2) / sqrt(2 pi) = exp2(-v^2 * log2(e)/2) * 0.3989...
-  const float pdf = 0.3989422804014327f * __builtin_amdgcn_exp2f(-0.72134752044448170368f * v * v);
-  return fmaf(v, pdf, 0.5f + half_erf);
-}
 
 // Epilogue forms of the grouped GEMM.
 //   0  C = (acc + bias) * row_scale
@@ -1255,11 +1213,12 @@ int zero_param_grads(void *grad_w, void *grad_b, int E, int n_out, int n_in, hip
 // (through in_rows):
 //   grad_in[gi_rows(j)] = grad_out[g_rows(j)] * w[e]            (grouped GEMM on w^T)
 //   grad_w[e] = grad_out_e^T * in_e,  grad_b[e] = column sums of grad_out_e
-int linear_backward(const half_t *grad_out, const int32_t *g_rows, const half_t *in,
+int linear_backward(half_t *grad_out, const int32_t *g_rows, const half_t *in,
                     const int32_t *in_rows, const int32_t *offsets, int max_rows, int E, int n_in,
                     int n_out, const half_t *w, half_t *grad_in, const int32_t *gi_rows,
                     half_t *grad_w, half_t *grad_b, void *workspace, size_t workspace_bytes,
-                    int d, int f, hipStream_t stream, const char *what, const half_t *gelu_pre = nullptr) {
+                    int d, int f, hipStream_t stream, const char *what, const half_t *gelu_pre = nullptr,
+                    const half_t *pre_inplace = nullptr) {
   CCF_REQUIRE(grad_out && in && offsets && w && grad_in && grad_w && grad_b, CCF_ERR_ARG,
               "%s: null pointer", what);
   CCF_REQUIRE(max_rows >= 0 && E > 0 && E <= 1024 && d > 0 && f > 0, CCF_ERR_ARG, "%s: bad size", what);
@@ -1272,6 +1231,17 @@ int linear_backward(const half_t *grad_out, const int32_t *g_rows, const half_t 
   CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
               "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);
   const BackwardWs ws = carve_backward(workspace, max_rows, E, d, f);
+  // K ranges of the weight-gradient GEMM, then the transposed copy of the gradient rows (with the bias
+  // gradient's partial sums).  With pre_inplace the incoming rows are gradients of gelu(pre): the same
+  // pass multiplies them by gelu'(pre) and writes them back, so that everything below sees the
+  // gradient of the pre-activation.
+  CCF_REQUIRE(!pre_inplace || !g_rows, CCF_ERR_ARG, "%s: the in-place GELU gradient needs rows in expert order", what);
+  if (int rc = launch_kseg(offsets, E, max_rows, n_out, ws.n_blk, ws.k_seg, ws.row_off, ws.blk_row0,
+                           ws.blk_cnt, stream))
+    return rc;
+  if (int rc = launch_transpose_rows(grad_out, g_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_out, ws.ld_t,
+                                     ws.a_t, ws.partial, stream, pre_inplace))
+    return rc;
   // input gradient: on the stored weight read as [K][N] where the shape allows, else on a transposed copy
   const bool kn = !g_dgrad_transpose && n_in % Cfg5::BN == 0 && static_cast<long long>(n_out) * n_in < (1ll << 31);
   if (!kn) {
@@ -1284,14 +1254,8 @@ int linear_backward(const half_t *grad_out, const int32_t *g_rows, const half_t 
                             what, kn, const_cast<half_t *>(gelu_pre)))
     return rc;
   // weight and bias gradients
-  if (int rc = launch_kseg(offsets, E, max_rows, n_out, ws.n_blk, ws.k_seg, ws.row_off, ws.blk_row0,
-                           ws.blk_cnt, stream))
-    return rc;
-  if (int rc = launch_transpose_rows(grad_out, g_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_out, ws.ld_t,
-                                     ws.a_t, ws.partial, stream))
-    return rc;
   if (int rc = launch_transpose_rows(in, in_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_in, ws.ld_t,
-                                     ws.b_t, nullptr, stream))
+                                     ws.b_t, nullptr, stream, nullptr))
     return rc;
   if (int rc = launch_bias_reduce(ws.partial, ws.k_seg, E, n_out, grad_b, stream)) return rc;
   return grouped_gemm_kseg(ws.a_t, ws.ld_t, ws.b_t, ws.ld_t, ws.k_seg, ws.row_off, E, n_out, n_in,
@@ -1496,7 +1460,7 @@ extern "C" int ccf_ffn2_backward(const void *grad_y_flat, const void *act, const
                                  ccf_stream_t stream) {
   using namespace ccf;
   if (max_rows == 0) return zero_param_grads(grad_w2, grad_b2, num_expert, d_model, d_ffn, as_stream(stream));
-  return linear_backward(static_cast<const half_t *>(grad_y_flat), dst_row,
+  return linear_backward(const_cast<half_t *>(static_cast<const half_t *>(grad_y_flat)), dst_row,
                          static_cast<const half_t *>(act), nullptr, offsets, max_rows, num_expert,
                          d_ffn, d_model, static_cast<const half_t *>(w2),
                          static_cast<half_t *>(grad_act), nullptr, static_cast<half_t *>(grad_w2),
@@ -1511,9 +1475,24 @@ extern "C" int ccf_ffn1_backward(const void *grad_h, const void *x, const int32_
                                  size_t workspace_bytes, ccf_stream_t stream) {
   using namespace ccf;
   if (max_rows == 0) return zero_param_grads(grad_w1, grad_b1, num_expert, d_ffn, d_model, as_stream(stream));
-  return linear_backward(static_cast<const half_t *>(grad_h), nullptr, static_cast<const half_t *>(x),
+  return linear_backward(const_cast<half_t *>(static_cast<const half_t *>(grad_h)), nullptr, static_cast<const half_t *>(x),
                          src_row, offsets, max_rows, num_expert, d_model, d_ffn,
                          static_cast<const half_t *>(w1), static_cast<half_t *>(grad_x_flat), dst_row,
                          static_cast<half_t *>(grad_w1), static_cast<half_t *>(grad_b1), workspace,
                          workspace_bytes, d_model, d_ffn, as_stream(stream), "ffn1_backward");
+}
+
+extern "C" int ccf_ffn1_backward_gelu(void *grad_act, const void *h_pre, const void *x, const int32_t *src_row,
+                                      const int32_t *dst_row, const int32_t *offsets, int max_rows,
+                                      int num_expert, int d_model, int d_ffn, const void *w1,
+                                      void *grad_x_flat, void *grad_w1, void *grad_b1, void *workspace,
+                                      size_t workspace_bytes, ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(h_pre && aligned16(h_pre), CCF_ERR_ARG, "ffn1_backward_gelu: the pre-activation is missing or unaligned");
+  if (max_rows == 0) return zero_param_grads(grad_w1, grad_b1, num_expert, d_ffn, d_model, as_stream(stream));
+  return linear_backward(static_cast<half_t *>(grad_act), nullptr, static_cast<const half_t *>(x), src_row, offsets,
+                         max_rows, num_expert, d_model, d_ffn, static_cast<const half_t *>(w1),
+                         static_cast<half_t *>(grad_x_flat), dst_row, static_cast<half_t *>(grad_w1),
+                         static_cast<half_t *>(grad_b1), workspace, workspace_bytes, d_model, d_ffn, as_stream(stream),
+                         "ffn1_backward_gelu", nullptr, static_cast<const half_t *>(h_pre));
 }

@@ -125,10 +125,11 @@ class MixMOEFusedFFN(Function):
     The reference keeps the activation a separate torch op between its two functions
     (mix_moe/mix_moe/transformer.py:82-91) so that autograd differentiates it; here the
     first GEMM's epilogue applies the GELU and also stores the pre-activation, so the
-    forward has no activation pass.  The backward applies GELU' with torch's elementwise
-    kernel: the input-gradient GEMM can multiply by it in its epilogue
-    (``ops.ffn2_backward(h_pre=...)``), but that epilogue runs with the matrix pipe idle
-    and measures slower (config 3: +0.21 ms against 0.14 ms for the separate pass)."""
+    forward has no activation pass.  In the backward GELU' is applied by the pass that
+    transposes the gradient rows for the first layer's weight gradient
+    (``ops.ffn1_backward(h_pre=...)``), in place.  The input-gradient GEMM of the second
+    layer can multiply by it in its epilogue too (``ops.ffn2_backward(h_pre=...)``), but
+    that epilogue runs with the matrix pipe idle and measures slower (config 3: +0.21 ms)."""
 
     @staticmethod
     def forward(ctx, input_buf, pos, moe_inp_block_infos, w1, b1, w2, b2):
@@ -152,10 +153,10 @@ class MixMOEFusedFFN(Function):
         grad_w2, grad_b2 = _param_grads(w2, E)
         grad_act, _, _ = ops.ffn2_backward(grad_y.contiguous(), act, dst_row, offsets, max_rows,
                                            w2.detach()[:E], grad_w2[:E], grad_b2[:E], may_drop=may_drop)
-        grad_h = torch.ops.aten.gelu_backward(grad_act, h_pre)
         grad_w1, grad_b1 = _param_grads(w1, E)
-        g_flat, _, _ = ops.ffn1_backward(grad_h, input_buf, src_row, dst_row, offsets, max_rows,
-                                         w1.detach()[:E], n_flat, grad_w1[:E], grad_b1[:E], may_drop=may_drop)
+        g_flat, _, _ = ops.ffn1_backward(grad_act, input_buf, src_row, dst_row, offsets, max_rows,
+                                         w1.detach()[:E], n_flat, grad_w1[:E], grad_b1[:E], may_drop=may_drop,
+                                         h_pre=h_pre)
         top_k = n_flat // input_buf.shape[0]
         ones = torch.ones(n_flat, dtype=g_flat.dtype, device=g_flat.device)
         grad_in = ops.combine(g_flat, ones, top_k, inv_pos)

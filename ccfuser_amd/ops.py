@@ -427,11 +427,17 @@ def ffn1_backward(grad_h: torch.Tensor, x: torch.Tensor, src_row: Optional[torch
                   dst_row: Optional[torch.Tensor], offsets: torch.Tensor, max_rows: int,
                   w1: torch.Tensor, n_flat: int,
                   grad_w: Optional[torch.Tensor] = None, grad_b: Optional[torch.Tensor] = None,
-                  may_drop: bool = True):
+                  may_drop: bool = True, h_pre: Optional[torch.Tensor] = None):
     """(grad_x_flat [n_flat, d], grad_w1 [E, f, d], grad_b1 [E, f]) of ``ffn1`` without the
     fused GELU.  ``grad_x_flat[dst_row[j]]`` is the gradient of sorted row j; rows nothing
-    maps to are zero (``may_drop=False`` promises every row is written)."""
+    maps to are zero (``may_drop=False`` promises every row is written).  With ``h_pre`` (from
+    ``ffn1_keep``) ``grad_h`` is the gradient of ``gelu(h_pre)`` on entry and is overwritten
+    with the gradient of ``h_pre``: the backward through the GELU and the linear layer."""
     _check(grad_h, "grad_h", dtype=torch.float16, ndim=2)
+    if h_pre is not None:
+        _check(h_pre, "h_pre", dtype=torch.float16, ndim=2)
+        if h_pre.shape != grad_h.shape:
+            raise ValueError("ffn1_backward: h_pre and grad_h differ in shape")
     _check(x, "x", dtype=torch.float16, ndim=2)
     _check(w1, "ffn1 weight", dtype=torch.float16, ndim=3)
     _check(offsets, "offsets", dtype=torch.int32, ndim=1)
@@ -452,9 +458,14 @@ def ffn1_backward(grad_h: torch.Tensor, x: torch.Tensor, src_row: Optional[torch
     g_w, g_b = _grad_outputs(w1, grad_w, grad_b)
     with torch.cuda.device(dev):
         ws = _backward_ws(max_rows, E, d, f, x)
-        _lib.call("ccf_ffn1_backward", _ptr(grad_h), _ptr(x), _ptr(src_row), _ptr(dst_row), _ptr(offsets),
-                  int(max_rows), E, d, f, _ptr(w1), _ptr(g_x), _ptr(g_w), _ptr(g_b), _ptr(ws),
-                  ws.numel(), _stream(x))
+        if h_pre is not None:
+            _lib.call("ccf_ffn1_backward_gelu", _ptr(grad_h), _ptr(h_pre), _ptr(x), _ptr(src_row), _ptr(dst_row),
+                      _ptr(offsets), int(max_rows), E, d, f, _ptr(w1), _ptr(g_x), _ptr(g_w), _ptr(g_b), _ptr(ws),
+                      ws.numel(), _stream(x))
+        else:
+            _lib.call("ccf_ffn1_backward", _ptr(grad_h), _ptr(x), _ptr(src_row), _ptr(dst_row), _ptr(offsets),
+                      int(max_rows), E, d, f, _ptr(w1), _ptr(g_x), _ptr(g_w), _ptr(g_b), _ptr(ws),
+                      ws.numel(), _stream(x))
     return g_x, g_w, g_b
 
 

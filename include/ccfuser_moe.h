@@ -425,6 +425,24 @@ int ccf_ffn1_backward(const void *grad_h, const void *x, const int32_t *src_row,
                       void *grad_x_flat, void *grad_w1, void *grad_b1, void *workspace,
                       size_t workspace_bytes, ccf_stream_t stream);
 
+/*
+ * Backward of ccf_ffn1_forward_keep: through the erf GELU and the first linear layer in one
+ * call.  grad_act holds the gradient of act = gelu(h_pre) on entry; the call multiplies it by
+ * gelu'(h_pre) in place (in the pass that also transposes it for the weight gradient), so on
+ * return it holds the gradient of the pre-activation, and everything else is ccf_ffn1_backward
+ * on that.  The reference leaves this product to autograd's GeluBackward between
+ * MixMOELinear2.backward and MixMOELinear1.backward (mix_moe/mix_moe/transformer.py:88,
+ * mix_moe/mix_moe/linear.py:91-113); mix_moe/csrc/mix_moe.h:300-388 is the rest.
+ *   grad_act    fp16 [max_rows, d_ffn]  in/out, expert order
+ *   h_pre       fp16 [max_rows, d_ffn]  from ccf_ffn1_forward_keep
+ *   the other arguments as in ccf_ffn1_backward
+ */
+int ccf_ffn1_backward_gelu(void *grad_act, const void *h_pre, const void *x, const int32_t *src_row,
+                           const int32_t *dst_row, const int32_t *offsets, int max_rows,
+                           int num_expert, int d_model, int d_ffn, const void *w1,
+                           void *grad_x_flat, void *grad_w1, void *grad_b1, void *workspace,
+                           size_t workspace_bytes, ccf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

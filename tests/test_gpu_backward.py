@@ -149,6 +149,18 @@ def _ffn_backward_stages(T, d, f, E, k, cap, skew, seed):
     _close(gin, gin_ref, "grad_in")
     _close(gw1, gw1_ref, "grad_w1")
     _close(gb1, gb1_ref, "grad_b1")
+    # the same through the GELU in one call: grad_act in, multiplied by gelu'(h_pre) in place
+    ga_in = torch.zeros(n, f, dtype=torch.float16)
+    ga_in[:R] = ga_ref.half()
+    gh_want = O.gelu_backward(ga_ref.half(), hp16)                  # what the call must leave in grad_act
+    gin_ref2, gw1_ref2, gb1_ref2 = O.ffn1_backward(gh_want.half(), p["x"], pos, k, offsets, p["w1"])
+    ga_dev = ga_in.cuda()
+    gx2, gw1_2, gb1_2 = ops.ffn1_backward(ga_dev, p["x"].cuda(), rt["src_row"], rt["dst_row"], rt["offsets"], n,
+                                          p["w1"].cuda(), n, h_pre=hp_pad.cuda())
+    _close(ga_dev[:R], gh_want, "grad_h left in place")
+    _close(ops.combine(gx2, ones, k, rt["inv_pos"]), gin_ref2, "grad_in through the GELU")
+    _close(gw1_2, gw1_ref2, "grad_w1 through the GELU")
+    _close(gb1_2, gb1_ref2, "grad_b1 through the GELU")
 
 
 @pytest.mark.parametrize("T,d,f,E,k,cf,seed", [
