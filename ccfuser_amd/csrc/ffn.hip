@@ -426,7 +426,7 @@ __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, in
   using C = SkinnyCfg;
   static_assert(C::STAGES * C::STAGE_BYTES <= 5 * 32768, "the stages share the ring's LDS");
   const int T = p.skinny[0], per_x = p.skinny[2];
-  const int4v *list = reinterpret_cast<const int4v *>(p.skinny + 4);
+  const int4v *list = reinterpret_cast<const int4v *>(p.skinny + kSkinnyHead);
   const int tid = fresh_tid(), lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int KT = p.K / C::BK;
@@ -483,17 +483,18 @@ __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, in
 // The skinny list as a launch of its own (plan.h): workgroup w of W takes K steps [w q, (w + 1) q) of the sequence
 // "tile 0's K steps, tile 1's, ..." and leaves one raw fp32 partial tile per list entry it touches, in fragment order
 // (block (tm, tn) of thread t at float4 index (4 tm + tn) * 256 + t), in its slots w * kSkTailSegs + 0, 1, ...
-__device__ __forceinline__ void skinny_tail_role(const GroupedArgs &p, int w, lds_char *lds, uint32_t lds_base) {
+// `inside`: called by the persistent launch (1) or by the launch behind it (0); the plan says which of them runs it.
+__device__ __forceinline__ void skinny_tail_role(const GroupedArgs &p, int w, int inside, lds_char *lds, uint32_t lds_base) {
   using C = SkinnyCfg;
   if (!p.skinny) return;
   const int T = p.skinny[0], q = p.skinny[3];
-  if (T <= 0 || q <= 0) return;
+  if (T <= 0 || q <= 0 || p.skinny[4] != inside) return;
   const int KT = p.K / C::BK;
   const int total = T * KT;
   const int s0 = w * q;
   if (s0 >= total) return;
   const int s1 = s0 + q < total ? s0 + q : total;
-  const int4v *list = reinterpret_cast<const int4v *>(p.skinny + 4);
+  const int4v *list = reinterpret_cast<const int4v *>(p.skinny + kSkinnyHead);
   const int tid = fresh_tid();
   uint32_t a_off[2], b_off[2];
   skinny_frag_offsets(tid, a_off, b_off);
@@ -511,6 +512,7 @@ __device__ __forceinline__ void skinny_tail_role(const GroupedArgs &p, int w, ld
       for (int tn = 0; tn < C::TN; ++tn) out[(tm * C::TN + tn) * 256] = acc[tm][tn];
   }
   wait_vmcnt<0>();
+  block_barrier();                                   // every wavefront is done with LDS before a caller's next tile loads
 }
 
 // Row block tm (16 rows) of skinny tile t: the sum of its partial tiles in K order, then the epilogue.
@@ -520,7 +522,7 @@ __device__ __forceinline__ void skinny_reduce_block(const GroupedArgs &p, int t,
   using C = SkinnyCfg;
   const int q = p.skinny[3];
   const int KT = p.K / C::BK;
-  const int4v ent = reinterpret_cast<const int4v *>(p.skinny + 4)[t];
+  const int4v ent = reinterpret_cast<const int4v *>(p.skinny + kSkinnyHead)[t];
   const int e = ent[0], row0 = ent[1], rows = ent[2], n0 = ent[3] * C::BN;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = tm * 16 + (lane & 15);
@@ -603,9 +605,23 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       }
     }
   }
-  if (slot_j >= slots_per_xcd) return;
-  int4v ent = plan[slot_j * 8 + xcd];
-  if (ent[0] < 0) return;                             // the used slots of an XCD are a prefix
+  // Skinny tiles cut along K inside this launch (plan.h): every workgroup takes its range of their K steps,
+  // half of the workgroups before their 256-row tiles and half behind them, so that at any time at most
+  // half of the chip streams weights for skinny tiles while the other half computes.  Groups of four
+  // consecutive slots (the M tiles of one N tile, which share their weight tiles) stay together.
+  constexpr bool kSkInside = !kSeg && !kKN && kEpi <= kEpiGeluKeep && Cfg::NW == 4;
+  const bool sk_first = ((slot_j >> 2) & 1) == 0;
+  if constexpr (kSkInside) {
+    if (sk_first) skinny_tail_role(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+  }
+  int4v ent = int4v{-1, 0, 0, 0};
+  if (slot_j < slots_per_xcd) ent = plan[slot_j * 8 + xcd];
+  if (ent[0] < 0) {                                   // no 256-row tile for this workgroup (the used slots of an XCD are a prefix)
+    if constexpr (kSkInside) {
+      if (!sk_first) skinny_tail_role(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+    }
+    return;
+  }
   // Plan entries are read through uniform indices (scalar loads, which do not queue behind the
   // epilogue's stores) and one tile ahead of their use: `ahead` is the entry after the next one.
   auto entry_at = [&](int j) {
@@ -731,6 +747,9 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   wait_vmcnt<0>();
+  if constexpr (kSkInside) {
+    if (!sk_first) skinny_tail_role(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+  }
 }
 
 
@@ -759,7 +778,7 @@ __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_tail_kernel(GroupedArgs p, int split_wgs) {
   using R = RingFor<Cfg, kKN>;
   if (static_cast<int>(blockIdx.x) >= split_wgs) {
-    if constexpr (!kKN) skinny_tail_role(p, static_cast<int>(blockIdx.x) - split_wgs, R::lds(), R::lds_addr());
+    if constexpr (!kKN) skinny_tail_role(p, static_cast<int>(blockIdx.x) - split_wgs, 0, R::lds(), R::lds_addr());
     return;
   }
   const int bmul = kKN ? p.N : 1;                      // elements between K rows of a [K][N] B
@@ -1287,8 +1306,8 @@ extern "C" int ccf_set_option(const char *name, int value) {
   if (!strcmp(name, "skinny")) {             // 0: off; 1: default; n > 1: cost of a skinny K step in percent (plan model);
                                              // -n: always, with n workgroups per XCD; -(kSkinnyMaxWgs + 1): always, as a
                                              // launch of their own
-    CCF_REQUIRE(value >= -kSkinnyMaxWgs - 1 && value <= 400, CCF_ERR_ARG, "set_option: skinny %d outside %d..400", value,
-                -kSkinnyMaxWgs - 1);
+    CCF_REQUIRE(value >= -kSkinnyMaxWgs - 2 && value <= 400, CCF_ERR_ARG, "set_option: skinny %d outside %d..400", value,
+                -kSkinnyMaxWgs - 2);
     g_skinny_pct = value == 1 ? 70 : value;
     return CCF_OK;
   }
@@ -1423,11 +1442,14 @@ extern "C" int ccf_ffn_plan_info(const void *workspace, int max_rows, int num_ex
   hipStream_t st = as_stream(stream);
   hipError_t e = hipSuccess;
   if (gs.split) e = hipMemcpyAsync(info, gs.tail, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, st);
+  int32_t where = 0;
   if (gs.skinny && e == hipSuccess) e = hipMemcpyAsync(info + 2, gs.skinny_list, 4 * sizeof(int32_t), hipMemcpyDeviceToHost, st);
+  if (gs.skinny && e == hipSuccess) e = hipMemcpyAsync(&where, gs.skinny_list + 4, sizeof(int32_t), hipMemcpyDeviceToHost, st);
   if (e == hipSuccess) e = hipStreamSynchronize(st);
   if (e != hipSuccess) return fail(CCF_ERR_HIP, "ffn_plan_info: %s", hipGetErrorString(e));
   info[6] = gs.grid;
   info[7] = static_cast<int32_t>(gs.wgs < (1ll << 31) ? gs.wgs : -1);
+  if (where == 1) info[5] = -info[5];                 // cut along K inside the persistent launch
   return CCF_OK;
 }
 

@@ -64,13 +64,16 @@ constexpr size_t kTailBytes = kTailHead + kSplitPartialBytes + kSkTailBytes;
 //
 // Layout of the list (int32):
 //   [0] tiles T   [1] ns   [2] tiles per XCD (XCD x owns entries [x * [2], (x + 1) * [2]))
-//   [3] q > 0: the tiles run as a launch of their own, q K steps per workgroup; 0 otherwise
-//   [4 + 4 i ...] entry i < T: {expert, first sorted row, rows (1..kSkinnyRows), N tile}
+//   [3] q > 0: the tiles are cut along K, q K steps per workgroup; 0 otherwise
+//   [4] with q > 0: 0 = as a launch of their own, 1 = inside the persistent launch (each of its
+//       workgroups runs its range before or behind its 256-row tiles)     [5..7] unused
+//   [kSkinnyHead + 4 i ...] entry i < T: {expert, first sorted row, rows (1..kSkinnyRows), N tile}
 constexpr int kSkinnyRows = 64;
 constexpr int kSkinnyMaxWgs = 4;                     // per XCD
+constexpr int kSkinnyHead = 8;                       // header integers in front of the entries
 __host__ __device__ inline size_t skinny_ints(int max_rows, int E, int n_tiles_n) {
   const int most = E < max_rows ? E : max_rows;      // at most one skinny M tile per expert
-  return 4 + 4 * static_cast<size_t>(most > 0 ? most : 0) * n_tiles_n;
+  return kSkinnyHead + 4 * static_cast<size_t>(most > 0 ? most : 0) * n_tiles_n;
 }
 
 // Time, in K steps of a 256-row tile, that F tiles of k_tiles K steps and an epilogue worth
@@ -88,7 +91,7 @@ __device__ inline int rounds_cost(int F, int spx, int k_tiles, int epi, bool may
       S = S > k_tiles / 4 ? k_tiles / 4 : S;
       S = (S >= 2 && 8 * r * S <= 256) ? S : 0;
     }
-    cost += S ? k_tiles / S + 16 : k_tiles + epi;    // 16: two more launches, pipeline fill, the reduction
+    cost += S ? k_tiles / S + 28 : k_tiles + epi;    // 28: two more launches, pipeline fill, the reduction (measured)
   }
   return cost;
 }
@@ -132,14 +135,19 @@ struct PlanReq {
   int epi_cost;     // the epilogue of a 256-row tile, in K steps
   int skinny_pct;   // a K step of a skinny tile in percent of a K step of a 256-row tile; 0 = never use skinny
                     // tiles; -n (n <= kSkinnyMaxWgs) = always, with n workgroups per XCD; -(kSkinnyMaxWgs + 1) =
-                    // always as a launch of their own (needs `tail`)
+                    // always cut along K as a launch of their own, -(kSkinnyMaxWgs + 2) = always cut along K inside
+                    // the persistent launch (both need `tail`)
   int sk_tail_ok;   // the skinny tiles may run as a launch of their own (the caller launches the kernels for it)
   int sk_beside_ok; // they may run in workgroups of the persistent launch (its four-wavefront form only)
 };
 
 // A K step of a skinny tile, in percent of a 256-row tile's, when the whole chip runs skinny tiles
 // and HBM bandwidth bounds them; and the fixed cost of that launch and its reduction, in K steps.
-constexpr int kSkTailStepPct = 90, kSkTailFixed = 16;
+// (Measured on 4096 x 4096 x 14336 layers, 80 and 280 skinny tiles, 70 K steps per workgroup: ~100 K steps'
+// worth of time for the launch of its own with its reduction, ~80 inside the persistent launch.)
+constexpr int kSkTailStepPct = 115, kSkTailFixed = 16;
+// The same when the ranges run inside the persistent launch, half of the chip at a time beside 256-row tiles.
+constexpr int kSkInsideStepPct = 105, kSkInsideFixed = 8;
 
 // Most tiles a range of q consecutive K steps can touch when a tile has k_tiles steps.
 __host__ __device__ inline int sk_tail_segments(int q, int k_tiles) { return (q - 1 + k_tiles - 1) / k_tiles + 1; }
@@ -168,11 +176,12 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   }
   __syncthreads();
   __shared__ int s_ns;             // workgroups per XCD given to skinny tiles (0: none)
-  __shared__ int s_tail_q;         // > 0: skinny tiles as a launch of their own, K steps per workgroup
+  __shared__ int s_tail_q;         // > 0: skinny tiles cut along K, K steps per workgroup
+  __shared__ int s_tail_inside;    // 1: inside the persistent launch, 0: as a launch of their own
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
     // Skinny tiles or not: tile counts both ways, then the cheaper plan by the model above.
-    int ns_wgs = 0, tail_q = 0;
+    int ns_wgs = 0, tail_q = 0, tail_inside = 0;
     if (skinny && rq.skinny_pct != 0 && rq.cus >= 64) {
       int nl0 = 0, nl1 = 0, nk1 = 0;                // 256-row tiles without / with skinny tiles, skinny M tiles
       for (int e = lane; e < E; e += 64) {
@@ -201,6 +210,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       }
       if (nk1 > 0 && rq.skinny_pct < -kSkinnyMaxWgs) {
         tail_q = q_c;                                  // forced (tests, measurements); 0 = not possible: no skinny tiles
+        tail_inside = rq.skinny_pct == -kSkinnyMaxWgs - 2 && rq.sk_beside_ok;
       } else if (nk1 > 0 && rq.skinny_pct < 0) {
         ns_wgs = rq.sk_beside_ok ? -rq.skinny_pct : 0; // forced
       } else if (nk1 > 0) {
@@ -218,11 +228,16 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
         if (q_c > 0) {
           const int c = rounds_cost(F1, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts) +
                         (q_c * kSkTailStepPct + 99) / 100 + kSkTailFixed;
-          if (c < best) { best = c; ns_wgs = 0; tail_q = q_c; }
+          if (c < best) { best = c; ns_wgs = 0; tail_q = q_c; tail_inside = 0; }
+          if (rq.sk_beside_ok) {
+            const int ci = rounds_cost(F1, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts) +
+                           (q_c * kSkInsideStepPct + 99) / 100 + kSkInsideFixed;
+            if (ci < best) { best = ci; ns_wgs = 0; tail_q = q_c; tail_inside = 1; }
+          }
         }
       }
     }
-    if (lane == 0) { s_ns = ns_wgs; s_tail_q = tail_q; }
+    if (lane == 0) { s_ns = ns_wgs; s_tail_q = tail_q; s_tail_inside = tail_inside; }
     int carry_l = 0, carry_s = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
@@ -273,6 +288,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     skinny[1] = ns_wgs;
     skinny[2] = (T + 7) / 8;
     skinny[3] = s_tail_q;
+    skinny[4] = s_tail_inside;
   }
   const int per_long = (total_long + 7) / 8;
   const int per_short = (total_short + 7) / 8;
@@ -361,7 +377,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       place(logical % per_long, logical / per_long, int4v{e, lo + first_row, rows, tn});   // hardware id = slot * 8 + XCD
     }
     if (ns && use_skinny) {
-      int4v *sk = reinterpret_cast<int4v *>(skinny + 4);
+      int4v *sk = reinterpret_cast<int4v *>(skinny + kSkinnyHead);
       const int first_s = s_short[e] * n_tiles_n;
       for (int tn = lane; tn < n_tiles_n; tn += 64) sk[first_s + tn] = int4v{e, lo + cnt_long, cnt - cnt_long, tn};
     } else if (ns) {

@@ -67,7 +67,9 @@ const char *ccf_last_error(void);
  *                     cost model says that beats a padded 256-row tile; n > 1 sets the model's cost of
  *                     such a tile's K step in percent of a 256-row tile's (default 70); -n (1..4) forces
  *                     them with n workgroups per XCD; -5 forces them as a launch of their own behind the
- *                     persistent kernel, cut along K over all workgroups (the model's third choice)
+ *                     persistent kernel, cut along K over all workgroups (the model's third choice); -6 forces
+ *                     them cut along K inside the persistent launch, each workgroup running its range before
+ *                     or behind its 256-row tiles (the fourth)
  *   "skinny_tail"     0/1 (default 1): the plan may choose that third way
  *   "fused_combine"   0/1 (default 0): ccf_moe_forward with top_k = 2 adds the gate-weighted expert outputs
  *                     into the output in the second GEMM's epilogue (packed fp16 atomic adds onto zeros)
@@ -248,7 +250,8 @@ size_t ccf_ffn_workspace_bytes(int max_rows, int num_expert, int d_model, int d_
  * integers to the host and synchronises the stream.  info (host, 8 ints):
  *   [0] tiles of the split last round, [1] parts each is cut into (0 = not split)
  *   [2] skinny tiles, [3] workgroups per XCD that run them beside the 256-row tiles,
- *   [4] skinny tiles per XCD, [5] K steps per workgroup when they run as a launch of their own (0 = not)
+ *   [4] skinny tiles per XCD, [5] K steps per workgroup when they are cut along K: > 0 as a launch of their
+ *       own, < 0 inside the persistent launch, 0 = not cut
  *   [6] workgroups of the persistent launch (0 = one workgroup per tile), [7] worst-case tile count
  */
 int ccf_ffn_plan_info(const void *workspace, int max_rows, int num_expert, int d_model, int d_ffn,

@@ -564,12 +564,15 @@ def test_split_k_tail_all_epilogues():
     (15360, 1088, 832, 60, False, 36, -4, "12"),      # N no multiple of 256 in either GEMM (832, 1088)
     (8192, 4096, 4096, 6, False, 37, -5, "12"),       # as a launch of their own, cut along K: a workgroup's range inside one tile
     (0, 1536, 4160, 40, False, 38, -5, "12"),         # experts of 17..64 rows only: ranges of four tiles, N = 4160
+    (8192, 4096, 4096, 6, False, 39, -6, "12"),       # cut along K inside the persistent launch, before / behind the 256-row tiles
+    (0, 1536, 4160, 40, False, 40, -6, "12"),         # the same where most workgroups have no 256-row tile at all
+    (20000, 2048, 2048, 12, False, 41, -6, "12"),     # several 256-row tiles per workgroup in front of / behind the ranges
 ])
 def test_skinny_tiles(R, d, f, E, skew, seed, mode, expect):
     """Rows beyond an expert's full 256-row tiles (at most 64) run as 64-row tiles: in workgroups
     the plan sets aside beside the 256-row tiles (mode -n: forced, n workgroups per XCD) or as a
-    launch of their own cut along K (mode -5: forced); mode 1 leaves the choice to the plan's
-    cost model.  All three forward epilogues with that path on and off, each against fp32.
+    launch of their own cut along K (mode -5: forced) or cut along K inside the persistent launch
+    (mode -6: forced); mode 1 leaves the choice to the plan's cost model.  All three forward epilogues with that path on and off, each against fp32.
     Beside the 256-row tiles the path adds over K in the same order as they do and must agree
     bit for bit; cut along K it agrees within rounding.  The plan must report that skinny tiles
     really ran where the case is built for them."""
@@ -594,7 +597,7 @@ def test_skinny_tiles(R, d, f, E, skew, seed, mode, expect):
         ops.set_option("skinny", m)
         # beside the 256-row tiles: keep those unsplit, the comparison is about the skinny path;
         # a launch of their own needs the split kernels launched (every K tile count allowed)
-        ops.set_option("split_tail", 2 if mode == -5 else 0)
+        ops.set_option("split_tail", 2 if mode <= -5 else 0)
         try:
             h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True, workspace=ws)
             info[m, 1] = ops.ffn_plan_info(ws, R, E, d, f, 1)
@@ -611,10 +614,12 @@ def test_skinny_tiles(R, d, f, E, skew, seed, mode, expect):
     _say(f"  plan, second GEMM: {info[mode, 2]}")
     for which in (1, 2):
         i = info[mode, which]
-        ran = i["skinny_tiles"] > 0 and (i["skinny_wgs_per_xcd"] > 0 or i["skinny_tail_steps"] > 0)
+        ran = i["skinny_tiles"] > 0 and (i["skinny_wgs_per_xcd"] > 0 or i["skinny_tail_steps"] != 0)
         if str(which) in expect:
             assert ran, (which, i)
-            assert (i["skinny_tail_steps"] > 0) == (mode == -5) and (i["skinny_wgs_per_xcd"] == -mode or mode == -5), i
+            # steps > 0: as a launch of their own; < 0: inside the persistent launch
+            assert (i["skinny_tail_steps"] > 0) == (mode == -5) and (i["skinny_tail_steps"] < 0) == (mode == -6), i
+            assert i["skinny_wgs_per_xcd"] == (-mode if mode > -5 else 0), i
         if mode < 0:
             assert info[0, which]["skinny_tiles"] == 0
     buf = x[pos].float()
@@ -637,7 +642,7 @@ def test_skinny_tiles(R, d, f, E, skew, seed, mode, expect):
         assert O.max_abs_err(y, y_ref) <= MAX_ABS and O.mean_rel_err(y, y_ref) <= MEAN_REL, m
     same = [torch.equal(a, b) for a, b in zip(res[mode], res[0])]
     _say(f"  skinny on/off bitwise equal (h, act, pre, y): {same}")
-    if mode == -5:
+    if mode <= -5:
         # another summation order: close, and not identical where skinny tiles ran
         for a, b in zip(res[mode], res[0]):
             assert O.max_abs_err(a, b.float()) <= MAX_ABS
