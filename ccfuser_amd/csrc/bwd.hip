@@ -37,9 +37,13 @@ constexpr int kPadK = 256;            // shortest K range the persistent GEMM ta
 __global__ void __launch_bounds__(1024)
 kseg_kernel(const int32_t *__restrict__ offsets, int E, int max_rows, int seg_rows, int n_blk,
             int32_t *__restrict__ k_seg, int32_t *__restrict__ row_off,
-            int32_t *__restrict__ blk_row0, int32_t *__restrict__ blk_cnt) {
+            int32_t *__restrict__ blk_row0, int32_t *__restrict__ blk_cnt, int32_t *__restrict__ row_lo,
+            half_t *__restrict__ zero_row) {
   __shared__ int s_k[1025];
   const int t = threadIdx.x;
+  // for the weight-gradient GEMM on row-major operands: the experts' row ranges, never past max_rows, and a row of zeros
+  if (row_lo && t <= E) row_lo[t] = offsets[t] < max_rows ? offsets[t] : max_rows;
+  if (zero_row && t < 256) zero_row[t] = static_cast<half_t>(0.0f);
   int lo = 0, cnt = 0;
   if (t < E) {
     lo = offsets[t] < max_rows ? offsets[t] : max_rows;
@@ -110,7 +114,9 @@ transpose_weights_kernel(const half_t *__restrict__ in, half_t *__restrict__ out
 // sum over the block's rows of column c, in row order, fp32.
 // kGelu: the rows are gradients of gelu(pre) (same layout, no row index): they are multiplied by
 // gelu'(pre), written back in place, and what is transposed and summed is the product.
-template <bool kGelu>
+// kT false: nothing is transposed; the (gathered) rows go to out_t as a row-major [rows, C] matrix in sorted
+// row order (out_t NULL: nowhere), and the pass is a row gather and / or the partial sums.
+template <bool kGelu, bool kT>
 __global__ void __launch_bounds__(256)
 transpose_rows_kernel(half_t *in, const int32_t *__restrict__ rows,
                       const int32_t *__restrict__ blk_row0, const int32_t *__restrict__ blk_cnt,
@@ -136,19 +142,26 @@ transpose_rows_kernel(half_t *in, const int32_t *__restrict__ rows,
           v[j] = static_cast<half_t>(static_cast<float>(v[j]) * gelu_erf_grad(static_cast<float>(p[j])));
         *reinterpret_cast<half8 *>(in + r * C + c0 + ch * 8) = v;
       }
+      if constexpr (!kT) {
+        if (out_t) *reinterpret_cast<half8 *>(out_t + static_cast<size_t>(row0 + i) * C + c0 + ch * 8) = v;
+      }
     }
+    if (kT || partial) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) tile[i][ch * 8 + j] = v[j];
+      for (int j = 0; j < 8; ++j) tile[i][ch * 8 + j] = v[j];
+    }
   }
   __syncthreads();
+  if constexpr (kT) {
 #pragma unroll
-  for (int it = 0; it < 2; ++it) {
-    const int q = threadIdx.x + it * 256;
-    const int c = q >> 3, ch = q & 7;
-    half8 v;
+    for (int it = 0; it < 2; ++it) {
+      const int q = threadIdx.x + it * 256;
+      const int c = q >> 3, ch = q & 7;
+      half8 v;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = tile[ch * 8 + j][c];
-    *reinterpret_cast<half8 *>(out_t + static_cast<size_t>(c0 + c) * ld_t + static_cast<size_t>(b) * kTile + ch * 8) = v;
+      for (int j = 0; j < 8; ++j) v[j] = tile[ch * 8 + j][c];
+      *reinterpret_cast<half8 *>(out_t + static_cast<size_t>(c0 + c) * ld_t + static_cast<size_t>(b) * kTile + ch * 8) = v;
+    }
   }
   if (partial && threadIdx.x < kTile) {
     float s = 0.0f;
@@ -229,9 +242,10 @@ int padded_rows(int max_rows, int E) {
 }
 
 int launch_kseg(const int32_t *offsets, int E, int max_rows, int seg_rows, int n_blk, int32_t *k_seg,
-                int32_t *row_off, int32_t *blk_row0, int32_t *blk_cnt, hipStream_t stream) {
+                int32_t *row_off, int32_t *blk_row0, int32_t *blk_cnt, int32_t *row_lo, half_t *zero_row,
+                hipStream_t stream) {
   hipLaunchKernelGGL(kseg_kernel, dim3(1), dim3(1024), 0, stream, offsets, E, max_rows, seg_rows,
-                     n_blk, k_seg, row_off, blk_row0, blk_cnt);
+                     n_blk, k_seg, row_off, blk_row0, blk_cnt, row_lo, zero_row);
   return check_launch("kseg_kernel");
 }
 
@@ -243,14 +257,22 @@ int launch_transpose_weights(const half_t *in, half_t *out, int E, int R, int C,
 
 int launch_transpose_rows(const half_t *in, const int32_t *rows, const int32_t *blk_row0,
                           const int32_t *blk_cnt, int n_blk, int C, int ld_t, half_t *out_t,
-                          float *partial, hipStream_t stream, const half_t *gelu_pre_inplace) {
+                          float *partial, hipStream_t stream, const half_t *gelu_pre_inplace, bool transposed) {
   half_t *src = const_cast<half_t *>(in);             // written only in the GELU form
-  if (gelu_pre_inplace)
-    hipLaunchKernelGGL(transpose_rows_kernel<true>, dim3(n_blk, C / kTile), dim3(256), 0, stream, src, rows,
-                       blk_row0, blk_cnt, C, ld_t, out_t, partial, gelu_pre_inplace);
+  const dim3 grid(n_blk, C / kTile);
+  const half_t *none = nullptr;
+  if (gelu_pre_inplace && transposed)
+    hipLaunchKernelGGL((transpose_rows_kernel<true, true>), grid, dim3(256), 0, stream, src, rows, blk_row0, blk_cnt, C, ld_t,
+                       out_t, partial, gelu_pre_inplace);
+  else if (gelu_pre_inplace)
+    hipLaunchKernelGGL((transpose_rows_kernel<true, false>), grid, dim3(256), 0, stream, src, rows, blk_row0, blk_cnt, C, ld_t,
+                       out_t, partial, gelu_pre_inplace);
+  else if (transposed)
+    hipLaunchKernelGGL((transpose_rows_kernel<false, true>), grid, dim3(256), 0, stream, src, rows, blk_row0, blk_cnt, C, ld_t,
+                       out_t, partial, none);
   else
-    hipLaunchKernelGGL(transpose_rows_kernel<false>, dim3(n_blk, C / kTile), dim3(256), 0, stream, src, rows,
-                       blk_row0, blk_cnt, C, ld_t, out_t, partial, static_cast<const half_t *>(nullptr));
+    hipLaunchKernelGGL((transpose_rows_kernel<false, false>), grid, dim3(256), 0, stream, src, rows, blk_row0, blk_cnt, C, ld_t,
+                       out_t, partial, none);
   return check_launch("transpose_rows_kernel");
 }
 

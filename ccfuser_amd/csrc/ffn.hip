@@ -25,15 +25,21 @@ namespace {
 
 // The main loop of a tile shape: eight wavefronts (two per SIMD, half the registers each) keep one
 // register buffer of token fragments, four wavefronts two.
-template <class Cfg, bool kKN>
-using RingFor = Ring16Mainloop<Cfg, kKN, Cfg::NW == 8>;
+template <class Cfg, bool kKN, bool kRows = false>
+using RingFor = Ring16Mainloop<Cfg, kKN, Cfg::NW == 8, kRows>;
 
 // ---- tile plan ---------------------------------------------------------------
 // build_plan() (plan.h) in a launch of its own; the layer's forward call lets the routing
 // stage build both of its plans instead.
-__global__ void __launch_bounds__(1024)
+// Several workgroups share the work (build_plan's `part`): enough that every expert has a wavefront, at most 8.
+constexpr int kPlanThreads = 256;
+__global__ void __launch_bounds__(kPlanThreads)
 plan_kernel(PlanReq rq, const int32_t *__restrict__ offsets, int E) {
-  build_plan(rq, offsets, E);
+  build_plan(rq, offsets, E, blockIdx.x, gridDim.x);
+}
+inline int plan_workgroups(int E) {
+  const int w = (E + kPlanThreads / 64 - 1) / (kPlanThreads / 64);
+  return w > 8 ? 8 : (w < 1 ? 1 : w);
 }
 
 // ---- grouped GEMM kernel -------------------------------------------------------
@@ -58,6 +64,10 @@ struct GroupedArgs {
   // split last round (layout in plan.h): header and part entries, fp32 partial tiles
   const int32_t *tail;
   float *partial;
+  // rows form (weight gradients without transposed copies): A [rows, lda] and B [rows, ldb] are row-major
+  // activation matrices in expert order, the contraction of expert e runs over rows k_seg[e] .. k_seg[e+1]
+  // (any number, also none), and rows past the end are fetched from this row of 256 zeros
+  const half_t *zero_row;
   // skinny list (layout in plan.h) of this GEMM, or NULL
   const int32_t *skinny;
   float *sk_partial;        // partial tiles of the skinny tiles when they run as a launch of their own
@@ -152,15 +162,45 @@ __device__ __forceinline__ int2v scalar_load2(const int32_t *q) {
 }
 
 // K tiles of expert e's contraction.
-template <class Cfg, bool kSeg>
+template <class Cfg, bool kSeg, bool kRows = false>
 __device__ __forceinline__ int k_tiles_of(const GroupedArgs &p, int e) {
-  if constexpr (kSeg) {
+  if constexpr (kRows) {
+    // rows form: the expert's rows in K tiles, the last one partly masked; never fewer than the pipeline needs
+    const int eu = __builtin_amdgcn_readfirstlane(e);
+    const int2v r = scalar_load2(p.k_seg + eu);
+    const int kt = (r[1] - r[0] + Cfg::BK - 1) / Cfg::BK;
+    return kt < 4 ? 4 : kt;
+  } else if constexpr (kSeg) {
     const int eu = __builtin_amdgcn_readfirstlane(e);
     const int2v r = scalar_load2(p.k_seg + eu);
     return (r[1] - r[0]) / Cfg::BK;
   } else {
     return p.K / Cfg::BK;
   }
+}
+
+// Rows form: sources of the tile loads of both operands for the tile {expert e, first output row row0, N tile},
+// and the K mask (the expert's row count seen from this lane's first K row).
+template <class Cfg>
+__device__ __forceinline__ void rows_sources(const GroupedArgs &p, int e, int row0, int tile_n, const half_t *(&a_src)[2],
+                                             const half_t *(&b_src)[2], typename RingFor<Cfg, true, true>::KMask &mk) {
+  using R = RingFor<Cfg, true, true>;
+  const int eu = __builtin_amdgcn_readfirstlane(e);
+  const int2v seg = scalar_load2(p.k_seg + eu);
+  const int m0 = row0 - eu * p.seg_rows, n0 = tile_n * Cfg::BN;
+  const int tid = fresh_tid();
+  const int unit = R::kn_dma_unit(tid);
+  const half_t *Ae = p.A + static_cast<size_t>(seg[0]) * p.lda + m0;
+  const half_t *Be = p.B + static_cast<size_t>(seg[0]) * p.ldb + n0;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {                           // loads 0 and 1; load i >= 2 is 16 rows below load i - 2
+    const int r = R::kn_dma_row(i, tid);
+    const int col = R::kn_col(r, unit);
+    a_src[i] = Ae + static_cast<size_t>(r) * p.lda + col;
+    b_src[i] = Be + static_cast<size_t>(r) * p.ldb + col;
+  }
+  mk.klim = seg[1] - seg[0] - R::kn_dma_row(0, tid);
+  mk.zero = p.zero_row + unit * 8;
 }
 
 // x, y: this lane's four columns of two neighbouring 16-column blocks.  Lanes 16 apart swap
@@ -587,8 +627,10 @@ template <class Cfg, int kEpi, bool kSeg = false, bool kKN = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   using ML = GemmMainloop<Cfg>;
-  using R = RingFor<Cfg, kKN>;
-  const int bmul = kKN ? p.N : 1;                     // elements between K rows of a [K][N] B
+  constexpr bool kRows = kSeg && kKN;                 // both operands row-major with the contraction over rows
+  using R = RingFor<Cfg, kKN, kRows>;
+  const int bmul = kRows ? p.ldb : (kKN ? p.N : 1);   // elements between K rows of a [K][N] B
+  const int amul = kRows ? p.lda : 1;                 // and of a [K][M] A
   constexpr int TM = R::TM, TN = R::TN;
   const int4v *plan = reinterpret_cast<const int4v *>(p.plan);
   const int xcd = blockIdx.x & 7;
@@ -631,13 +673,15 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   };
   int4v ahead = entry_at(slot_j + stride);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const half_t *a_src[Cfg::A_DMA];
+  const half_t *a_src[R::A_SRCS];
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
-  tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
+  typename R::KMask mk{0, nullptr};
+  if constexpr (kRows) rows_sources<Cfg>(p, ent[0], ent[1], ent[3], a_src, b_src, mk);
+  else tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
   int a_off[2], b_off[2];
   R::frag_offsets(a_off, b_off);
   half8 fa[R::AB][TM], fb[2][TN];
-  R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg>(p, ent[0]), a_off, b_off, wave, bmul);
+  R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg, kRows>(p, ent[0]), a_off, b_off, wave, bmul, amul, mk);
   R::reserve();
   int phase = 0;
 
@@ -648,12 +692,12 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
     const int4v nent = has_next ? ahead : ent;
     ahead = has_next ? entry_at(nj + stride) : ahead;  // used by the next tile: its latency hides under this one
     const int n_row0 = nent[1], n_rows = nent[2];
-    const int KT = k_tiles_of<Cfg, kSeg>(p, ent[0]);
+    const int KT = k_tiles_of<Cfg, kSeg, kRows>(p, ent[0]);
     const int k_end = KT * Cfg::BK;
 
     R::zero_acc();
 
-    int next_row[Cfg::A_DMA];                         // A row of the next tile per tile load
+    int next_row[kRows ? 1 : Cfg::A_DMA];             // A row of the next tile per tile load
     if constexpr (!kSeg) {
       const int tid0 = fresh_tid();
 #pragma unroll
@@ -672,14 +716,22 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
     // The eight-wavefront form runs the MFMAs of padded row blocks too (they repeat real rows and are not
     // stored): with half the registers, the branch around each row block makes the compiler park values in
     // accumulation registers, which this kernel owns.
-    const int live_m = Cfg::NW == 8 ? TM : R::live_blocks(ent[2]);
+    const int live_m = (Cfg::NW == 8 || kRows) ? TM : R::live_blocks(ent[2]);   // rows form: the tile's rows are weight rows, all real
     R::acc_settle();
     if (live_m == TM) {
-      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m, bmul);
+      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m, bmul,
+                                amul, mk);
     } else {
-      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m, bmul);
+      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, KT - 2, 2 * Cfg::BK, k_end, phase, wave, live_m, bmul,
+                                 amul, mk);
     }
-    {
+    if constexpr (kRows) {
+      // sources and K mask of the next tile
+      int n_e = __builtin_amdgcn_readfirstlane(nent[0]), n_r0 = __builtin_amdgcn_readfirstlane(nent[1]),
+          n_tn = __builtin_amdgcn_readfirstlane(nent[3]);
+      asm volatile("" : "+s"(n_e), "+s"(n_r0), "+s"(n_tn));
+      rows_sources<Cfg>(p, n_e, n_r0, n_tn, a_src, b_src, mk);
+    } else {
       // sources of the next tile (tile_sources() with the row indices already at hand); the
       // empty asm keeps the compiler from computing them before the loop above and holding
       // 16 more registers across it
@@ -734,9 +786,9 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       }
     }
     if (live_m == TM) {
-      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul);
+      R::template k_range<true>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul, amul, mk);
     } else {
-      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul);
+      R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul, amul, mk);
     }
     R::acc_settle();
     epilogue16<Cfg, kEpi, kSeg>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
@@ -900,6 +952,7 @@ constexpr int kWideMaxKT = 0;        // forward GEMMs with at most this many K t
 constexpr int kDefaultVariant = 0;
 int g_variant = kDefaultVariant;
 int g_dgrad_transpose = 0;   // 1: input gradients always on a transposed copy of the weight
+int g_wgrad_transpose = 0;   // 1: weight gradients always on transposed copies of the activations
 int g_split_tail = 1;        // 0: the last round of tiles is not cut along K
 constexpr int kSplitTailMinKT = 64;
 int g_split_tail_min_kt = kSplitTailMinKT;
@@ -1080,7 +1133,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   const long long wgs = gs.wgs;
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
   if (!plan_ready) {
-    hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream, gs.req, offsets, E);
+    hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream, gs.req, offsets, E);
     if (int rc = check_launch("plan_kernel")) return rc;
   }
   int32_t *plan = gs.plan, *tail = gs.tail;
@@ -1104,6 +1157,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.tail = tail;
   p.partial = partial;
   p.sk_partial = gs.sk_partial;
+  p.zero_row = nullptr;
   p.skinny = gs.skinny ? gs.skinny_list : nullptr;
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;                // wgs is a multiple of 8
@@ -1144,7 +1198,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const int n_tiles_n = (N + Cfg5::BN - 1) / Cfg5::BN;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
-  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, stream,
+  hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream,
                      PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0, 0, 0}, row_off, E);
   if (int rc = check_launch("plan_kernel")) return rc;
   GroupedArgs p;
@@ -1167,6 +1221,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   p.tail = nullptr;
   p.partial = nullptr;
   p.sk_partial = nullptr;
+  p.zero_row = nullptr;
   p.skinny = nullptr;
   const int grid = persistent_grid();
   if (grid >= 8) {
@@ -1180,11 +1235,60 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   return check_launch(what);
 }
 
+// C[e*M + m, n] = sum over the rows j of expert e (row_lo[e] <= j < row_lo[e+1]) of A[j, m] * B[j, n]: the weight
+// gradient of expert e straight from the two row-major activation matrices (no transposed copies): both
+// operands go through LDS as [K][*] tiles and transposing reads, rows past an expert's end read as zero.
+// M and N multiples of 256; row_off[e] = e*M.
+int grouped_gemm_krows(const half_t *A, int lda, const half_t *B, int ldb, const int32_t *row_lo,
+                       const int32_t *row_off, int E, int M, int N, half_t *C, int32_t *workspace,
+                       const half_t *zero_row, int grid, hipStream_t stream, const char *what) {
+  CCF_REQUIRE(A && B && row_lo && row_off && C && workspace && zero_row, CCF_ERR_ARG, "%s: null pointer", what);
+  int32_t *plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(workspace) + kTailBytes);
+  CCF_REQUIRE(lda % 8 == 0 && ldb % 8 == 0 && M % Cfg5::BM == 0 && N % Cfg5::BN == 0 && grid >= 8, CCF_ERR_SHAPE,
+              "%s: the row-major weight-gradient form needs widths that are multiples of 256", what);
+  CCF_REQUIRE(static_cast<long long>(E) * M < (1ll << 31), CCF_ERR_SHAPE, "%s: output too tall", what);
+  const int max_rows = E * M;
+  const int max_tiles = max_tiles_for(max_rows, E, Cfg5::BM);
+  const int n_tiles_n = N / Cfg5::BN;
+  const long long wgs = launched_wgs(max_tiles, n_tiles_n);
+  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
+  hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream,
+                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0, 0, 0}, row_off, E);
+  if (int rc = check_launch("plan_kernel")) return rc;
+  GroupedArgs p;
+  p.A = A;
+  p.a_rows = nullptr;
+  p.B = B;
+  p.bias = nullptr;
+  p.C = C;
+  p.C2 = nullptr;
+  p.c_rows = nullptr;
+  p.row_scale = nullptr;
+  p.scale_rows = nullptr;
+  p.plan = plan;
+  p.N = N;
+  p.K = 0;
+  p.k_seg = row_lo;
+  p.lda = lda;
+  p.ldb = ldb;
+  p.seg_rows = M;
+  p.tail = nullptr;
+  p.partial = nullptr;
+  p.sk_partial = nullptr;
+  p.zero_row = zero_row;
+  p.skinny = nullptr;
+  const long long g = grid < wgs ? grid : wgs;
+  hipLaunchKernelGGL((grouped_gemm_persistent_kernel<Cfg5, kEpiPlain, true, true>), dim3(static_cast<unsigned>(g)),
+                     dim3(Cfg5::THREADS), 0, stream, p, static_cast<int>(wgs / 8));
+  return check_launch(what);
+}
+
 // Workspace of the backward entry points, carved in this order.
 struct BackwardWs {
   int32_t *plan_rows;      // tile plan of the input-gradient GEMM
   int32_t *plan_w;         // tile plan of the weight-gradient GEMM
-  int32_t *k_seg, *row_off, *blk_row0, *blk_cnt;
+  int32_t *k_seg, *row_off, *blk_row0, *blk_cnt, *row_lo;
+  half_t *zero_row;        // 256 zeros
   half_t *w_t;             // [E, in, out] transposed weight
   half_t *a_t, *b_t;       // [out, ld_t], [in, ld_t] transposed activations
   float *partial;          // [ld_t / 64, out] bias partial sums
@@ -1210,6 +1314,8 @@ BackwardWs carve_backward(void *base, int max_rows, int E, int d, int f) {
   w.row_off = static_cast<int32_t *>(take(sizeof(int32_t) * (E + 1)));
   w.blk_row0 = static_cast<int32_t *>(take(sizeof(int32_t) * w.n_blk));
   w.blk_cnt = static_cast<int32_t *>(take(sizeof(int32_t) * w.n_blk));
+  w.row_lo = static_cast<int32_t *>(take(sizeof(int32_t) * (E + 1)));
+  w.zero_row = static_cast<half_t *>(take(sizeof(half_t) * 256));
   w.w_t = static_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(E) * d * f));
   w.a_t = static_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(big) * w.ld_t));
   w.b_t = static_cast<half_t *>(take(sizeof(half_t) * static_cast<size_t>(big) * w.ld_t));
@@ -1250,16 +1356,25 @@ int linear_backward(half_t *grad_out, const int32_t *g_rows, const half_t *in,
   CCF_REQUIRE(workspace && workspace_bytes >= need, CCF_ERR_WORKSPACE,
               "%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);
   const BackwardWs ws = carve_backward(workspace, max_rows, E, d, f);
-  // K ranges of the weight-gradient GEMM, then the transposed copy of the gradient rows (with the bias
-  // gradient's partial sums).  With pre_inplace the incoming rows are gradients of gelu(pre): the same
-  // pass multiplies them by gelu'(pre) and writes them back, so that everything below sees the
-  // gradient of the pre-activation.
+  // The weight gradient contracts over an expert's rows.  Where the widths allow, its GEMM reads the two
+  // row-major activation matrices as they are (rows form: transposing LDS reads of both operands); what
+  // remains of the data movement is a gather of the operand that arrives through a row index, and one pass
+  // over the gradient rows for the bias gradient's partial sums.  Otherwise both matrices are transposed
+  // into [columns, padded rows] first.
+  const int grid = persistent_grid();
+  const int wide = n_out > n_in ? n_out : n_in;
+  const bool rows_form = !g_wgrad_transpose && n_out % Cfg5::BM == 0 && n_in % Cfg5::BN == 0 && grid >= 8 &&
+                         static_cast<long long>(max_rows + 256) * wide < (1ll << 31);
+  // With pre_inplace the incoming rows are gradients of gelu(pre): the pass over them multiplies them by
+  // gelu'(pre) and writes them back, so that everything below sees the gradient of the pre-activation.
   CCF_REQUIRE(!pre_inplace || !g_rows, CCF_ERR_ARG, "%s: the in-place GELU gradient needs rows in expert order", what);
   if (int rc = launch_kseg(offsets, E, max_rows, n_out, ws.n_blk, ws.k_seg, ws.row_off, ws.blk_row0,
-                           ws.blk_cnt, stream))
+                           ws.blk_cnt, ws.row_lo, ws.zero_row, stream))
     return rc;
+  // rows form: gathered gradient rows go to a_t as a plain [rows, n_out] matrix; rows already in expert order stay
+  const half_t *g_mat = (rows_form && !g_rows) ? grad_out : ws.a_t;
   if (int rc = launch_transpose_rows(grad_out, g_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_out, ws.ld_t,
-                                     ws.a_t, ws.partial, stream, pre_inplace))
+                                     (rows_form && !g_rows) ? nullptr : ws.a_t, ws.partial, stream, pre_inplace, !rows_form))
     return rc;
   // input gradient: on the stored weight read as [K][N] where the shape allows, else on a transposed copy
   const bool kn = !g_dgrad_transpose && n_in % Cfg5::BN == 0 && static_cast<long long>(n_out) * n_in < (1ll << 31);
@@ -1273,10 +1388,16 @@ int linear_backward(half_t *grad_out, const int32_t *g_rows, const half_t *in,
                             what, kn, const_cast<half_t *>(gelu_pre)))
     return rc;
   // weight and bias gradients
-  if (int rc = launch_transpose_rows(in, in_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_in, ws.ld_t,
-                                     ws.b_t, nullptr, stream, nullptr))
-    return rc;
+  const half_t *in_mat = (rows_form && !in_rows) ? in : ws.b_t;
+  if (!rows_form || in_rows) {
+    if (int rc = launch_transpose_rows(in, in_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_in, ws.ld_t,
+                                       ws.b_t, nullptr, stream, nullptr, !rows_form))
+      return rc;
+  }
   if (int rc = launch_bias_reduce(ws.partial, ws.k_seg, E, n_out, grad_b, stream)) return rc;
+  if (rows_form)
+    return grouped_gemm_krows(g_mat, n_out, in_mat, n_in, ws.row_lo, ws.row_off, E, n_out, n_in, grad_w, ws.plan_w,
+                              ws.zero_row, grid, stream, what);
   return grouped_gemm_kseg(ws.a_t, ws.ld_t, ws.b_t, ws.ld_t, ws.k_seg, ws.row_off, E, n_out, n_in,
                            grad_w, ws.plan_w, stream, what);
 }
@@ -1317,6 +1438,10 @@ extern "C" int ccf_set_option(const char *name, int value) {
   }
   if (!strcmp(name, "dgrad_transpose")) {
     g_dgrad_transpose = value != 0;
+    return CCF_OK;
+  }
+  if (!strcmp(name, "wgrad_transpose")) {
+    g_wgrad_transpose = value != 0;
     return CCF_OK;
   }
   if (!strcmp(name, "gate_waves")) {

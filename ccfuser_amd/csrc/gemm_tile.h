@@ -221,10 +221,24 @@ struct GemmMainloop {
 // leave during the substep before their use, so the ring schedule above is unchanged; what
 // changes is that a row block's new fragment has one substep less one row block of lead
 // instead of a whole substep, which the second wavefront of the SIMD covers.
-template <class Cfg, bool B_KN = false, bool ROLL_A = false>
+//
+// A_KM (with B_KN): the A operand is stored [K][M] as well, read through the same transposing
+// reads, and K rows at or past a per-lane limit are fetched from a row of zeros instead (KMask):
+// the form of a weight gradient, whose contraction runs over an expert's rows of two row-major
+// activation matrices, any number of rows.
+template <class Cfg, bool B_KN = false, bool ROLL_A = false, bool A_KM = false>
 struct Ring16Mainloop {
   using acc_t = float4v;
   static constexpr int AB = ROLL_A ? 1 : 2;                      // register buffers of the token fragments
+  static_assert(!A_KM || (B_KN && !ROLL_A && Cfg::WTM == 128 && Cfg::A_DMA % 2 == 0 && Cfg::BM == Cfg::BN),
+                "the [K][M] form of A mirrors the [K][N] form of B");
+  static constexpr int A_SRCS = A_KM ? 2 : Cfg::A_DMA;
+  // Tile load l of a [K][*] operand fetches K row 8 l + own (own < 8 fixed per lane) of the K tile; with
+  // klim = (rows of the contraction) - own, that row exists while (first K row of the tile) + 8 l < klim.
+  struct KMask {
+    int klim;
+    const half_t *zero;        // this lane's 16 bytes of a row of zeros
+  };
   static constexpr int KN_PITCH = Cfg::BN * 2;                   // bytes per K row of a [K][N] half tile
   // Source pointers a lane holds for its B tile loads.  [N][K]: one per load.  [K][N]: load i
   // fetches K row 8*i + r0 (r0 < 8 fixed per lane), whose chunk XOR depends on i%2 only, so
@@ -280,11 +294,19 @@ struct Ring16Mainloop {
       return src[l] + k_elem;
     }
   }
+  // The same with the K mask of the A_KM form: krow = first K row of the tile being loaded.
+  template <bool KN2, int N>
+  static __device__ __forceinline__ const half_t *load_src_m(const half_t *const (&src)[N], int l, int k_elem, int mul,
+                                                             int krow, const KMask &mk) {
+    const half_t *p = load_src<KN2>(src, l, k_elem, mul);
+    if constexpr (A_KM) p = (krow + 8 * l < mk.klim) ? p : mk.zero;
+    return p;
+  }
   template <bool KN2, int NLOAD, int N>
   static __device__ __forceinline__ void issue_all(const half_t *const (&src)[N], int k_elem, int slot_off, int wave,
-                                                   int bmul = 1) {
+                                                   int bmul = 1, int krow = 0, const KMask &mk = KMask{0, nullptr}) {
     static_for<0, NLOAD>([&](auto I) {
-      lds_dma16(load_src<KN2>(src, I.value, k_elem, bmul), lds() + slot_off + (I.value * Cfg::NW + wave) * 1024);
+      lds_dma16(load_src_m<KN2>(src, I.value, k_elem, bmul, krow, mk), lds() + slot_off + (I.value * Cfg::NW + wave) * 1024);
     });
   }
 
@@ -301,6 +323,11 @@ struct Ring16Mainloop {
       } else {
         b[I] = lds_read_b128<I * 16 * Cfg::CPR * 16>(rb);
       }
+    } else if constexpr (A_KM) {
+      const uint32_t addr = ra ^ ((I - TN) * 32);
+      const half4 lo = lds_read_tr_b64<0>(addr);
+      const half4 hi = lds_read_tr_b64<4 * KN_PITCH>(addr);
+      a[I - TN] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     } else {
       a[I - TN] = lds_read_b128<(I - TN) * 16 * Cfg::CPR * 16>(ra);
     }
@@ -359,7 +386,8 @@ struct Ring16Mainloop {
   template <int SUB, int NLOAD, bool FULL, bool KN2 = false, int NSRC>
   static __device__ __forceinline__ void substep(half8 (&a)[AB][TM], half8 (&b)[2][TN],
                                                  const half_t *const (&src)[NSRC], int k_elem, uint32_t ra,
-                                                 uint32_t rb, int ws, int wave, int live_m, int bmul = 1) {
+                                                 uint32_t rb, int ws, int wave, int live_m, int bmul = 1, int krow = 0,
+                                                 const KMask &mk = KMask{0, nullptr}) {
     constexpr int AS = ROLL_A ? 0 : SUB, AN = ROLL_A ? 0 : SUB ^ 1;     // token fragment buffer in use / being filled
     // what goes out behind MFMA i
     auto behind = [&](auto II) {
@@ -373,7 +401,7 @@ struct Ring16Mainloop {
       }
       if constexpr (i % Cfg::DMA_EVERY == 1 && i / Cfg::DMA_EVERY < NLOAD) {
         constexpr int l = i / Cfg::DMA_EVERY;
-        lds_dma16(load_src<KN2>(src, l, k_elem, bmul), lds() + ws + (l * Cfg::NW + wave) * 1024);
+        lds_dma16(load_src_m<KN2>(src, l, k_elem, bmul, krow, mk), lds() + ws + (l * Cfg::NW + wave) * 1024);
       }
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -393,19 +421,21 @@ struct Ring16Mainloop {
   }
 
   // K tile kt in ring phase ph; k2 / kb2: element offset from the A / B sources of the K
-  // tile that the loads of this step fetch (A into the fifth slot, B into the slot A(kt) leaves).
+  // tile that the loads of this step fetch (A into the fifth slot, B into the slot A(kt) leaves);
+  // krow: that tile's first K row (for the K mask of the A_KM form).
   template <bool FULL>
   static __device__ __forceinline__ void step(half8 (&a)[AB][TM], half8 (&b)[2][TN],
-                                              const half_t *const (&a_src)[Cfg::A_DMA],
+                                              const half_t *const (&a_src)[A_SRCS],
                                               const half_t *const (&b_src)[B_SRCS], const int (&a_off)[2],
-                                              const int (&b_off)[2], int k2, int kb2, int ph, int wave, int live_m, int bmul) {
+                                              const int (&b_off)[2], int k2, int kb2, int ph, int wave, int live_m, int bmul,
+                                              int amul = 1, int krow = 0, const KMask &mk = KMask{0, nullptr}) {
     const Slots s = slots_of(ph);
     const uint32_t base = lds_addr();
     frags_ready(a[0], b[0]);
     __builtin_amdgcn_sched_barrier(0);
     // K half 0; fetch the fragments of K half 1 of this tile; load A(kt+2)
-    substep<0, Cfg::A_DMA, FULL>(a, b, a_src, k2, base + s.a + a_off[1], base + s.b + b_off[1], s.wa, wave,
-                                 live_m);
+    substep<0, Cfg::A_DMA, FULL, A_KM>(a, b, a_src, k2, base + s.a + a_off[1], base + s.b + b_off[1], s.wa, wave,
+                                       live_m, amul, krow, mk);
     // B(kt+1) and everything older have landed; A(kt+2) may stay in flight
     wait_vmcnt<Cfg::A_DMA>();
     block_barrier();
@@ -413,23 +443,25 @@ struct Ring16Mainloop {
     __builtin_amdgcn_sched_barrier(0);
     // K half 1; fetch the fragments of K half 0 of tile kt+1; load B(kt+2) into A(kt)'s slot
     substep<1, Cfg::B_DMA, FULL, B_KN>(a, b, b_src, kb2, base + s.na + a_off[0], base + s.nb + b_off[0], s.a, wave,
-                                       live_m, bmul);
+                                       live_m, bmul, krow, mk);
   }
 
   // `steps` consecutive K-tile steps starting in ring phase `phase` (updated).
-  // Step i loads the K tile at element offset min(k2_first + i*BK, k2_max); bmul: elements
-  // between consecutive K rows of a [K][N] B operand.
+  // Step i loads the K tile at element offset min(k2_first + i*BK, k2_max); bmul / amul: elements
+  // between consecutive K rows of a [K][N] B / [K][M] A operand.
   template <bool FULL>
   static __device__ __forceinline__ void k_range(half8 (&a)[AB][TM], half8 (&b)[2][TN],
-                                                 const half_t *const (&a_src)[Cfg::A_DMA],
+                                                 const half_t *const (&a_src)[A_SRCS],
                                                  const half_t *const (&b_src)[B_SRCS], const int (&a_off)[2],
                                                  const int (&b_off)[2], int steps, int k2_first, int k2_max,
-                                                 int &phase, int wave, int live_m, int bmul = 1) {
+                                                 int &phase, int wave, int live_m, int bmul = 1, int amul = 1,
+                                                 const KMask &mk = KMask{0, nullptr}) {
     int ph = phase;
     int k2 = k2_first;
     for (int i = 0; i < steps; ++i) {
       const int kc = k2 < k2_max ? k2 : k2_max;
-      step<FULL>(a, b, a_src, b_src, a_off, b_off, kc, B_KN ? kc * bmul : kc, ph, wave, live_m, bmul);
+      step<FULL>(a, b, a_src, b_src, a_off, b_off, A_KM ? kc * amul : kc, B_KN ? kc * bmul : kc, ph, wave, live_m, bmul,
+                 amul, kc, mk);
       k2 += Cfg::BK;
       ph = ph == NSLOT - 1 ? 0 : ph + 1;
     }
@@ -445,7 +477,13 @@ struct Ring16Mainloop {
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       const int c = sub * 4 + (lane >> 4);
-      a_off[sub] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
+      if constexpr (A_KM) {
+        const int j = lane & 15;
+        const int row = sub * 32 + 8 * (lane >> 4) + (j >> 2);
+        a_off[sub] = row * KN_PITCH + (wave / Cfg::WN) * (Cfg::WTM * 2) + (kn_swz(row) << 5) + ((j & 3) << 3);
+      } else {
+        a_off[sub] = (ra * Cfg::CPR + (c ^ swz<Cfg::CPR>(ra))) * 16;
+      }
       if constexpr (B_KN) {
         // source lane j of its group of 16 points at K row 8*group + j/4, columns 4*(j%4) ..
         const int j = lane & 15;
@@ -494,15 +532,15 @@ struct Ring16Mainloop {
   // Phase 0: A(0) -> slot 0, B(0) -> slot 1, A(1) -> slot 2, B(1) -> slot 3, then
   // the fragments of K half 0 of tile 0 into a[0], b[0].
   static __device__ __forceinline__ void prologue(half8 (&a)[AB][TM], half8 (&b)[2][TN],
-                                                  const half_t *const (&a_src)[Cfg::A_DMA],
+                                                  const half_t *const (&a_src)[A_SRCS],
                                                   const half_t *const (&b_src)[B_SRCS], int KT,
                                                   const int (&a_off)[2], const int (&b_off)[2], int wave,
-                                                  int bmul = 1) {
+                                                  int bmul = 1, int amul = 1, const KMask &mk = KMask{0, nullptr}) {
     const int k1 = (KT > 1 ? 1 : 0) * Cfg::BK;
-    issue_all<false, Cfg::A_DMA>(a_src, 0, 0 * SLOT_BYTES, wave);
-    issue_all<B_KN, Cfg::B_DMA>(b_src, 0, 1 * SLOT_BYTES, wave, bmul);
-    issue_all<false, Cfg::A_DMA>(a_src, k1, 2 * SLOT_BYTES, wave);
-    issue_all<B_KN, Cfg::B_DMA>(b_src, B_KN ? k1 * bmul : k1, 3 * SLOT_BYTES, wave, bmul);
+    issue_all<A_KM, Cfg::A_DMA>(a_src, 0, 0 * SLOT_BYTES, wave, amul, 0, mk);
+    issue_all<B_KN, Cfg::B_DMA>(b_src, 0, 1 * SLOT_BYTES, wave, bmul, 0, mk);
+    issue_all<A_KM, Cfg::A_DMA>(a_src, A_KM ? k1 * amul : k1, 2 * SLOT_BYTES, wave, amul, k1, mk);
+    issue_all<B_KN, Cfg::B_DMA>(b_src, B_KN ? k1 * bmul : k1, 3 * SLOT_BYTES, wave, bmul, k1, mk);
     wait_vmcnt<Cfg::A_DMA + Cfg::B_DMA>();
     block_barrier();
     const uint32_t ra = lds_addr() + a_off[0], rb = lds_addr() + SLOT_BYTES + b_off[0];
@@ -513,6 +551,7 @@ struct Ring16Mainloop {
   static __device__ __forceinline__ void run(const half_t *const (&a_src)[Cfg::A_DMA],
                                              const half_t *const (&b_src)[B_SRCS], int K, int rows,
                                              int bmul = 1) {
+    static_assert(!A_KM, "the [K][M] form runs in the persistent kernel only");
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int KT = K / Cfg::BK;
     const int live_m = live_blocks(rows);

@@ -82,6 +82,8 @@ const char *ccf_last_error(void);
  *                     of a workgroup by the same number (0 = chosen by the token count)
  *   "dgrad_transpose" 0/1: the backward's input-gradient GEMM runs on a transposed copy of the
  *                     weight instead of reading the stored one
+ *   "wgrad_transpose" 0/1: the backward's weight-gradient GEMM runs on transposed copies of the two
+ *                     activation matrices instead of reading them row-major
  *   "gate_waves"      1..8 (default 8): most wavefronts of a gate workgroup; each takes other parts of K
  */
 int ccf_set_option(const char *name, int value);

@@ -49,13 +49,16 @@ def _case(T, d, f, E, k, seed, skew=False):
 ])
 @pytest.mark.parametrize("transpose", [0, 1])
 def test_ffn_backward_stages(T, d, f, E, k, cap, skew, seed, transpose):
-    """transpose=0: input gradients read the stored weight as [K][N] where the width allows;
-    transpose=1: always on a transposed copy."""
+    """transpose=0: input gradients read the stored weight as [K][N], and weight gradients the
+    two activation matrices row-major, where the widths allow; transpose=1: always on transposed
+    copies."""
     from ccfuser_amd import ops
     ops.set_option("dgrad_transpose", transpose)
+    ops.set_option("wgrad_transpose", transpose)
     try:
         _ffn_backward_stages(T, d, f, E, k, cap, skew, seed)
     finally:
+        ops.set_option("wgrad_transpose", 0)
         ops.set_option("dgrad_transpose", 0)
 
 
