@@ -357,6 +357,9 @@ struct SkinnyCfg {
   static constexpr int LOADS = A_DMA + B_DMA;
 };
 
+// Layout of a [K][N] weight tile of 64 x 256 in LDS: the one the 256 x 256 main loop uses.
+using SkinnyKN = RingFor<GemmCfg<256, 256, 64, 2, 2, 8>, true>;
+
 // acc += w (16 weight rows) x t (16 token rows), K = 32, on ordinary registers
 __device__ __forceinline__ void mfma16_v(float4v &acc, const half8 &w, const half8 &t) {
   asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(t));
@@ -367,20 +370,32 @@ __device__ __forceinline__ void mfma16_v(float4v &acc, const half8 &w, const hal
 typedef float4v SkinnyAcc[SkinnyCfg::TM][SkinnyCfg::TN];
 
 // This lane's fragment chunk of row block 0, per K half (16x16x32 operand: row lane % 16, K chunk lane / 16).
+// kKN: the weight tile sits in LDS as [K][N] rows in the main loop's layout of such a tile (its column
+// blocks of 16 are XOR-swizzled inside each half of 128 columns; wavefront w reads blocks 4 (w % 2) .. + 3
+// of half w / 2 through transposing reads, block tn at the address XOR 32 tn).
+template <bool kKN>
 __device__ __forceinline__ void skinny_frag_offsets(int tid, uint32_t (&a_off)[2], uint32_t (&b_off)[2]) {
   using C = SkinnyCfg;
+  using KN = SkinnyKN;
   const int lane = tid & 63, wave = tid >> 6;
   const int ra = lane & 15, rb = wave * 64 + (lane & 15);
 #pragma unroll
   for (int sub = 0; sub < 2; ++sub) {
     const int c = sub * 4 + (lane >> 4);
     a_off[sub] = (ra * 8 + (c ^ swz<8>(ra))) * 16;
-    b_off[sub] = C::A_BYTES + (rb * 8 + (c ^ swz<8>(rb))) * 16;
+    if constexpr (kKN) {
+      const int j = lane & 15;
+      const int row = sub * 32 + 8 * (lane >> 4) + (j >> 2);
+      b_off[sub] = C::A_BYTES + row * KN::KN_PITCH + (wave >> 1) * 256 + ((KN::kn_swz(row) ^ ((wave & 1) * 4)) << 5) + ((j & 3) << 3);
+    } else {
+      b_off[sub] = C::A_BYTES + (rb * 8 + (c ^ swz<8>(rb))) * 16;
+    }
   }
 }
 
 // acc = the tile of list entry `ent` over K tiles [kt0, kt0 + nkt) (nkt >= 1), accumulated over K in 32-wide steps
-// in ascending order.  All four wavefronts of the workgroup call it together.
+// in ascending order.  All four wavefronts of the workgroup call it together.  kKN: the weights are [E, K, N].
+template <bool kKN>
 __device__ __forceinline__ void skinny_mainloop(const GroupedArgs &p, const int4v ent, int kt0, int nkt, SkinnyAcc &acc,
                                                 const uint32_t (&a_off)[2], const uint32_t (&b_off)[2], int tid,
                                                 lds_char *lds, uint32_t lds_base) {
@@ -392,7 +407,8 @@ __device__ __forceinline__ void skinny_mainloop(const GroupedArgs &p, const int4
   live_m = __builtin_amdgcn_readfirstlane(live_m > C::TM ? C::TM : live_m);
   // global source of every tile load of this lane, at K tile kt0
   const half_t *a_src[C::A_DMA], *b_src[C::B_DMA];
-  const half_t *Be = p.B + static_cast<size_t>(e) * p.N * p.K + static_cast<size_t>(kt0) * C::BK;
+  const half_t *Be = p.B + static_cast<size_t>(e) * p.N * p.K + static_cast<size_t>(kt0) * C::BK * (kKN ? p.N : 1);
+  const int bmul = kKN ? p.N : 1;                                  // elements between K rows of the weights
 #pragma unroll
   for (int j = 0; j < C::A_DMA; ++j) {
     const int r = (j * 4 + wave) * 8 + (lane >> 3);
@@ -402,9 +418,16 @@ __device__ __forceinline__ void skinny_mainloop(const GroupedArgs &p, const int4
   }
 #pragma unroll
   for (int j = 0; j < C::B_DMA; ++j) {
-    const int r = (j * 4 + wave) * 8 + (lane >> 3);
-    const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
-    b_src[j] = Be + static_cast<size_t>(n) * p.K + ((lane & 7) ^ swz<8>(r)) * 8;
+    if constexpr (kKN) {
+      // a load is two K rows of 256 columns (N % 256 == 0); which columns a 16-byte unit holds: the main loop's layout
+      using KN = SkinnyKN;
+      const int r = KN::kn_dma_row(j, tid);
+      b_src[j] = Be + static_cast<size_t>(r) * p.N + n0 + KN::kn_col(r, KN::kn_dma_unit(tid));
+    } else {
+      const int r = (j * 4 + wave) * 8 + (lane >> 3);
+      const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
+      b_src[j] = Be + static_cast<size_t>(n) * p.K + ((lane & 7) ^ swz<8>(r)) * 8;
+    }
   }
   auto issue = [&](int kt, int stage) {                            // K tile kt0 + kt into a stage
     const int k_elem = (kt < nkt ? kt : nkt - 1) * C::BK;          // past the end: the last tile again, into a stage nobody reads
@@ -412,7 +435,8 @@ __device__ __forceinline__ void skinny_mainloop(const GroupedArgs &p, const int4
 #pragma unroll
     for (int j = 0; j < C::A_DMA; ++j) lds_dma16(a_src[j] + k_elem, base + (j * 4 + wave) * 1024);
 #pragma unroll
-    for (int j = 0; j < C::B_DMA; ++j) lds_dma16(b_src[j] + k_elem, base + C::A_BYTES + (j * 4 + wave) * 1024);
+    for (int j = 0; j < C::B_DMA; ++j)
+      lds_dma16(b_src[j] + static_cast<size_t>(k_elem) * bmul, base + C::A_BYTES + (j * 4 + wave) * 1024);
   };
 #pragma unroll
   for (int tm = 0; tm < C::TM; ++tm)
@@ -434,7 +458,16 @@ __device__ __forceinline__ void skinny_mainloop(const GroupedArgs &p, const int4
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       half8 a[C::TM], b[C::TN];
-      static_for<0, C::TN>([&](auto J) { b[J.value] = lds_read_b128<J.value * 2048>(sb + b_off[sub]); });
+      static_for<0, C::TN>([&](auto J) {
+        if constexpr (kKN) {
+          const uint32_t addr = (sb + b_off[sub]) ^ (J.value * 32);
+          const half4 lo = lds_read_tr_b64<0>(addr);
+          const half4 hi = lds_read_tr_b64<4 * SkinnyKN::KN_PITCH>(addr);
+          b[J.value] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+          b[J.value] = lds_read_b128<J.value * 2048>(sb + b_off[sub]);
+        }
+      });
       static_for<0, C::TM>([&](auto I) { a[I.value] = lds_read_b128<I.value * 2048>(sb + a_off[sub]); });
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
@@ -460,7 +493,7 @@ __device__ __forceinline__ void skinny_mainloop(const GroupedArgs &p, const int4
     for (int tn = 0; tn < C::TN; ++tn) asm volatile("" : "+v"(acc[tm][tn]));
 }
 
-template <int kEpi>
+template <int kEpi, bool kKN>
 __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, int ns, int xcd, lds_char *lds,
                                             uint32_t lds_base) {
   using C = SkinnyCfg;
@@ -471,7 +504,7 @@ __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, in
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int KT = p.K / C::BK;
   uint32_t a_off[2], b_off[2];
-  skinny_frag_offsets(tid, a_off, b_off);
+  skinny_frag_offsets<kKN>(tid, a_off, b_off);
   for (int i = worker; i < per_x; i += ns) {
     const int w = xcd * per_x + i;
     if (w >= T) break;
@@ -480,7 +513,7 @@ __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, in
     int live_m = (rows + 15) / 16;
     live_m = __builtin_amdgcn_readfirstlane(live_m > C::TM ? C::TM : live_m);
     SkinnyAcc acc;
-    skinny_mainloop(p, ent, 0, KT, acc, a_off, b_off, tid, lds, lds_base);
+    skinny_mainloop<kKN>(p, ent, 0, KT, acc, a_off, b_off, tid, lds, lds_base);
     // epilogue: bias, GELU or row scale, fp16 through the row index; 8-byte stores
     const half_t *bias_e = p.bias + static_cast<size_t>(e) * p.N;
     const int colb = n0 + wave * 64 + 4 * (lane >> 4);             // column of block tn = colb + 16 tn
@@ -524,6 +557,7 @@ __device__ __forceinline__ void skinny_role(const GroupedArgs &p, int worker, in
 // "tile 0's K steps, tile 1's, ..." and leaves one raw fp32 partial tile per list entry it touches, in fragment order
 // (block (tm, tn) of thread t at float4 index (4 tm + tn) * 256 + t), in its slots w * kSkTailSegs + 0, 1, ...
 // `inside`: called by the persistent launch (1) or by the launch behind it (0); the plan says which of them runs it.
+template <bool kKN>
 __device__ __forceinline__ void skinny_tail_role(const GroupedArgs &p, int w, int inside, lds_char *lds, uint32_t lds_base) {
   using C = SkinnyCfg;
   if (!p.skinny) return;
@@ -537,13 +571,13 @@ __device__ __forceinline__ void skinny_tail_role(const GroupedArgs &p, int w, in
   const int4v *list = reinterpret_cast<const int4v *>(p.skinny + kSkinnyHead);
   const int tid = fresh_tid();
   uint32_t a_off[2], b_off[2];
-  skinny_frag_offsets(tid, a_off, b_off);
+  skinny_frag_offsets<kKN>(tid, a_off, b_off);
   int t = s0 / KT;
   for (int seg = 0; seg < kSkTailSegs && t * KT < s1; ++seg, ++t) {
     const int k0 = (s0 > t * KT ? s0 : t * KT) - t * KT;
     const int k1 = (s1 < (t + 1) * KT ? s1 : (t + 1) * KT) - t * KT;
     SkinnyAcc acc;
-    skinny_mainloop(p, list[t], k0, k1 - k0, acc, a_off, b_off, tid, lds, lds_base);
+    skinny_mainloop<kKN>(p, list[t], k0, k1 - k0, acc, a_off, b_off, tid, lds, lds_base);
     float4v *out = reinterpret_cast<float4v *>(p.sk_partial) +
                    static_cast<size_t>(w * kSkTailSegs + seg) * (C::TM * C::TN * 256) + tid;
 #pragma unroll
@@ -636,13 +670,13 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   const int xcd = blockIdx.x & 7;
   int stride = gridDim.x >> 3;
   int slot_j = blockIdx.x >> 3;
-  if constexpr (!kSeg && !kKN && kEpi <= kEpiGeluKeep && Cfg::NW == 4) {
+  if constexpr (!kSeg && kEpi <= kEpiGeluKeep && Cfg::NW == 4) {
     // the last ns workgroups of each XCD do the skinny tiles (if the plan has any), the others the 256-row tiles
     if (p.skinny) {
       const int ns = __builtin_amdgcn_readfirstlane(p.skinny[1]);
       stride -= ns;
       if (slot_j >= stride) {
-        skinny_role<kEpi>(p, slot_j - stride, ns, xcd, R::lds(), R::lds_addr());
+        skinny_role<kEpi, kKN>(p, slot_j - stride, ns, xcd, R::lds(), R::lds_addr());
         return;
       }
     }
@@ -651,16 +685,16 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   // half of the workgroups before their 256-row tiles and half behind them, so that at any time at most
   // half of the chip streams weights for skinny tiles while the other half computes.  Groups of four
   // consecutive slots (the M tiles of one N tile, which share their weight tiles) stay together.
-  constexpr bool kSkInside = !kSeg && !kKN && kEpi <= kEpiGeluKeep && Cfg::NW == 4;
+  constexpr bool kSkInside = !kSeg && kEpi <= kEpiGeluKeep && Cfg::NW == 4;
   const bool sk_first = ((slot_j >> 2) & 1) == 0;
   if constexpr (kSkInside) {
-    if (sk_first) skinny_tail_role(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+    if (sk_first) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
   }
   int4v ent = int4v{-1, 0, 0, 0};
   if (slot_j < slots_per_xcd) ent = plan[slot_j * 8 + xcd];
   if (ent[0] < 0) {                                   // no 256-row tile for this workgroup (the used slots of an XCD are a prefix)
     if constexpr (kSkInside) {
-      if (!sk_first) skinny_tail_role(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+      if (!sk_first) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
     }
     return;
   }
@@ -800,7 +834,7 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   wait_vmcnt<0>();
   if constexpr (kSkInside) {
-    if (!sk_first) skinny_tail_role(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+    if (!sk_first) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
   }
 }
 
@@ -830,7 +864,7 @@ __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD)
 grouped_gemm_tail_kernel(GroupedArgs p, int split_wgs) {
   using R = RingFor<Cfg, kKN>;
   if (static_cast<int>(blockIdx.x) >= split_wgs) {
-    if constexpr (!kKN) skinny_tail_role(p, static_cast<int>(blockIdx.x) - split_wgs, 0, R::lds(), R::lds_addr());
+    skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x) - split_wgs, 0, R::lds(), R::lds_addr());
     return;
   }
   const int bmul = kKN ? p.N : 1;                      // elements between K rows of a [K][N] B
@@ -1090,8 +1124,8 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
   // worth its two small launches only where a tile is long: K of 4096 and more)
   g.split = opt.split_tail && (b_kn ? epi == kEpiPlain : epi <= kEpiGeluKeep) && g.grid >= 8 && g.grid <= g.wgs &&
             g.grid <= kTailMaxParts && v.bm == Cfg5::BM && v.bn == Cfg5::BN && K / 64 >= opt.split_tail_min_kt;
-  // remainder rows as skinny tiles: forward epilogues of the persistent 256 x 256 kernel with the [N][K] weight
-  g.skinny = opt.skinny_pct != 0 && !b_kn && epi <= kEpiGeluKeep && g.grid >= 64 && g.grid <= g.wgs &&
+  // remainder rows as skinny tiles: forward epilogues of the persistent 256 x 256 kernel (either weight layout)
+  g.skinny = opt.skinny_pct != 0 && (b_kn ? epi == kEpiPlain && N % 256 == 0 : epi <= kEpiGeluKeep) && g.grid >= 64 && g.grid <= g.wgs &&
              v.bm == Cfg5::BM && v.bn == Cfg5::BN && v.persistent_plain && (!wide || g.split);
   g.skinny_list = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.plan) + plan_core_bytes(max_rows, E, N > K ? N : K));
   g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, opt.split_max_parts, g.plan,
@@ -1167,7 +1201,8 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
       if (int rc = check_launch(what)) return rc;
       // the skinny list may run as a launch of its own: `grid` more workgroups for it, more blocks in the reduction
       const bool sk = gs.req.sk_tail_ok;
-      if (b_kn) hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, true>), dim3(grid), dim3(Cfg5::THREADS), 0, stream, p, grid);
+      if (b_kn) hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, true>), dim3(sk ? 2 * grid : grid), dim3(Cfg5::THREADS), 0,
+                                   stream, p, grid);
       else hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, false>), dim3(sk ? 2 * grid : grid), dim3(Cfg5::THREADS), 0,
                               stream, p, grid);
       if (int rc = check_launch("grouped_gemm_tail_kernel")) return rc;
