@@ -22,6 +22,7 @@
 // The reference leaves grad_bias uninitialised (mix_moe.h:342, 488).
 #include "ccf_common.h"
 #include "gelu.h"
+#include "plan.h"
 
 namespace ccf {
 namespace {
@@ -38,7 +39,14 @@ __global__ void __launch_bounds__(1024)
 kseg_kernel(const int32_t *__restrict__ offsets, int E, int max_rows, int seg_rows, int n_blk,
             int32_t *__restrict__ k_seg, int32_t *__restrict__ row_off,
             int32_t *__restrict__ blk_row0, int32_t *__restrict__ blk_cnt, int32_t *__restrict__ row_lo,
-            half_t *__restrict__ zero_row) {
+            half_t *__restrict__ zero_row, PlanReq rows_plan, int rows_plan_wgs, PlanReq w_plan, int w_plan_wgs) {
+  // workgroups behind the first build the tile plans of the call's two GEMMs
+  if (blockIdx.x > 0) {
+    const int b = static_cast<int>(blockIdx.x) - 1;
+    if (b < rows_plan_wgs) build_plan(rows_plan, offsets, E, b, rows_plan_wgs);
+    else build_plan(w_plan, nullptr, E, b - rows_plan_wgs, w_plan_wgs, seg_rows);
+    return;
+  }
   __shared__ int s_k[1025];
   const int t = threadIdx.x;
   // for the weight-gradient GEMM on row-major operands: the experts' row ranges, never past max_rows, and a row of zeros
@@ -243,9 +251,13 @@ int padded_rows(int max_rows, int E) {
 
 int launch_kseg(const int32_t *offsets, int E, int max_rows, int seg_rows, int n_blk, int32_t *k_seg,
                 int32_t *row_off, int32_t *blk_row0, int32_t *blk_cnt, int32_t *row_lo, half_t *zero_row,
-                hipStream_t stream) {
-  hipLaunchKernelGGL(kseg_kernel, dim3(1), dim3(1024), 0, stream, offsets, E, max_rows, seg_rows,
-                     n_blk, k_seg, row_off, blk_row0, blk_cnt, row_lo, zero_row);
+                const PlanReq *rows_plan, const PlanReq *w_plan, hipStream_t stream) {
+  const int per_plan = (E + 15) / 16 > 8 ? 8 : (E + 15) / 16;     // a wavefront per expert, at most 8 workgroups
+  const int na = rows_plan ? per_plan : 0, nb = w_plan ? per_plan : 0;
+  const PlanReq none{};
+  hipLaunchKernelGGL(kseg_kernel, dim3(1 + na + nb), dim3(1024), 0, stream, offsets, E, max_rows, seg_rows,
+                     n_blk, k_seg, row_off, blk_row0, blk_cnt, row_lo, zero_row, rows_plan ? *rows_plan : none, na,
+                     w_plan ? *w_plan : none, nb);
   return check_launch("kseg_kernel");
 }
 

@@ -42,9 +42,6 @@ typedef int int4v __attribute__((ext_vector_type(4)));
 // bwd.hip: data movement of the backward pass
 int padded_rows(int max_rows, int E);
 int launch_zero(half_t *dst, size_t halves, hipStream_t stream);
-int launch_kseg(const int32_t *offsets, int E, int max_rows, int seg_rows, int n_blk, int32_t *k_seg,
-                int32_t *row_off, int32_t *blk_row0, int32_t *blk_cnt, int32_t *row_lo, half_t *zero_row,
-                hipStream_t stream);
 int launch_transpose_weights(const half_t *in, half_t *out, int E, int R, int C, hipStream_t stream);
 int launch_transpose_rows(const half_t *in, const int32_t *rows, const int32_t *blk_row0,
                           const int32_t *blk_cnt, int n_blk, int C, int ld_t, half_t *out_t,

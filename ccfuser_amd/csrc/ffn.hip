@@ -1219,11 +1219,21 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   return check_launch(what);
 }
 
+// Plan request of a weight-gradient GEMM: E experts of M output rows each, N columns; the plan sits behind the
+// (unused) split scratch in `workspace`.
+PlanReq wgrad_plan_request(int E, int M, int N, int32_t *workspace) {
+  int32_t *plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(workspace) + kTailBytes);
+  const int max_rows = E * M;
+  return PlanReq{Cfg5::BM, max_tiles_for(max_rows, E, Cfg5::BM), max_rows, (N + Cfg5::BN - 1) / Cfg5::BN, 0, 0, 0, plan,
+                 nullptr, nullptr, 0, 0, 0, 0, 0};
+}
+
 // C[e*M + m, n] = sum over k in [k_seg[e], k_seg[e+1]) of A[m, k] * B[n, k]: the weight
 // gradient of expert e from the two transposed activation matrices.  row_off[e] = e*M.
+// plan_ready: wgrad_plan_request()'s plan was already built in `workspace`.
 int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const int32_t *k_seg,
                       const int32_t *row_off, int E, int M, int N, half_t *C, int32_t *workspace,
-                      hipStream_t stream, const char *what) {
+                      hipStream_t stream, const char *what, bool plan_ready = false) {
   CCF_REQUIRE(A && B && k_seg && row_off && C && workspace, CCF_ERR_ARG, "%s: null pointer", what);
   int32_t *plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(workspace) + kTailBytes);
   CCF_REQUIRE(lda % 8 == 0 && ldb % 8 == 0 && N % 8 == 0, CCF_ERR_SHAPE, "%s: strides and N must be multiples of 8", what);
@@ -1233,9 +1243,11 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const int n_tiles_n = (N + Cfg5::BN - 1) / Cfg5::BN;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
-  hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream,
-                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0, 0, 0}, row_off, E);
-  if (int rc = check_launch("plan_kernel")) return rc;
+  if (!plan_ready) {
+    hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream,
+                       wgrad_plan_request(E, M, N, workspace), row_off, E);
+    if (int rc = check_launch("plan_kernel")) return rc;
+  }
   GroupedArgs p;
   p.A = A;
   p.a_rows = nullptr;
@@ -1276,7 +1288,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
 // M and N multiples of 256; row_off[e] = e*M.
 int grouped_gemm_krows(const half_t *A, int lda, const half_t *B, int ldb, const int32_t *row_lo,
                        const int32_t *row_off, int E, int M, int N, half_t *C, int32_t *workspace,
-                       const half_t *zero_row, int grid, hipStream_t stream, const char *what) {
+                       const half_t *zero_row, int grid, hipStream_t stream, const char *what, bool plan_ready = false) {
   CCF_REQUIRE(A && B && row_lo && row_off && C && workspace && zero_row, CCF_ERR_ARG, "%s: null pointer", what);
   int32_t *plan = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(workspace) + kTailBytes);
   CCF_REQUIRE(lda % 8 == 0 && ldb % 8 == 0 && M % Cfg5::BM == 0 && N % Cfg5::BN == 0 && grid >= 8, CCF_ERR_SHAPE,
@@ -1287,9 +1299,11 @@ int grouped_gemm_krows(const half_t *A, int lda, const half_t *B, int ldb, const
   const int n_tiles_n = N / Cfg5::BN;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
   CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
-  hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream,
-                     PlanReq{Cfg5::BM, max_tiles, max_rows, n_tiles_n, 0, 0, 0, plan, nullptr, nullptr, 0, 0, 0, 0, 0}, row_off, E);
-  if (int rc = check_launch("plan_kernel")) return rc;
+  if (!plan_ready) {
+    hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream,
+                       wgrad_plan_request(E, M, N, workspace), row_off, E);
+    if (int rc = check_launch("plan_kernel")) return rc;
+  }
   GroupedArgs p;
   p.A = A;
   p.a_rows = nullptr;
@@ -1403,24 +1417,30 @@ int linear_backward(half_t *grad_out, const int32_t *g_rows, const half_t *in,
   // With pre_inplace the incoming rows are gradients of gelu(pre): the pass over them multiplies them by
   // gelu'(pre) and writes them back, so that everything below sees the gradient of the pre-activation.
   CCF_REQUIRE(!pre_inplace || !g_rows, CCF_ERR_ARG, "%s: the in-place GELU gradient needs rows in expert order", what);
+  // input gradient: on the stored weight read as [K][N] where the shape allows, else on a transposed copy
+  const bool kn = !g_dgrad_transpose && n_in % Cfg5::BN == 0 && static_cast<long long>(n_out) * n_in < (1ll << 31);
+  const int dgrad_epi = gelu_pre ? kEpiGeluGrad : kEpiPlain;
+  // the launch that lays out the K ranges also builds the tile plans of both GEMMs
+  const PlanReq rows_plan = setup_gemm(max_rows, E, n_in, n_out, dgrad_epi, kn, ws.plan_rows, 0, current_options()).req;
+  const PlanReq w_plan = wgrad_plan_request(E, n_out, n_in, ws.plan_w);
+  const bool plans = max_rows > 0 && static_cast<long long>(E) * n_out < (1ll << 31);
   if (int rc = launch_kseg(offsets, E, max_rows, n_out, ws.n_blk, ws.k_seg, ws.row_off, ws.blk_row0,
-                           ws.blk_cnt, ws.row_lo, ws.zero_row, stream))
+                           ws.blk_cnt, ws.row_lo, ws.zero_row, plans ? &rows_plan : nullptr, plans ? &w_plan : nullptr,
+                           stream))
     return rc;
   // rows form: gathered gradient rows go to a_t as a plain [rows, n_out] matrix; rows already in expert order stay
   const half_t *g_mat = (rows_form && !g_rows) ? grad_out : ws.a_t;
   if (int rc = launch_transpose_rows(grad_out, g_rows, ws.blk_row0, ws.blk_cnt, ws.n_blk, n_out, ws.ld_t,
                                      (rows_form && !g_rows) ? nullptr : ws.a_t, ws.partial, stream, pre_inplace, !rows_form))
     return rc;
-  // input gradient: on the stored weight read as [K][N] where the shape allows, else on a transposed copy
-  const bool kn = !g_dgrad_transpose && n_in % Cfg5::BN == 0 && static_cast<long long>(n_out) * n_in < (1ll << 31);
   if (!kn) {
     if (int rc = launch_transpose_weights(w, ws.w_t, E, n_out, n_in, stream)) return rc;
   }
   // gelu_pre: the input was gelu(gelu_pre); the gradient is then taken through the GELU in the epilogue
   CCF_REQUIRE(!gelu_pre || !gi_rows, CCF_ERR_ARG, "%s: the GELU gradient needs rows in expert order", what);
   if (int rc = grouped_gemm(grad_out, g_rows, offsets, max_rows, E, n_in, n_out, kn ? w : ws.w_t, nullptr,
-                            gelu_pre ? kEpiGeluGrad : kEpiPlain, grad_in, gi_rows, nullptr, ws.plan_rows, stream,
-                            what, kn, const_cast<half_t *>(gelu_pre)))
+                            dgrad_epi, grad_in, gi_rows, nullptr, ws.plan_rows, stream,
+                            what, kn, const_cast<half_t *>(gelu_pre), 0, plans))
     return rc;
   // weight and bias gradients
   const half_t *in_mat = (rows_form && !in_rows) ? in : ws.b_t;
@@ -1432,9 +1452,9 @@ int linear_backward(half_t *grad_out, const int32_t *g_rows, const half_t *in,
   if (int rc = launch_bias_reduce(ws.partial, ws.k_seg, E, n_out, grad_b, stream)) return rc;
   if (rows_form)
     return grouped_gemm_krows(g_mat, n_out, in_mat, n_in, ws.row_lo, ws.row_off, E, n_out, n_in, grad_w, ws.plan_w,
-                              ws.zero_row, grid, stream, what);
+                              ws.zero_row, grid, stream, what, plans);
   return grouped_gemm_kseg(ws.a_t, ws.ld_t, ws.b_t, ws.ld_t, ws.k_seg, ws.row_off, E, n_out, n_in,
-                           grad_w, ws.plan_w, stream, what);
+                           grad_w, ws.plan_w, stream, what, plans);
 }
 
 }  // namespace

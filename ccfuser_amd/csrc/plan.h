@@ -156,8 +156,9 @@ __host__ __device__ inline int sk_tail_segments(int q, int k_tiles) { return (q 
 // this with the workgroup's `part`).  Every workgroup repeats the small scans and takes a share
 // of the experts and of the idle entries; which entries stay idle is known in closed form, so
 // no entry is written by two workgroups and their order does not matter.
+// uniform_rows > 0: every expert has that many rows (offsets is not read).
 __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__ offsets, int E,
-                                  int part = 0, int nparts = 1) {
+                                  int part = 0, int nparts = 1, int uniform_rows = 0) {
   const int BM = rq.BM, max_tiles = rq.max_tiles, max_rows = rq.max_rows, n_tiles_n = rq.n_tiles_n;
   const int k_tiles = rq.k_tiles;
   int spx = rq.spx;                 // lowered below by the workgroups given to skinny tiles
@@ -171,7 +172,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   __shared__ int s_long[1025];     // exclusive scan of long M tiles per expert
   __shared__ int s_short[1025];    // exclusive scan of short M tiles per expert (0 or 1 each)
   for (int e = threadIdx.x; e <= E; e += blockDim.x) {
-    int v = offsets[e];
+    int v = uniform_rows > 0 ? e * uniform_rows : offsets[e];
     s_off[e] = v < max_rows ? v : max_rows;          // never plan past the caller's bound
   }
   __syncthreads();
@@ -415,6 +416,13 @@ int ffn2_forward_combine(const void *h, const int32_t *token_row, const int32_t 
                          int max_rows, int num_expert, int d_model, int d_ffn, const void *w2, const void *b2,
                          const void *score, void *out, void *workspace, size_t workspace_bytes, hipStream_t stream,
                          const GemmOptions *planned);
+// bwd.hip: the padded K ranges and row blocks of a backward call; the same launch builds the tile plan of its
+// input-gradient GEMM (`rows_plan`, from the offsets) and of its weight-gradient GEMM (`w_plan`: every expert
+// has seg_rows output rows) when given.
+int launch_kseg(const int32_t *offsets, int E, int max_rows, int seg_rows, int n_blk, int32_t *k_seg,
+                int32_t *row_off, int32_t *blk_row0, int32_t *blk_cnt, int32_t *row_lo, half_t *zero_row,
+                const PlanReq *rows_plan, const PlanReq *w_plan, hipStream_t stream);
+
 // route.hip: ccf_route(), whose last launch also builds n_plans (0..2) tile plans from the offsets.  gate_row_len > 0:
 // the head of the workspace already holds the gate kernel's counts, one row per gate_row_len flat indices.
 int route_with_plans(const int64_t *gate_idx, int n_flat, int num_expert, int top_k, int capacity,
