@@ -25,6 +25,8 @@ SIGNATURES = {
     "ccf_last_error": (C.c_char_p, []),
     "ccf_set_option": (_i, [C.c_char_p, _i]),
     "ccf_gate_topk_softmax": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
+    "ccf_gate_backward_workspace_bytes": (_sz, [_i, _i]),
+    "ccf_gate_backward": (_i, [_p, _p, _p, _i, _i, _i, _p, _p, _p, _sz, _p]),
     "ccf_route_workspace_bytes": (_sz, [_i, _i]),
     "ccf_expert_count": (_i, [_p, _i, _p, _i, _p]),
     "ccf_assign_pos": (_i, [_p, _p, _i, _i, _p, _p, _sz, _p]),

@@ -472,6 +472,121 @@ int gate_forward(const void *x, const void *wg, const void *bg, int tokens, int 
 }
 }  // namespace ccf
 
+namespace ccf {
+namespace {
+
+// ---- backward of the softmax over the selected logits and of the selection --------------
+// A workgroup takes kGbTokens tokens: thread t computes the k values of its token,
+//   g_j = s_j (grad_j - sum_i s_i grad_i)    (fp32),
+// the workgroup zero-fills its rows of grad_logits and, behind a barrier, every thread stores its
+// k values at their experts' columns.  The bias gradient is the column sum of the unrounded
+// values: wavefront w sums experts w, w + 4, ... over the workgroup's tokens (lane l takes
+// entries l, l + 64, ... in order, then a fixed tree over the lanes), so the result does not
+// depend on scheduling; gate_bias_reduce_kernel adds the workgroups' sums in order.
+constexpr int kGbTokens = 256;
+
+__global__ void __launch_bounds__(kGbTokens)
+gate_backward_kernel(const half_t *__restrict__ score, const half_t *__restrict__ grad_score,
+                     const int64_t *__restrict__ idx, int tokens, int top_k, int E,
+                     half_t *__restrict__ grad_logits, float *__restrict__ partial) {
+  __shared__ float s_val[kGbTokens * kMaxTopK];
+  __shared__ int s_idx[kGbTokens * kMaxTopK];
+  const int t = threadIdx.x;
+  const int tok0 = blockIdx.x * kGbTokens;
+  const int tok = tok0 + t;
+  float g[kMaxTopK];
+  int ex[kMaxTopK];
+  if (tok < tokens) {
+    float s[kMaxTopK], dot = 0.0f;
+    for (int j = 0; j < top_k; ++j) {
+      s[j] = static_cast<float>(score[static_cast<size_t>(tok) * top_k + j]);
+      g[j] = static_cast<float>(grad_score[static_cast<size_t>(tok) * top_k + j]);
+      dot = fmaf(s[j], g[j], dot);
+    }
+    for (int j = 0; j < top_k; ++j) {
+      g[j] = s[j] * (g[j] - dot);
+      const int64_t e = idx[static_cast<size_t>(tok) * top_k + j];
+      ex[j] = (e >= 0 && e < E) ? static_cast<int>(e) : -1;
+    }
+  } else {
+    for (int j = 0; j < top_k; ++j) {
+      g[j] = 0.0f;
+      ex[j] = -1;
+    }
+  }
+  for (int j = 0; j < top_k; ++j) {
+    s_val[t * top_k + j] = g[j];
+    s_idx[t * top_k + j] = ex[j];
+  }
+  // this workgroup's rows of grad_logits are one contiguous range
+  const int n_tok = tokens - tok0 < kGbTokens ? tokens - tok0 : kGbTokens;
+  half_t *rows = grad_logits + static_cast<size_t>(tok0) * E;
+  const size_t n_el = static_cast<size_t>(n_tok) * E;
+  for (size_t i = t; i < n_el; i += kGbTokens) rows[i] = static_cast<half_t>(0.0f);
+  __syncthreads();                                  // the zeros are written (and s_val, s_idx)
+  if (tok < tokens) {
+    for (int j = 0; j < top_k; ++j)
+      if (ex[j] >= 0) rows[static_cast<size_t>(t) * E + ex[j]] = static_cast<half_t>(g[j]);
+  }
+  if (!partial) return;
+  const int lane = t & 63, wave = t >> 6;
+  const int n_ent = kGbTokens * top_k;
+  for (int e = wave; e < E; e += kGbTokens / 64) {
+    float acc = 0.0f;
+    for (int i = lane; i < n_ent; i += 64) acc += s_idx[i] == e ? s_val[i] : 0.0f;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (lane == 0) partial[static_cast<size_t>(blockIdx.x) * E + e] = acc;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+gate_bias_reduce_kernel(const float *__restrict__ partial, int n_wg, int E, half_t *__restrict__ grad_bias) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= E) return;
+  float acc = 0.0f;
+  for (int w = 0; w < n_wg; ++w) acc += partial[static_cast<size_t>(w) * E + e];
+  grad_bias[e] = static_cast<half_t>(acc);
+}
+
+}  // namespace
+}  // namespace ccf
+
+extern "C" size_t ccf_gate_backward_workspace_bytes(int tokens, int tot_expert) {
+  if (tokens <= 0 || tot_expert <= 0) return 0;
+  return sizeof(float) * static_cast<size_t>((tokens + ccf::kGbTokens - 1) / ccf::kGbTokens) * tot_expert;
+}
+
+extern "C" int ccf_gate_backward(const void *score, const void *grad_score, const int64_t *idx, int tokens,
+                                 int top_k, int tot_expert, void *grad_logits, void *grad_bias, void *workspace,
+                                 size_t workspace_bytes, ccf_stream_t stream) {
+  using namespace ccf;
+  CCF_REQUIRE(tokens >= 0 && tot_expert > 0 && tot_expert <= 1024, CCF_ERR_ARG, "gate_backward: bad size");
+  CCF_REQUIRE(top_k >= 1 && top_k <= kMaxTopK && top_k <= tot_expert, CCF_ERR_SHAPE,
+              "gate_backward: top_k=%d outside 1..min(%d, tot_expert=%d)", top_k, kMaxTopK, tot_expert);
+  if (tokens == 0) {                                 // no rows to write; a sum over nothing
+    if (!grad_bias) return CCF_OK;
+    hipLaunchKernelGGL(gate_bias_reduce_kernel, dim3((tot_expert + 255) / 256), dim3(256), 0, as_stream(stream),
+                       static_cast<const float *>(nullptr), 0, tot_expert, static_cast<half_t *>(grad_bias));
+    return check_launch("gate_bias_reduce_kernel");
+  }
+  CCF_REQUIRE(score && grad_score && idx && grad_logits, CCF_ERR_ARG, "gate_backward: null pointer");
+  const size_t need = ccf_gate_backward_workspace_bytes(tokens, tot_expert);
+  CCF_REQUIRE(!grad_bias || (workspace && workspace_bytes >= need), CCF_ERR_WORKSPACE,
+              "gate_backward: workspace of %zu bytes needed for the bias gradient, %zu given", need, workspace_bytes);
+  const int n_wg = (tokens + kGbTokens - 1) / kGbTokens;
+  hipLaunchKernelGGL(gate_backward_kernel, dim3(n_wg), dim3(kGbTokens), 0, as_stream(stream),
+                     static_cast<const half_t *>(score), static_cast<const half_t *>(grad_score), idx, tokens, top_k,
+                     tot_expert, static_cast<half_t *>(grad_logits), grad_bias ? static_cast<float *>(workspace) : nullptr);
+  if (int rc = check_launch("gate_backward_kernel")) return rc;
+  if (grad_bias) {
+    hipLaunchKernelGGL(gate_bias_reduce_kernel, dim3((tot_expert + 255) / 256), dim3(256), 0, as_stream(stream),
+                       static_cast<const float *>(workspace), n_wg, tot_expert, static_cast<half_t *>(grad_bias));
+    return check_launch("gate_bias_reduce_kernel");
+  }
+  return CCF_OK;
+}
+
 extern "C" int ccf_gate_topk_softmax(const void *x, const void *wg, const void *bg, int tokens,
                                      int d_model, int tot_expert, int top_k, int dtype,
                                      int64_t *idx_out, void *score_out, void *logits_out,

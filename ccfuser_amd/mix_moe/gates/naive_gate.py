@@ -11,8 +11,9 @@ from .base_gate import BaseGate
 class _GateFunction(torch.autograd.Function):
     """The fused gate kernel with the backward autograd derives for the reference's
     linear -> topk -> softmax (naive_gate.py:31-38): softmax over the k selected
-    logits, the selection as a scatter into [T, E], then the linear layer.  The two
-    products with the [T, E] gradient are small library GEMMs."""
+    logits, the selection as a scatter into [T, E], then the linear layer.  For fp16 the
+    first two are one HIP kernel (``ops.gate_backward``); the two products with the [T, E]
+    gradient are small library GEMMs."""
 
     @staticmethod
     def forward(ctx, x, weight, bias, top_k, return_logits):
@@ -30,15 +31,19 @@ class _GateFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_idx, grad_score, grad_logits=None):
         x, weight, idx, score = ctx.saved_tensors
-        s = score.float()
-        g = grad_score.float()
-        g_val = s * (g - (s * g).sum(-1, keepdim=True))
-        g_logits = torch.zeros(x.shape[0], weight.shape[0], dtype=torch.float32, device=x.device)
-        g_logits.scatter_add_(1, idx, g_val)
-        g16 = g_logits.to(x.dtype)
+        want_bias = ctx.has_bias and ctx.needs_input_grad[2]
+        if x.dtype == torch.float16:
+            g16, grad_b = ops.gate_backward(score, grad_score.contiguous(), idx, weight.shape[0], want_bias)
+        else:
+            s = score.float()
+            g = grad_score.float()
+            g_val = s * (g - (s * g).sum(-1, keepdim=True))
+            g_logits = torch.zeros(x.shape[0], weight.shape[0], dtype=torch.float32, device=x.device)
+            g_logits.scatter_add_(1, idx, g_val)
+            g16 = g_logits.to(x.dtype)
+            grad_b = g_logits.sum(0).to(x.dtype) if want_bias else None
         grad_x = torch.mm(g16, weight) if ctx.needs_input_grad[0] else None
         grad_w = torch.mm(g16.t(), x) if ctx.needs_input_grad[1] else None
-        grad_b = g_logits.sum(0).to(x.dtype) if ctx.has_bias and ctx.needs_input_grad[2] else None
         return grad_x, grad_w, grad_b, None, None
 
 

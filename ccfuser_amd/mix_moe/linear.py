@@ -118,6 +118,20 @@ class MixMOELinear2(Function):
         return g_act, None, None, grad_w, grad_b
 
 
+_ONES = {}
+
+
+def _ones(n, dtype, device):
+    """A constant vector of ones (the scores of a plain sum over the k slots), made once per size."""
+    key = (n, dtype, device)
+    t = _ONES.get(key)
+    if t is None:
+        if len(_ONES) >= 8:
+            _ONES.clear()
+        t = _ONES[key] = torch.ones(n, dtype=dtype, device=device)
+    return t
+
+
 class MixMOEFusedFFN(Function):
     """Both expert linears with the erf GELU between them as one differentiable step:
     ``y_flat[pos[j]] = gelu(x[pos[j] // k] @ W1[e]^T + b1[e]) @ W2[e]^T + b2[e]``.
@@ -158,8 +172,7 @@ class MixMOEFusedFFN(Function):
                                          w1.detach()[:E], n_flat, grad_w1[:E], grad_b1[:E], may_drop=may_drop,
                                          h_pre=h_pre)
         top_k = n_flat // input_buf.shape[0]
-        ones = torch.ones(n_flat, dtype=g_flat.dtype, device=g_flat.device)
-        grad_in = ops.combine(g_flat, ones, top_k, inv_pos)
+        grad_in = ops.combine(g_flat, _ones(n_flat, g_flat.dtype, g_flat.device), top_k, inv_pos)
         return grad_in, None, None, grad_w1, grad_b1, grad_w2, grad_b2
 
 

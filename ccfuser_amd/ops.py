@@ -70,6 +70,27 @@ def gate_topk_softmax(x: torch.Tensor, wg: torch.Tensor, bg: Optional[torch.Tens
     return (idx, score, logits) if return_logits else (idx, score)
 
 
+def gate_backward(score: torch.Tensor, grad_score: torch.Tensor, idx: torch.Tensor, tot_expert: int,
+                  want_bias: bool = True):
+    """(grad_logits fp16 [T, E], grad_bias fp16 [E] or None): the gate's top-k softmax and
+    selection, backwards."""
+    _check(score, "score", dtype=torch.float16, ndim=2)
+    _check(grad_score, "grad_score", dtype=torch.float16, ndim=2)
+    _check(idx, "idx", dtype=torch.int64, ndim=2)
+    if grad_score.shape != score.shape or idx.shape != score.shape:
+        raise ValueError("score, grad_score and idx must have one shape")
+    T, k = score.shape
+    E = int(tot_expert)
+    g_logits = torch.empty(T, E, dtype=torch.float16, device=score.device)
+    g_bias = torch.empty(E, dtype=torch.float16, device=score.device) if want_bias else None
+    with torch.cuda.device(score.device):
+        nbytes = _lib.lib().ccf_gate_backward_workspace_bytes(T, E) if want_bias else 0
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=score.device) if want_bias else None
+        _lib.call("ccf_gate_backward", _ptr(score), _ptr(grad_score), _ptr(idx), T, k, E, _ptr(g_logits),
+                  _ptr(g_bias), _ptr(ws), nbytes, _stream(score))
+    return g_logits, g_bias
+
+
 # --------------------------------------------------------------- routing
 def expert_count(gate_idx: torch.Tensor, expert_count_out: torch.Tensor) -> None:
     """Accumulate the histogram of ``gate_idx`` into ``expert_count_out`` (int32)."""

@@ -108,6 +108,24 @@ int ccf_gate_topk_softmax(const void *x, const void *wg, const void *bg,
                           int dtype, int64_t *idx_out, void *score_out,
                           void *logits_out, ccf_stream_t stream);
 
+/* Bytes of workspace ccf_gate_backward needs when it returns the bias gradient (no counterpart in the reference). */
+size_t ccf_gate_backward_workspace_bytes(int tokens, int tot_expert);
+
+/*
+ * Backward of the gate's softmax over the k selected logits and of the selection:
+ *   grad_logits[t, idx[t, j]] = s_j * (g_j - sum_i s_i g_i),  s = score[t, :], g = grad_score[t, :],
+ * zero in every other column (fp32 arithmetic, rounded once to fp16), and grad_bias[e] = the sum of column e
+ * over the tokens (of the unrounded values, in a fixed order).  The two products of grad_logits with the input
+ * and with the gate weight, which complete the linear layer's backward, are plain GEMMs and stay with the caller.
+ * What autograd derives for NaiveGate.forward's topk -> softmax, mix_moe/mix_moe/gates/naive_gate.py:31-38.
+ *   score, grad_score fp16 [tokens, top_k]; idx int64 [tokens, top_k] (entries outside 0 .. tot_expert-1 are
+ *   skipped); grad_logits fp16 [tokens, tot_expert]; grad_bias fp16 [tot_expert] or NULL (then no workspace).
+ */
+int ccf_gate_backward(const void *score, const void *grad_score, const int64_t *idx,
+                      int tokens, int top_k, int tot_expert, void *grad_logits,
+                      void *grad_bias, void *workspace, size_t workspace_bytes,
+                      ccf_stream_t stream);
+
 /* --------------------------------------------------------------- routing */
 
 /* Bytes of workspace ccf_route / ccf_assign_pos need for n_flat indices. */

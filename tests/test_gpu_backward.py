@@ -91,6 +91,31 @@ def test_ffn_backward_stages_with_split_last_round(transpose):
         ops.set_option("skinny", 1)
 
 
+@pytest.mark.parametrize("T,k,E,seed", [(4096, 2, 8, 0), (300, 3, 64, 1), (1000, 8, 1024, 2), (257, 1, 5, 3), (1, 1, 1, 4)])
+def test_gate_backward_of_softmax_and_selection(T, k, E, seed):
+    """ccf_gate_backward against the oracle's formula (softmax over the k selected logits
+    backwards, scattered into [T, E]; the bias gradient its column sums): the scattered values
+    are the fp32 values rounded once, so they must match a float32 evaluation to one fp16 step;
+    twice the same bits; and no bias gradient when none is asked for."""
+    from ccfuser_amd import ops
+    _say(f"gate backward T={T} k={k} E={E}")
+    g = torch.Generator().manual_seed(seed)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    score = torch.softmax(torch.randn(T, k, generator=g), dim=-1).half()
+    gs = torch.randn(T, k, generator=g).half()
+    s32, g32 = score.float(), gs.float()
+    g_val = s32 * (g32 - (s32 * g32).sum(-1, keepdim=True))
+    ref = torch.zeros(T, E).scatter_add_(1, idx, g_val)
+    gl, gb = ops.gate_backward(score.cuda(), gs.cuda(), idx.cuda(), E)
+    gl2, gb2 = ops.gate_backward(score.cuda(), gs.cuda(), idx.cuda(), E)
+    torch.cuda.synchronize()
+    assert torch.equal(gl, gl2) and torch.equal(gb, gb2)
+    assert float((gl.cpu().float() - ref).abs().max()) <= 2.0 ** -10 * max(1.0, float(ref.abs().max()))
+    _close(gb, ref.sum(0), "grad_bias")
+    gl3, none = ops.gate_backward(score.cuda(), gs.cuda(), idx.cuda(), E, want_bias=False)
+    assert none is None and torch.equal(gl3, gl)
+
+
 @pytest.mark.parametrize("mode", [-1, -3, -5, -6, 1])
 def test_input_gradient_with_skinny_tiles(mode):
     """The input-gradient GEMM on the stored [K][N] weight with every expert's remainder rows
