@@ -22,6 +22,7 @@ class _GateFunction(torch.autograd.Function):
                                     return_logits=return_logits)
         ctx.save_for_backward(x, weight, res[0], res[1])
         ctx.has_bias = bias is not None
+        ctx.set_materialize_grads(False)                 # no zero-filled gradients for the index outputs
         ctx.mark_non_differentiable(res[0])
         if return_logits:
             ctx.mark_non_differentiable(res[2])
@@ -31,6 +32,8 @@ class _GateFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_idx, grad_score, grad_logits=None):
         x, weight, idx, score = ctx.saved_tensors
+        if grad_score is None:                           # the scores were not used
+            return None, None, None, None, None
         want_bias = ctx.has_bias and ctx.needs_input_grad[2]
         if x.dtype == torch.float16:
             g16, grad_b = ops.gate_backward(score, grad_score.contiguous(), idx, weight.shape[0], want_bias)
