@@ -502,3 +502,42 @@ def test_fused_layer_with_many_experts(T, d, f, E, k):
     assert O.max_abs_err(fused.cpu(), ref["out"]) <= MAX_ABS
     assert O.mean_rel_err(fused.cpu(), ref["out"]) <= MEAN_REL
     assert torch.equal(fused, _staged_forward(ops, args, E, k, -1))
+
+
+def _random_layer_shapes(count, seed):
+    g = torch.Generator().manual_seed(seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    shapes = []
+    for i in range(count):
+        E = ri(1, 40)
+        k = ri(1, min(4, E))
+        T = ri(1, 3000)
+        d, f = 64 * ri(1, 12), 64 * ri(1, 16)
+        cap = -1 if i % 3 else max(1, (T * k) // (2 * E))       # every third case drops about half of the busier experts' slots
+        shapes.append((T, d, f, E, k, cap, 9000 + i))
+    return shapes + [(1, 64, 64, 1, 1, -1, 9100), (257, 832, 320, 3, 3, 100, 9101)]
+
+
+@pytest.mark.parametrize("T,d,f,E,k,cap,seed", _random_layer_shapes(12, 777))
+def test_fused_layer_random_shapes(T, d, f, E, k, cap, seed):
+    """Shapes drawn at random (1-3000 tokens, widths any multiple of 64 up to 768 x 1024, 1-40
+    experts, top-1..4, every third with a binding capacity) plus a single token and widths that
+    are no multiple of 256: routing bit-exact, output within the tolerance, fused call = staged
+    calls bit for bit."""
+    from ccfuser_amd import ops
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).half()
+    x, wg, bg = r(T, d), r(E, d, sc=0.3), r(E, sc=0.3)
+    w1, b1, w2, b2 = r(E, f, d, sc=0.1), r(E, f, sc=0.1), r(E, d, f, sc=0.1), r(E, d, sc=0.1)
+    _say(f"random layer T={T} d={d} f={f} E={E} k={k} cap={cap}")
+    args = [a.cuda() for a in (x, wg, bg, w1, b1, w2, b2)]
+    fused, rt = ops.moe_forward(*args, k, cap, return_routing=True)
+    ref = O.moe_layer_forward(x, wg, bg, w1, b1, w2, b2, k, capacity=cap)
+    R = int(ref["offsets"][-1])
+    assert torch.equal(rt["idx"].cpu().view(-1), ref["idx_kept"].view(-1))      # after the capacity limit
+    assert torch.equal(rt["offsets"].cpu().long(), ref["offsets"].long())
+    assert torch.equal(rt["pos"].cpu()[:R], ref["pos"])
+    assert O.max_abs_err(fused.cpu(), ref["out"]) <= MAX_ABS
+    if float(ref["out"].abs().mean()) > 1e-6:
+        assert O.mean_rel_err(fused.cpu(), ref["out"]) <= MEAN_REL
+    assert torch.equal(fused, _staged_forward(ops, args, E, k, cap))
