@@ -71,6 +71,7 @@ struct GroupedArgs {
   // skinny list (layout in plan.h) of this GEMM, or NULL
   const int32_t *skinny;
   float *sk_partial;        // partial tiles of the skinny tiles when they run as a launch of their own
+  int sk_positions;         // skinny ranges inside the persistent launch: most points in time they are spread over (0: one per round)
 };
 
 // Epilogue forms of the grouped GEMM.
@@ -94,10 +95,11 @@ __device__ __forceinline__ int tile_row_to_local(int r, int rows) {
 // Global source of every tile load of this lane for the tile of plan entry
 // `ent`: K element 0 of the (clamped) A row and B row, at this lane's K chunk.
 // Padded A rows re-read the tile's last real row, B rows past N the last row.
+// tid: threadIdx.x, or fresh_tid() where what is derived from it must not be kept from an earlier call.
 template <class Cfg, bool kSeg = false, bool kKN = false>
 __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v ent,
                                              const half_t *(&a_src)[Cfg::A_DMA],
-                                             const half_t *(&b_src)[kKN ? 2 : Cfg::B_DMA]) {
+                                             const half_t *(&b_src)[kKN ? 2 : Cfg::B_DMA], int tid) {
   using ML = GemmMainloop<Cfg>;
   const int row0 = ent[1], rows = ent[2], n0 = ent[3] * Cfg::BN;
   const int lda = kSeg ? p.lda : p.K, ldb = kSeg ? p.ldb : p.K;
@@ -111,21 +113,20 @@ __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v e
   }
 #pragma unroll
   for (int i = 0; i < Cfg::A_DMA; ++i) {
-    const int r = ML::dma_row(i);
+    const int r = ML::dma_row(i, tid);
     const int rc = tile_row_to_local<Cfg>(r, rows);
     int g = row0 + rc;
     if constexpr (kSeg) g -= ent[0] * p.seg_rows;      // sorted row j of expert e is row j - e*seg_rows of A
     else if (p.a_rows) g = p.a_rows[g];
     if constexpr (kSeg) {
-      a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(g)) * static_cast<uint32_t>(lda) + ML::dma_chunk(r) * 8;
+      a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(g)) * static_cast<uint32_t>(lda) + ML::dma_chunk(r, tid) * 8;
     } else {
-      a_src[i] = p.A + static_cast<size_t>(g) * p.K + ML::dma_chunk(r) * 8;
+      a_src[i] = p.A + static_cast<size_t>(g) * p.K + ML::dma_chunk(r, tid) * 8;
     }
   }
   if constexpr (kKN) {
     // B is [E, K, N]: K row r of the tile, the columns LDS unit u of that row holds (N % BN == 0)
     using R = RingFor<Cfg, true>;
-    const int tid = threadIdx.x;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {                          // loads 0 and 1; load i >= 2 is 16 rows below load i - 2
       const int r = R::kn_dma_row(i, tid);
@@ -134,12 +135,12 @@ __device__ __forceinline__ void tile_sources(const GroupedArgs &p, const int4v e
   } else {
 #pragma unroll
     for (int i = 0; i < Cfg::B_DMA; ++i) {
-      const int r = ML::dma_row(i);
+      const int r = ML::dma_row(i, tid);
       const int n = (n0 + r) < p.N ? (n0 + r) : p.N - 1;
       if constexpr (kSeg) {
-        b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r) * 8;
+        b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r, tid) * 8;
       } else {
-        b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r) * 8;
+        b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r, tid) * 8;
       }
     }
   }
@@ -333,7 +334,7 @@ grouped_gemm_kernel(GroupedArgs p) {
   if (e < 0) return;                                 // surplus workgroup of the worst-case grid
   const half_t *a_src[Cfg::A_DMA];
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
-  tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
+  tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src, threadIdx.x);
   RingFor<Cfg, kKN>::run(a_src, b_src, k_tiles_of<Cfg, kSeg>(p, e) * Cfg::BK, ent[2], p.N);
   epilogue16<Cfg, kEpi, kSeg>(p, e, ent[1], ent[2], ent[3] * Cfg::BN);
 }
@@ -681,20 +682,33 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       }
     }
   }
-  // Skinny tiles cut along K inside this launch (plan.h): every workgroup takes its range of their K steps,
-  // half of the workgroups before their 256-row tiles and half behind them, so that at any time at most
-  // half of the chip streams weights for skinny tiles while the other half computes.  Groups of four
-  // consecutive slots (the M tiles of one N tile, which share their weight tiles) stay together.
+  // Skinny tiles cut along K inside this launch (plan.h): every workgroup takes its range of their K steps
+  // at some point between its 256-row tiles: behind its first sk_pos tiles (0 = in front of all, more than
+  // it has = behind all).  The points are spread over the launch by groups of four consecutive slots (the
+  // M tiles of one N tile, which share their weight tiles, stay together), so that at any time only a
+  // fraction of the chip streams weights for skinny tiles while the rest computes: with one point per
+  // round of tiles that fraction is 1 / (rounds + 1), and a skinny K step then runs at the pace of a few
+  // workgroups per XCD beside the others instead of at what HBM gives the whole chip.
   constexpr bool kSkInside = !kSeg && kEpi <= kEpiGeluKeep && Cfg::NW == 4;
-  const bool sk_first = ((slot_j >> 2) & 1) == 0;
+  int sk_pos = -1;                                    // -1: no range to run
   if constexpr (kSkInside) {
-    if (sk_first) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+    if (p.skinny && p.skinny[4] == 1 && p.skinny[0] > 0) {
+      const int rounds = __builtin_amdgcn_readfirstlane(p.skinny[5]);
+      int npos = rounds + 1;
+      npos = (p.sk_positions >= 2 && p.sk_positions < npos) ? p.sk_positions : npos;
+      const int at = (slot_j >> 2) % npos;
+      sk_pos = (at * rounds + (npos - 1) / 2) / (npos - 1);     // npos >= 2: rounds >= 1
+    }
+    if (sk_pos == 0) {
+      skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+      sk_pos = -1;
+    }
   }
   int4v ent = int4v{-1, 0, 0, 0};
   if (slot_j < slots_per_xcd) ent = plan[slot_j * 8 + xcd];
   if (ent[0] < 0) {                                   // no 256-row tile for this workgroup (the used slots of an XCD are a prefix)
     if constexpr (kSkInside) {
-      if (!sk_first) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+      if (sk_pos > 0) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
     }
     return;
   }
@@ -711,18 +725,22 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
   typename R::KMask mk{0, nullptr};
   if constexpr (kRows) rows_sources<Cfg>(p, ent[0], ent[1], ent[3], a_src, b_src, mk);
-  else tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src);
+  else tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src, threadIdx.x);
   int a_off[2], b_off[2];
   R::frag_offsets(a_off, b_off);
   half8 fa[R::AB][TM], fb[2][TN];
   R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg, kRows>(p, ent[0]), a_off, b_off, wave, bmul, amul, mk);
   R::reserve();
   int phase = 0;
+  int tiles_done = 0;
 
   for (;;) {
-    // the entry after this one; without one, the tail steps re-fetch this tile's first K tiles
+    // the entry after this one; without one, the tail steps re-fetch this tile's first K tiles.  When the
+    // skinny range comes behind this tile, the next tile starts from scratch behind it instead.
     const int nj = slot_j + stride;
-    const bool has_next = ahead[0] >= 0;
+    const bool real_next = ahead[0] >= 0;
+    const bool pause = kSkInside && real_next && tiles_done + 1 == sk_pos;
+    const bool has_next = real_next && !pause;
     const int4v nent = has_next ? ahead : ent;
     ahead = has_next ? entry_at(nj + stride) : ahead;  // used by the next tile: its latency hides under this one
     const int n_row0 = nent[1], n_rows = nent[2];
@@ -827,14 +845,31 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
     R::acc_settle();
     epilogue16<Cfg, kEpi, kSeg>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
     R::acc_settle();
-    if (!has_next) break;
+    ++tiles_done;
+    if (!real_next) break;
+    if constexpr (kSkInside) {
+      if (pause) {
+        // the skinny range, then the next tile as the first one was started
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_vmcnt<0>();
+        skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+        sk_pos = -1;
+        ent = ahead;
+        slot_j = nj;
+        ahead = entry_at(nj + stride);
+        tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src, fresh_tid());
+        R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg, kRows>(p, ent[0]), a_off, b_off, wave, bmul, amul, mk);
+        phase = 0;
+        continue;
+      }
+    }
     ent = nent;
     slot_j = nj;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   wait_vmcnt<0>();
   if constexpr (kSkInside) {
-    if (!sk_first) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
+    if (sk_pos > 0) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
   }
 }
 
@@ -879,7 +914,7 @@ grouped_gemm_tail_kernel(GroupedArgs p, int split_wgs) {
   const half_t *a_src[Cfg::A_DMA];
   constexpr int NB = kKN ? 2 : Cfg::B_DMA;
   const half_t *b_src[NB];
-  tile_sources<Cfg, false, kKN>(p, ent, a_src, b_src);
+  tile_sources<Cfg, false, kKN>(p, ent, a_src, b_src, threadIdx.x);
 #pragma unroll
   for (int i = 0; i < Cfg::A_DMA; ++i) a_src[i] += first * Cfg::BK;
 #pragma unroll
@@ -993,6 +1028,7 @@ int g_split_tail_min_kt = kSplitTailMinKT;
 int g_split_max_parts = 8;
 int g_fused_combine = 0;     // 1: top-2 layers add the gate-weighted expert outputs in the second GEMM's epilogue
 int g_skinny_pct = 70;       // a K step of a skinny tile in percent of a 256-row tile's (plan model); 0: no skinny tiles
+int g_skinny_positions = 0;  // skinny ranges inside the persistent launch: 0 = a point per round of tiles, 2 = in front of / behind all tiles
 int g_skinny_tail = 1;       // 0: skinny tiles never run as a launch of their own
 
 // The tuning knobs a grouped GEMM's plan and launches depend on, read once per call: the plan
@@ -1173,6 +1209,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   int32_t *plan = gs.plan, *tail = gs.tail;
   float *partial = gs.partial;
   GroupedArgs p;
+  p.sk_positions = g_skinny_positions;
   p.A = A;
   p.a_rows = a_rows;
   p.B = B;
@@ -1249,6 +1286,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
     if (int rc = check_launch("plan_kernel")) return rc;
   }
   GroupedArgs p;
+  p.sk_positions = g_skinny_positions;
   p.A = A;
   p.a_rows = nullptr;
   p.B = B;
@@ -1305,6 +1343,7 @@ int grouped_gemm_krows(const half_t *A, int lda, const half_t *B, int ldb, const
     if (int rc = check_launch("plan_kernel")) return rc;
   }
   GroupedArgs p;
+  p.sk_positions = g_skinny_positions;
   p.A = A;
   p.a_rows = nullptr;
   p.B = B;
@@ -1493,6 +1532,10 @@ extern "C" int ccf_set_option(const char *name, int value) {
   }
   if (!strcmp(name, "dgrad_transpose")) {
     g_dgrad_transpose = value != 0;
+    return CCF_OK;
+  }
+  if (!strcmp(name, "skinny_positions")) {
+    g_skinny_positions = value < 0 ? 0 : value;
     return CCF_OK;
   }
   if (!strcmp(name, "wgrad_transpose")) {

@@ -66,7 +66,8 @@ constexpr size_t kTailBytes = kTailHead + kSplitPartialBytes + kSkTailBytes;
 //   [0] tiles T   [1] ns   [2] tiles per XCD (XCD x owns entries [x * [2], (x + 1) * [2]))
 //   [3] q > 0: the tiles are cut along K, q K steps per workgroup; 0 otherwise
 //   [4] with q > 0: 0 = as a launch of their own, 1 = inside the persistent launch (each of its
-//       workgroups runs its range before or behind its 256-row tiles)     [5..7] unused
+//       workgroups runs its range at some point between its 256-row tiles)
+//   [5] most 256-row tiles a workgroup of the persistent launch runs     [6..7] unused
 //   [kSkinnyHead + 4 i ...] entry i < T: {expert, first sorted row, rows (1..kSkinnyRows), N tile}
 constexpr int kSkinnyRows = 64;
 constexpr int kSkinnyMaxWgs = 4;                     // per XCD
@@ -290,6 +291,11 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     skinny[2] = (T + 7) / 8;
     skinny[3] = s_tail_q;
     skinny[4] = s_tail_inside;
+    // most 256-row tiles a persistent workgroup runs (full rounds; a split last round goes elsewhere)
+    const int cus_x = rq.cus / 8 - ns_wgs;
+    const int per_x = ((use_skinny ? s_long[E] : s_long[E] + s_short[E]) * n_tiles_n + 7) / 8;
+    const int rounds = cus_x > 0 ? (per_x + cus_x - 1) / cus_x : 1;
+    skinny[5] = rounds > 0 ? rounds : 1;
   }
   const int per_long = (total_long + 7) / 8;
   const int per_short = (total_short + 7) / 8;

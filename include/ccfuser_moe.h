@@ -68,9 +68,12 @@ const char *ccf_last_error(void);
  *                     such a tile's K step in percent of a 256-row tile's (default 70); -n (1..4) forces
  *                     them with n workgroups per XCD; -5 forces them as a launch of their own behind the
  *                     persistent kernel, cut along K over all workgroups (the model's third choice); -6 forces
- *                     them cut along K inside the persistent launch, each workgroup running its range before
- *                     or behind its 256-row tiles (the fourth)
+ *                     them cut along K inside the persistent launch, each workgroup running its range at
+ *                     some point between its 256-row tiles (the fourth)
  *   "skinny_tail"     0/1 (default 1): the plan may choose that third way
+ *   "skinny_positions" 0 (default) or n >= 2: over how many points in time the fourth way spreads the
+ *                     workgroups' ranges (0: one in front of every round of tiles and one behind the last;
+ *                     2: half of the workgroups in front of all their tiles, half behind)
  *   "fused_combine"   0/1 (default 0): ccf_moe_forward with top_k = 2 adds the gate-weighted expert outputs
  *                     into the output in the second GEMM's epilogue (packed fp16 atomic adds onto zeros)
  *                     instead of running the combine pass; measured slower, kept for comparison
