@@ -684,11 +684,10 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   }
   // Skinny tiles cut along K inside this launch (plan.h): every workgroup takes its range of their K steps
   // at some point between its 256-row tiles: behind its first sk_pos tiles (0 = in front of all, more than
-  // it has = behind all).  The points are spread over the launch by groups of four consecutive slots (the
-  // M tiles of one N tile, which share their weight tiles, stay together), so that at any time only a
-  // fraction of the chip streams weights for skinny tiles while the rest computes: with one point per
-  // round of tiles that fraction is 1 / (rounds + 1), and a skinny K step then runs at the pace of a few
-  // workgroups per XCD beside the others instead of at what HBM gives the whole chip.
+  // it has = behind all).  The points are spread over the launch by XCD: the workgroups of an XCD pause
+  // together, so they stay in step with each other and keep sharing operand tiles through their L2 (spread
+  // by groups of slots inside an XCD measured slower), and at any time only about 1 / (rounds + 1) of the
+  // chip streams weights for skinny tiles while the rest computes.
   constexpr bool kSkInside = !kSeg && kEpi <= kEpiGeluKeep && Cfg::NW == 4;
   int sk_pos = -1;                                    // -1: no range to run
   if constexpr (kSkInside) {
@@ -696,7 +695,7 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       const int rounds = __builtin_amdgcn_readfirstlane(p.skinny[5]);
       int npos = rounds + 1;
       npos = (p.sk_positions >= 2 && p.sk_positions < npos) ? p.sk_positions : npos;
-      const int at = (slot_j >> 2) % npos;
+      const int at = xcd % npos;
       sk_pos = (at * rounds + (npos - 1) / 2) / (npos - 1);     // npos >= 2: rounds >= 1
     }
     if (sk_pos == 0) {
