@@ -71,6 +71,7 @@ struct GroupedArgs {
   // skinny list (layout in plan.h) of this GEMM, or NULL
   const int32_t *skinny;
   float *sk_partial;        // partial tiles of the skinny tiles when they run as a launch of their own
+  int tail_inside;          // 1: the persistent launch runs the parts of the split last round itself (no tail launch)
   int sk_positions;         // skinny ranges inside the persistent launch: most points in time they are spread over (0: one per round)
 };
 
@@ -160,6 +161,13 @@ __device__ __forceinline__ int2v scalar_load2(const int32_t *q) {
   int2v r;
   asm volatile("s_load_dwordx2 %0, %1, 0x0\n s_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(q) : "memory");
   return r;
+}
+
+// K tiles [first, first + count) of part `part` of S over k_tiles K tiles.
+__device__ __forceinline__ void part_range(int k_tiles, int part, int S, int &first, int &count) {
+  const int base = k_tiles / S, rem = k_tiles % S;
+  count = base + (part < rem ? 1 : 0);
+  first = part * base + (part < rem ? part : rem);
 }
 
 // K tiles of expert e's contraction.
@@ -703,32 +711,74 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       sk_pos = -1;
     }
   }
-  int4v ent = int4v{-1, 0, 0, 0};
-  if (slot_j < slots_per_xcd) ent = plan[slot_j * 8 + xcd];
-  if (ent[0] < 0) {                                   // no 256-row tile for this workgroup (the used slots of an XCD are a prefix)
+  // Plan entries are read through uniform indices (scalar loads, which do not queue behind the
+  // epilogue's stores) and one tile ahead of their use: `ahead` is the entry after the next one.
+  // The used slots of an XCD are a prefix; behind a workgroup's last tile comes, once, its part of
+  // the split last round (entry blockIdx.x of the split list, marked by its part count in bits 24..),
+  // when the launcher leaves the parts to this launch.
+  constexpr bool kTailInside = !kSeg && kEpi <= kEpiGeluKeep && Cfg::NW == 4;
+  bool tail_left = false;
+  if constexpr (kTailInside) tail_left = p.tail_inside != 0 && p.tail != nullptr;
+  auto entry_at = [&](int j) {
+    int4v t = int4v{-1, 0, 0, 0};
+    if (j < slots_per_xcd) t = scalar_load4(plan + __builtin_amdgcn_readfirstlane(j * 8 + xcd));
+    if constexpr (kTailInside) {
+      if (t[0] < 0 && tail_left) {
+        tail_left = false;
+        const int2v hd = scalar_load2(p.tail);            // tiles, parts
+        const int me = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x));
+        if (me < hd[0] * hd[1]) t = scalar_load4(reinterpret_cast<const int4v *>(p.tail + 64) + me);
+      }
+    }
+    return t;
+  };
+  // K tiles of an entry and the first of them: all of K, or the part's range
+  auto k_span = [&](const int4v &e, int &first) {
+    int kt = k_tiles_of<Cfg, kSeg, kRows>(p, e[0]);
+    first = 0;
+    if constexpr (kTailInside) {
+      const int S = e[3] >> 24;
+      if (S) part_range(kt, (e[3] >> 16) & 0xff, S, first, kt);
+    }
+    return kt;
+  };
+  int4v ent = entry_at(slot_j);
+  if (ent[0] < 0) {                                   // neither a 256-row tile nor a part for this workgroup
     if constexpr (kSkInside) {
       if (sk_pos > 0) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());
     }
     return;
   }
-  // Plan entries are read through uniform indices (scalar loads, which do not queue behind the
-  // epilogue's stores) and one tile ahead of their use: `ahead` is the entry after the next one.
-  auto entry_at = [&](int j) {
-    int4v t = int4v{-1, 0, 0, 0};
-    if (j < slots_per_xcd) t = scalar_load4(plan + __builtin_amdgcn_readfirstlane(j * 8 + xcd));
-    return t;
-  };
   int4v ahead = entry_at(slot_j + stride);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const half_t *a_src[R::A_SRCS];
   const half_t *b_src[kKN ? 2 : Cfg::B_DMA];
   typename R::KMask mk{0, nullptr};
-  if constexpr (kRows) rows_sources<Cfg>(p, ent[0], ent[1], ent[3], a_src, b_src, mk);
-  else tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src, threadIdx.x);
+  // sources of an entry from scratch (the first tile, and the tile behind a skinny range)
+  auto sources_of = [&](const int4v &e, int first, int tid) {
+    if constexpr (kRows) {
+      rows_sources<Cfg>(p, e[0], e[1], e[3], a_src, b_src, mk);
+    } else {
+      int4v e2 = e;
+      e2[3] &= 0xffff;
+      tile_sources<Cfg, kSeg, kKN>(p, e2, a_src, b_src, tid);
+      if constexpr (kTailInside) {
+        if (first) {
+#pragma unroll
+          for (int i = 0; i < Cfg::A_DMA; ++i) a_src[i] += first * Cfg::BK;
+#pragma unroll
+          for (int i = 0; i < (kKN ? 2 : Cfg::B_DMA); ++i) b_src[i] += static_cast<size_t>(first * Cfg::BK) * bmul;
+        }
+      }
+    }
+  };
+  int k_first0 = 0;
+  const int kt0 = k_span(ent, k_first0);
+  sources_of(ent, k_first0, threadIdx.x);
   int a_off[2], b_off[2];
   R::frag_offsets(a_off, b_off);
   half8 fa[R::AB][TM], fb[2][TN];
-  R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg, kRows>(p, ent[0]), a_off, b_off, wave, bmul, amul, mk);
+  R::prologue(fa, fb, a_src, b_src, kt0, a_off, b_off, wave, bmul, amul, mk);
   R::reserve();
   int phase = 0;
   int tiles_done = 0;
@@ -743,7 +793,9 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
     const int4v nent = has_next ? ahead : ent;
     ahead = has_next ? entry_at(nj + stride) : ahead;  // used by the next tile: its latency hides under this one
     const int n_row0 = nent[1], n_rows = nent[2];
-    const int KT = k_tiles_of<Cfg, kSeg, kRows>(p, ent[0]);
+    int k_first = 0, n_first = 0;
+    const int KT = k_span(ent, k_first);
+    k_span(nent, n_first);
     const int k_end = KT * Cfg::BK;
 
     R::zero_acc();
@@ -786,8 +838,9 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       // sources of the next tile (tile_sources() with the row indices already at hand); the
       // empty asm keeps the compiler from computing them before the loop above and holding
       // 16 more registers across it
-      int n_e = __builtin_amdgcn_readfirstlane(nent[0]), n_tn = __builtin_amdgcn_readfirstlane(nent[3]);
-      asm volatile("" : "+s"(n_e), "+s"(n_tn));
+      int n_e = __builtin_amdgcn_readfirstlane(nent[0]), n_tn = __builtin_amdgcn_readfirstlane(nent[3] & 0xffff);
+      int n_k0 = __builtin_amdgcn_readfirstlane(n_first * Cfg::BK);      // a part starts inside K
+      asm volatile("" : "+s"(n_e), "+s"(n_tn), "+s"(n_k0));
       const int lda = kSeg ? p.lda : p.K, ldb = kSeg ? p.ldb : p.K;
       const half_t *Ae = p.A, *Be;
       if constexpr (kSeg) {
@@ -814,14 +867,14 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
           a_src[i] = Ae + static_cast<size_t>(static_cast<uint32_t>(next_row[i])) * static_cast<uint32_t>(lda) +
                      ML::dma_chunk(r, tid1) * 8;
         } else {
-          a_src[i] = p.A + static_cast<size_t>(next_row[i]) * p.K + ML::dma_chunk(r, tid1) * 8;
+          a_src[i] = p.A + static_cast<size_t>(next_row[i]) * p.K + (n_k0 + ML::dma_chunk(r, tid1) * 8);
         }
       }
       if constexpr (kKN) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
           const int r = R::kn_dma_row(i, tid1);
-          b_src[i] = Be + static_cast<size_t>(r) * p.N + n0 + R::kn_col(r, R::kn_dma_unit(tid1));
+          b_src[i] = Be + (static_cast<size_t>(r) + n_k0) * p.N + n0 + R::kn_col(r, R::kn_dma_unit(tid1));
         }
       } else {
 #pragma unroll
@@ -831,7 +884,7 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
           if constexpr (kSeg) {
             b_src[i] = Be + static_cast<size_t>(n) * ldb + ML::dma_chunk(r, tid1) * 8;
           } else {
-            b_src[i] = Be + static_cast<size_t>(n) * p.K + ML::dma_chunk(r, tid1) * 8;
+            b_src[i] = Be + static_cast<size_t>(n) * p.K + (n_k0 + ML::dma_chunk(r, tid1) * 8);
           }
         }
       }
@@ -842,7 +895,28 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
       R::template k_range<false>(fa, fb, a_src, b_src, a_off, b_off, 2, 0, 4 * Cfg::BK, phase, wave, live_m, bmul, amul, mk);
     }
     R::acc_settle();
-    epilogue16<Cfg, kEpi, kSeg>(p, ent[0], ent[1], ent[2], ent[3] * Cfg::BN);
+    bool is_part = false;
+    if constexpr (kTailInside) is_part = (ent[3] >> 24) != 0;
+    if (is_part) {
+      // a part of the split last round: raw accumulators for the reduction launch, by workgroup id
+      float *out = p.partial + static_cast<size_t>(blockIdx.x) * (Cfg::BM * Cfg::BN);
+      const int tid = fresh_tid();
+      static_for<0, TM>([&](auto T) {
+        constexpr int tm = T.value;
+        const int tr = acc16_row<Cfg>(tm, tid);
+        static_for<0, TN>([&](auto J) {
+          constexpr int tn = J.value;
+          float4v v;
+          v[0] = R::template acc_get<tm, tn, 0>();
+          v[1] = R::template acc_get<tm, tn, 1>();
+          v[2] = R::template acc_get<tm, tn, 2>();
+          v[3] = R::template acc_get<tm, tn, 3>();
+          *reinterpret_cast<float4v *>(out + tr * Cfg::BN + acc16_col4<Cfg>(tn, tid)) = v;
+        });
+      });
+    } else {
+      epilogue16<Cfg, kEpi, kSeg>(p, ent[0], ent[1], ent[2], (ent[3] & 0xffff) * Cfg::BN);
+    }
     R::acc_settle();
     ++tiles_done;
     if (!real_next) break;
@@ -856,8 +930,10 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
         ent = ahead;
         slot_j = nj;
         ahead = entry_at(nj + stride);
-        tile_sources<Cfg, kSeg, kKN>(p, ent, a_src, b_src, fresh_tid());
-        R::prologue(fa, fb, a_src, b_src, k_tiles_of<Cfg, kSeg, kRows>(p, ent[0]), a_off, b_off, wave, bmul, amul, mk);
+        int first_p = 0;
+        const int kt_p = k_span(ent, first_p);
+        sources_of(ent, first_p, fresh_tid());
+        R::prologue(fa, fb, a_src, b_src, kt_p, a_off, b_off, wave, bmul, amul, mk);
         phase = 0;
         continue;
       }
@@ -883,13 +959,6 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
 // leave raw fp32 accumulators in a scratch area; splitk_reduce adds a tile's parts in part
 // order and applies the epilogue.  The area sits in front of the plan in the caller's workspace
 // (kTailHead, kTailBytes above).
-
-// K tiles [first, first + count) of part `part` of S over k_tiles K tiles.
-__device__ __forceinline__ void part_range(int k_tiles, int part, int S, int &first, int &count) {
-  const int base = k_tiles / S, rem = k_tiles % S;
-  count = base + (part < rem ? 1 : 0);
-  first = part * base + (part < rem ? part : rem);
-}
 
 // One part of one tail tile per workgroup: the main loop over its K range, raw accumulators out.
 // Workgroups from `split_wgs` on run the skinny list as a launch of its own (skinny_tail_role).
@@ -1028,7 +1097,8 @@ int g_split_max_parts = 8;
 int g_fused_combine = 0;     // 1: top-2 layers add the gate-weighted expert outputs in the second GEMM's epilogue
 int g_skinny_pct = 70;       // a K step of a skinny tile in percent of a 256-row tile's (plan model); 0: no skinny tiles
 int g_skinny_positions = 0;  // skinny ranges inside the persistent launch: 0 = a point per round of tiles, 2 = in front of / behind all tiles
-int g_skinny_tail = 1;       // 0: skinny tiles never run as a launch of their own
+int g_split_inside = 1;      // 1: the parts of a split last round run inside the persistent launch, 0: as a launch of their own
+int g_skinny_tail = 0;       // 0: skinny tiles never run as a launch of their own
 
 // The tuning knobs a grouped GEMM's plan and launches depend on, read once per call: the plan
 // and the kernels that consume it must agree even if another thread calls ccf_set_option
@@ -1209,6 +1279,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   float *partial = gs.partial;
   GroupedArgs p;
   p.sk_positions = g_skinny_positions;
+  p.tail_inside = 0;
   p.A = A;
   p.a_rows = a_rows;
   p.B = B;
@@ -1231,18 +1302,28 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   p.skinny = gs.skinny ? gs.skinny_list : nullptr;
   if (grid >= 8) {
     const long long g = grid < wgs ? grid : wgs;                // wgs is a multiple of 8
+    // the parts of a split last round: run by the persistent workgroups themselves behind their tiles (the
+    // four-wavefront kernels; part i is workgroup i's), else by a launch of their own
+    const bool parts_inside = split && g_split_inside && gs.v != &kVariants[kFwd8Variant];
+    p.tail_inside = parts_inside ? 1 : 0;
     hipLaunchKernelGGL(second ? v.persistent_gelu : v.persistent_plain, dim3(static_cast<unsigned>(g)),
                        dim3(v.threads), 0, stream, p, static_cast<int>(wgs / 8));
     if (split) {
       if (int rc = check_launch(what)) return rc;
-      // the skinny list may run as a launch of its own: `grid` more workgroups for it, more blocks in the reduction
+      // the skinny list may run as a launch of its own: `grid` more workgroups for it; whenever it may be cut
+      // along K (there or inside the persistent launch), more blocks in the reduction
       const bool sk = gs.req.sk_tail_ok;
-      if (b_kn) hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, true>), dim3(sk ? 2 * grid : grid), dim3(Cfg5::THREADS), 0,
-                                   stream, p, grid);
-      else hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, false>), dim3(sk ? 2 * grid : grid), dim3(Cfg5::THREADS), 0,
-                              stream, p, grid);
-      if (int rc = check_launch("grouped_gemm_tail_kernel")) return rc;
-      const dim3 rgrid(kTailMaxTiles + (sk ? kSkReduceX : 0), Cfg5::BM / 16);
+      const bool sk_cut = gs.skinny;
+      if (!parts_inside || sk) {
+        const int split_wgs = parts_inside ? 0 : grid;            // workgroups in front of the skinny list's
+        const int tail_grid = split_wgs + (sk ? grid : 0);
+        if (b_kn) hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, true>), dim3(tail_grid), dim3(Cfg5::THREADS), 0,
+                                     stream, p, split_wgs);
+        else hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, false>), dim3(tail_grid), dim3(Cfg5::THREADS), 0,
+                                stream, p, split_wgs);
+        if (int rc = check_launch("grouped_gemm_tail_kernel")) return rc;
+      }
+      const dim3 rgrid(kTailMaxTiles + (sk_cut ? kSkReduceX : 0), Cfg5::BM / 16);
       if (epi == kEpiPlain) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiPlain>), rgrid, dim3(256), 0, stream, p);
       else if (epi == kEpiGelu) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGelu>), rgrid, dim3(256), 0, stream, p);
       else hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGeluKeep>), rgrid, dim3(256), 0, stream, p);
@@ -1286,6 +1367,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   }
   GroupedArgs p;
   p.sk_positions = g_skinny_positions;
+  p.tail_inside = 0;
   p.A = A;
   p.a_rows = nullptr;
   p.B = B;
@@ -1343,6 +1425,7 @@ int grouped_gemm_krows(const half_t *A, int lda, const half_t *B, int ldb, const
   }
   GroupedArgs p;
   p.sk_positions = g_skinny_positions;
+  p.tail_inside = 0;
   p.A = A;
   p.a_rows = nullptr;
   p.B = B;
@@ -1531,6 +1614,10 @@ extern "C" int ccf_set_option(const char *name, int value) {
   }
   if (!strcmp(name, "dgrad_transpose")) {
     g_dgrad_transpose = value != 0;
+    return CCF_OK;
+  }
+  if (!strcmp(name, "split_inside")) {
+    g_split_inside = value != 0;
     return CCF_OK;
   }
   if (!strcmp(name, "skinny_positions")) {

@@ -205,14 +205,15 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       // workgroup's range stays within kSkTailSegs tiles
       const int tail_wgs = rq.cus < kSkTailMaxWgs ? rq.cus : kSkTailMaxWgs;
       int q_c = 0;
-      if (tail && rq.sk_tail_ok && nk1 > 0 && k_tiles > 0) {
+      if (tail && (rq.sk_tail_ok || rq.sk_beside_ok) && nk1 > 0 && k_tiles > 0) {
         const long long steps = static_cast<long long>(nk1) * n_tiles_n * k_tiles;
         const long long q = (steps + tail_wgs - 1) / tail_wgs;
         if (q < (1 << 20) && sk_tail_segments(static_cast<int>(q), k_tiles) <= kSkTailSegs) q_c = static_cast<int>(q);
       }
       if (nk1 > 0 && rq.skinny_pct < -kSkinnyMaxWgs) {
-        tail_q = q_c;                                  // forced (tests, measurements); 0 = not possible: no skinny tiles
-        tail_inside = rq.skinny_pct == -kSkinnyMaxWgs - 2 && rq.sk_beside_ok;
+        // forced (tests, measurements); 0 = not possible: no skinny tiles
+        tail_inside = rq.skinny_pct == -kSkinnyMaxWgs - 2;
+        tail_q = (tail_inside ? rq.sk_beside_ok : rq.sk_tail_ok) ? q_c : 0;
       } else if (nk1 > 0 && rq.skinny_pct < 0) {
         ns_wgs = rq.sk_beside_ok ? -rq.skinny_pct : 0; // forced
       } else if (nk1 > 0) {
@@ -230,7 +231,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
         if (q_c > 0) {
           const int c = rounds_cost(F1, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts) +
                         (q_c * kSkTailStepPct + 99) / 100 + kSkTailFixed;
-          if (c < best) { best = c; ns_wgs = 0; tail_q = q_c; tail_inside = 0; }
+          if (rq.sk_tail_ok && c < best) { best = c; ns_wgs = 0; tail_q = q_c; tail_inside = 0; }
           if (rq.sk_beside_ok) {
             const int ci = rounds_cost(F1, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts) +
                            (q_c * kSkInsideStepPct + 99) / 100 + kSkInsideFixed;

@@ -70,7 +70,10 @@ const char *ccf_last_error(void);
  *                     persistent kernel, cut along K over all workgroups (the model's third choice); -6 forces
  *                     them cut along K inside the persistent launch, each workgroup running its range at
  *                     some point between its 256-row tiles (the fourth)
- *   "skinny_tail"     0/1 (default 1): the plan may choose that third way
+ *   "skinny_tail"     0/1 (default 0): the plan may choose that third way (it costs a launch that the
+ *                     fourth way does without, and measured slower wherever both apply)
+ *   "split_inside"    0/1 (default 1): the parts of a split last round are run by the persistent workgroups
+ *                     themselves, each one part behind its tiles, instead of by a launch of their own
  *   "skinny_positions" 0 (default) or n >= 2: over how many points in time the fourth way spreads the
  *                     workgroups' ranges (0: one in front of every round of tiles and one behind the last;
  *                     2: half of the workgroups in front of all their tiles, half behind)

@@ -140,6 +140,7 @@ def test_input_gradient_with_skinny_tiles(mode):
     # cutting along K (the skinny tiles, and with them the last round of 256-row tiles) is forced on: K = 2048 is
     # below its default threshold; where bits are compared nothing is cut
     ops.set_option("split_tail", 0 if mode in (-1, -3) else 4)
+    ops.set_option("skinny_tail", 1 if mode == -5 else 0)
     try:
         ops.set_option("skinny", 0)
         whole = ops.ffn2_backward(gy, act, rt["dst_row"], rt["offsets"], n, w2)[0]
@@ -149,6 +150,7 @@ def test_input_gradient_with_skinny_tiles(mode):
     finally:
         ops.set_option("skinny", 1)
         ops.set_option("split_tail", 1)
+        ops.set_option("skinny_tail", 0)
     rows = gy[rt["dst_row"].long()].float()
     off = rt["offsets"].cpu().tolist()
     ref = torch.cat([rows[off[e]:off[e + 1]] @ w2[e].float() for e in range(E)])

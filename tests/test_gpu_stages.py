@@ -456,10 +456,14 @@ def test_ffn_special_cases():
     assert O.max_abs_err(pre.cpu(), ref) <= MAX_ABS
 
 
-def test_split_k_tail_at_its_default_threshold():
+@pytest.mark.parametrize("inside", [1, 0])
+def test_split_k_tail_at_its_default_threshold(inside):
     """K = 4096 is where the split of the last round switches on by itself: 36 M tiles x 16 N
-    tiles = 2.25 rounds of 256 workgroups, in both GEMMs, whole outputs against fp32."""
+    tiles = 2.25 rounds of 256 workgroups, in both GEMMs, whole outputs against fp32.  The parts
+    run inside the persistent launch (each workgroup one, behind its tiles) or as a launch of
+    their own."""
     from ccfuser_amd import ops
+    ops.set_option("split_inside", inside)
     g = torch.Generator().manual_seed(22)
     R, d, f, E = 8192, 4096, 4096, 6
     x = torch.randn(R, d, generator=g).half()
@@ -495,6 +499,7 @@ def test_split_k_tail_at_its_default_threshold():
     assert O.max_abs_err(out[1][1], y_ref) <= MAX_ABS and O.mean_rel_err(out[1][1], y_ref) <= MEAN_REL
     # the split did run: bits differ from the unsplit kernels
     assert not torch.equal(out[1][0], out[0][0]) and not torch.equal(out[1][1], out[0][1])
+    ops.set_option("split_inside", 1)
 
 
 def test_split_k_tail_all_epilogues():
@@ -518,8 +523,9 @@ def test_split_k_tail_all_epilogues():
     _say(f"split-K tail R={R} d={d} f={f} E={E} counts={r['counts'].tolist()}")
     results = {}
     ops.set_option("skinny", 0)               # every row in 256-row tiles: the tile count this test is built on
-    for mode in (0, 4):
-        ops.set_option("split_tail", mode)
+    for mode in (0, 4, -4):                   # -4: as 4, the parts as a launch of their own
+        ops.set_option("split_tail", abs(mode))
+        ops.set_option("split_inside", 0 if mode < 0 else 1)
         try:
             h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True)
             act, pre = ops.ffn1_keep(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1))
@@ -528,7 +534,10 @@ def test_split_k_tail_all_epilogues():
             results[mode] = [t.cpu() for t in (h, act, pre, y)]
         finally:
             ops.set_option("split_tail", 1)
+            ops.set_option("split_inside", 1)
     ops.set_option("skinny", 1)
+    # the same parts and the same order of summation wherever they run
+    assert all(torch.equal(a, b) for a, b in zip(results[4], results[-4]))
     buf = x[torch.div(pos, 1, rounding_mode="floor")].float()
     h_ref = torch.zeros(R, f)
     pre_ref = torch.zeros(R, f)
@@ -598,6 +607,7 @@ def test_skinny_tiles(R, d, f, E, skew, seed, mode, expect):
         # beside the 256-row tiles: keep those unsplit, the comparison is about the skinny path;
         # a launch of their own needs the split kernels launched (every K tile count allowed)
         ops.set_option("split_tail", 2 if mode <= -5 else 0)
+        ops.set_option("skinny_tail", 1 if mode == -5 else 0)   # the launch of their own is off by default
         try:
             h = ops.ffn1(dev(x), r["src_row"], r["offsets"], R, dev(w1), dev(b1), gelu=True, workspace=ws)
             info[m, 1] = ops.ffn_plan_info(ws, R, E, d, f, 1)
@@ -610,6 +620,7 @@ def test_skinny_tiles(R, d, f, E, skew, seed, mode, expect):
         finally:
             ops.set_option("skinny", 1)
             ops.set_option("split_tail", 1)
+            ops.set_option("skinny_tail", 0)
     _say(f"  plan, first GEMM: {info[mode, 1]}")
     _say(f"  plan, second GEMM: {info[mode, 2]}")
     for which in (1, 2):
