@@ -157,6 +157,13 @@ __device__ __forceinline__ int4v scalar_load4(const int4v *q) {
   asm volatile("s_load_dwordx4 %0, %1, 0x0\n s_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(q) : "memory");
   return r;
 }
+// two entries with one wait
+__device__ __forceinline__ void scalar_load4x2(const int4v *q0, const int4v *q1, int4v &r0, int4v &r1) {
+  asm volatile("s_load_dwordx4 %0, %2, 0x0\n s_load_dwordx4 %1, %3, 0x0\n s_waitcnt lgkmcnt(0)"
+               : "=&s"(r0), "=&s"(r1)
+               : "s"(q0), "s"(q1)
+               : "memory");
+}
 __device__ __forceinline__ int2v scalar_load2(const int32_t *q) {
   int2v r;
   asm volatile("s_load_dwordx2 %0, %1, 0x0\n s_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(q) : "memory");
@@ -714,22 +721,37 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
   // Plan entries are read through uniform indices (scalar loads, which do not queue behind the
   // epilogue's stores) and one tile ahead of their use: `ahead` is the entry after the next one.
   // The used slots of an XCD are a prefix; behind a workgroup's last tile comes, once, its part of
-  // the split last round (entry blockIdx.x of the split list, marked by its part count in bits 24..),
-  // when the launcher leaves the parts to this launch.
+  // the split last round (entry blockIdx.x of the split list, expert -1 when there is none, marked by
+  // its part count in bits 24..), when the launcher leaves the parts to this launch.  That entry is
+  // fetched together with the first plan entry, so it costs no wait of its own.
   constexpr bool kTailInside = !kSeg && kEpi <= kEpiGeluKeep && Cfg::NW == 4;
-  bool tail_left = false;
-  if constexpr (kTailInside) tail_left = p.tail_inside != 0 && p.tail != nullptr;
+  int4v tail_ent = int4v{-1, 0, 0, 0};
+  int4v ent = int4v{-1, 0, 0, 0};
+  {
+    const int4v *first = plan + __builtin_amdgcn_readfirstlane((slot_j < slots_per_xcd ? slot_j : 0) * 8 + xcd);
+    bool with_tail = false;
+    if constexpr (kTailInside) with_tail = p.tail_inside != 0 && p.tail != nullptr;
+    if (with_tail) {
+      const int me = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x));
+      scalar_load4x2(first, reinterpret_cast<const int4v *>(p.tail + 64) + me, ent, tail_ent);
+    } else {
+      ent = scalar_load4(first);
+    }
+    if (slot_j >= slots_per_xcd) ent[0] = -1;
+  }
+  auto take_tail = [&](int4v &t) {
+    if constexpr (kTailInside) {
+      if (t[0] < 0 && tail_ent[0] >= 0) {
+        t = tail_ent;
+        tail_ent[0] = -1;
+      }
+    }
+  };
+  take_tail(ent);
   auto entry_at = [&](int j) {
     int4v t = int4v{-1, 0, 0, 0};
     if (j < slots_per_xcd) t = scalar_load4(plan + __builtin_amdgcn_readfirstlane(j * 8 + xcd));
-    if constexpr (kTailInside) {
-      if (t[0] < 0 && tail_left) {
-        tail_left = false;
-        const int2v hd = scalar_load2(p.tail);            // tiles, parts
-        const int me = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x));
-        if (me < hd[0] * hd[1]) t = scalar_load4(reinterpret_cast<const int4v *>(p.tail + 64) + me);
-      }
-    }
+    take_tail(t);
     return t;
   };
   // K tiles of an entry and the first of them: all of K, or the part's range
@@ -742,7 +764,6 @@ grouped_gemm_persistent_kernel(GroupedArgs p, int slots_per_xcd) {
     }
     return kt;
   };
-  int4v ent = entry_at(slot_j);
   if (ent[0] < 0) {                                   // neither a 256-row tile nor a part for this workgroup
     if constexpr (kSkInside) {
       if (sk_pos > 0) skinny_tail_role<kKN>(p, static_cast<int>(blockIdx.x), 1, R::lds(), R::lds_addr());

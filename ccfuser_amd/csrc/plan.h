@@ -207,8 +207,9 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       int q_c = 0;
       if (tail && (rq.sk_tail_ok || rq.sk_beside_ok) && nk1 > 0 && k_tiles > 0) {
         const long long steps = static_cast<long long>(nk1) * n_tiles_n * k_tiles;
-        const long long q = (steps + tail_wgs - 1) / tail_wgs;
-        if (q < (1 << 20) && sk_tail_segments(static_cast<int>(q), k_tiles) <= kSkTailSegs) q_c = static_cast<int>(q);
+        // (a 32-bit division: more steps than fit one are more than a workgroup's range may hold anyway)
+        const int q = steps < (1ll << 30) ? (static_cast<int>(steps) + tail_wgs - 1) / tail_wgs : (1 << 20);
+        if (q < (1 << 20) && sk_tail_segments(q, k_tiles) <= kSkTailSegs) q_c = q;
       }
       if (nk1 > 0 && rq.skinny_pct < -kSkinnyMaxWgs) {
         // forced (tests, measurements); 0 = not possible: no skinny tiles
@@ -220,23 +221,38 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
         const int cus_x = rq.cus / 8;
         const bool may_split = spx > 0;
         const int F0 = (nl0 * n_tiles_n + 7) / 8, F1 = (nl1 * n_tiles_n + 7) / 8, T_x = (nk1 * n_tiles_n + 7) / 8;
-        int best = rounds_cost(F0, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts);
-        const int sk_tile = (k_tiles * rq.skinny_pct + 99) / 100 + 3;         // one skinny tile, in K steps
-        for (int n = 1; n <= kSkinnyMaxWgs && n * 4 <= cus_x && rq.sk_beside_ok; ++n) {
-          const int main_c = rounds_cost(F1, cus_x - n, k_tiles, rq.epi_cost, may_split, rq.max_parts);
+        // The candidates are priced together, one per lane (the prices are chains of integer divisions, and
+        // this wavefront is on the critical path of the launch): 0 = every row in 256-row tiles, 1 ..
+        // kSkinnyMaxWgs = that many workgroups per XCD beside them, then the launch of their own and the
+        // ranges inside the persistent launch.  The cheapest wins; of equals, the first in that order.
+        const int cand = lane & 7;
+        const int n = (cand >= 1 && cand <= kSkinnyMaxWgs) ? cand : 0;
+        int cost = rounds_cost(cand == 0 ? F0 : F1, cus_x - n, k_tiles, rq.epi_cost, may_split, rq.max_parts);
+        bool ok = cand <= kSkinnyMaxWgs + 2;
+        if (n > 0) {
+          const int sk_tile = (k_tiles * rq.skinny_pct + 99) / 100 + 3;       // one skinny tile, in K steps
           const int sk_c = (T_x + n - 1) / n * sk_tile;
-          const int c = main_c > sk_c ? main_c : sk_c;
-          if (c < best) { best = c; ns_wgs = n; }
+          cost = cost > sk_c ? cost : sk_c;
+          ok = n * 4 <= cus_x && rq.sk_beside_ok;
+        } else if (cand == kSkinnyMaxWgs + 1) {
+          cost += (q_c * kSkTailStepPct + 99) / 100 + kSkTailFixed;
+          ok = q_c > 0 && rq.sk_tail_ok;
+        } else if (cand == kSkinnyMaxWgs + 2) {
+          cost += (q_c * kSkInsideStepPct + 99) / 100 + kSkInsideFixed;
+          ok = q_c > 0 && rq.sk_beside_ok;
         }
-        if (q_c > 0) {
-          const int c = rounds_cost(F1, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts) +
-                        (q_c * kSkTailStepPct + 99) / 100 + kSkTailFixed;
-          if (rq.sk_tail_ok && c < best) { best = c; ns_wgs = 0; tail_q = q_c; tail_inside = 0; }
-          if (rq.sk_beside_ok) {
-            const int ci = rounds_cost(F1, cus_x, k_tiles, rq.epi_cost, may_split, rq.max_parts) +
-                           (q_c * kSkInsideStepPct + 99) / 100 + kSkInsideFixed;
-            if (ci < best) { best = ci; ns_wgs = 0; tail_q = q_c; tail_inside = 1; }
-          }
+        cost = cost < (1 << 26) ? cost : (1 << 26);
+        int key = ok ? (cost << 3) | cand : INT_MAX;
+#pragma unroll
+        for (int off = 4; off >= 1; off >>= 1) {
+          const int other = __shfl_xor(key, off, 64);
+          key = other < key ? other : key;
+        }
+        const int win = key & 7;                                   // candidate 0 is always there
+        ns_wgs = (win >= 1 && win <= kSkinnyMaxWgs) ? win : 0;
+        if (win > kSkinnyMaxWgs) {
+          tail_q = q_c;
+          tail_inside = win == kSkinnyMaxWgs + 2 ? 1 : 0;
         }
       }
     }
