@@ -183,9 +183,9 @@ def cpu_baseline(wl, max_seconds=30.0):
 
 
 def bench_backward(a, wl, ops):
-    """One training step of the layer: forward in grad mode (gate, FFN1, torch GELU, FFN2,
-    combine) and the backward of all of it, K times; then the two expert-GEMM backward calls
-    alone, with events around each."""
+    """One training step of the layer: forward in grad mode (gate, FFN1 with the GELU in its
+    epilogue and the pre-activation kept, FFN2, combine) and the backward of all of it, K times;
+    then the two expert-GEMM backward calls alone, with events around each."""
     import torch
     from ccfuser_amd.mix_moe import MixMOETransformerMLP
     t = wl.tensors
@@ -229,9 +229,11 @@ def bench_backward(a, wl, ops):
         gw1, gw2 = torch.empty_like(w1), torch.empty_like(w2)
         gb1 = torch.empty(E, f, dtype=torch.float16, device="cuda")
         gb2 = torch.empty(E, d, dtype=torch.float16, device="cuda")
-        calls = {"ffn2_backward": lambda: ops.ffn2_backward(gy, act, rt["dst_row"], rt["offsets"], n, w2, gw2, gb2),
+        drop = wl.capacity >= 0                          # without a capacity limit every output row is written: no zero fill
+        calls = {"ffn2_backward": lambda: ops.ffn2_backward(gy, act, rt["dst_row"], rt["offsets"], n, w2, gw2, gb2,
+                                                            may_drop=drop),
                  "ffn1_backward": lambda: ops.ffn1_backward(gh, x.detach(), rt["src_row"], rt["dst_row"],
-                                                            rt["offsets"], n, w1, n, gw1, gb1)}
+                                                            rt["offsets"], n, w1, n, gw1, gb1, may_drop=drop)}
         stage_ms = {}
         for name, fn in calls.items():
             for _ in range(max(2, W)):
