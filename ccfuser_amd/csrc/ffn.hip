@@ -621,12 +621,24 @@ __device__ __forceinline__ void skinny_reduce_block(const GroupedArgs &p, int t,
   float4v acc[C::TN];
 #pragma unroll
   for (int tn = 0; tn < C::TN; ++tn) acc[tn] = float4v{0, 0, 0, 0};
-  for (int w = w_lo; w <= w_hi; ++w) {
-    const int seg = t - (w * q) / KT;
-    const float4v *src = reinterpret_cast<const float4v *>(p.sk_partial) +
-                         static_cast<size_t>(w * kSkTailSegs + seg) * (C::TM * C::TN * 256) + (tm * C::TN) * 256 + tid;
+  // four partial tiles at a time: their loads leave together, the sums stay in K order
+  for (int w0 = w_lo; w0 <= w_hi; w0 += 4) {
+    float4v v[4][C::TN];
 #pragma unroll
-    for (int tn = 0; tn < C::TN; ++tn) acc[tn] += src[tn * 256];
+    for (int u = 0; u < 4; ++u) {
+      const int w = w0 + u <= w_hi ? w0 + u : w_hi;              // past the end: a copy that is not added
+      const int seg = t - (w * q) / KT;
+      const float4v *src = reinterpret_cast<const float4v *>(p.sk_partial) +
+                           static_cast<size_t>(w * kSkTailSegs + seg) * (C::TM * C::TN * 256) + (tm * C::TN) * 256 + tid;
+#pragma unroll
+      for (int tn = 0; tn < C::TN; ++tn) v[u][tn] = src[tn * 256];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (w0 + u <= w_hi) {
+#pragma unroll
+        for (int tn = 0; tn < C::TN; ++tn) acc[tn] += v[u][tn];
+      }
   }
   if (r >= rows) return;
   const int j = row0 + r;
@@ -1027,26 +1039,13 @@ grouped_gemm_tail_kernel(GroupedArgs p, int split_wgs) {
 }
 
 // out tile = sum of its S partial tiles (in part order) + bias, then the epilogue kEpi of the
-// grouped GEMM.  grid (kTailMaxTiles [+ kSkReduceX], BM / 16): block (t, q) with t < kTailMaxTiles
-// does tile rows 16q .. 16q+15 of tile slot t, a thread four rows of four columns; the blocks past
-// them reduce the skinny tiles that ran as a launch of their own.  It runs at the speed the partial tiles
-// stream back in (config 3, FFN2: 63 MB in 13 us).
+// grouped GEMM.  grid (kReduceX, BM / 16): block (x, q) does tile rows 16q .. 16q+15 of tile slots
+// x, x + kReduceX, ... of the split last round, a thread four rows of four columns, and then its share
+// of the (tile, row block) pairs of skinny tiles that were cut along K.  It runs at the speed the
+// partial tiles stream back in (config 3, FFN2: 63 MB in 13 us when its last round was split).
 template <class Cfg, int kEpi>
-__global__ void __launch_bounds__(256)
-splitk_reduce_kernel(GroupedArgs p) {
+__device__ __forceinline__ void reduce_split_tile(const GroupedArgs &p, int t, int S) {
   using R = RingFor<Cfg, false>;
-  if (blockIdx.x >= kTailMaxTiles) {
-    // the skinny tiles of a launch of their own: (tile, row block) pairs over the blocks past the split's
-    if (!p.skinny || p.skinny[3] <= 0) return;
-    const int pairs = p.skinny[0] * SkinnyCfg::TM;
-    const int nblk = (gridDim.x - kTailMaxTiles) * gridDim.y;
-    for (int i = (blockIdx.x - kTailMaxTiles) * gridDim.y + blockIdx.y; i < pairs; i += nblk)
-      skinny_reduce_block<kEpi>(p, i / SkinnyCfg::TM, i % SkinnyCfg::TM);
-    return;
-  }
-  const int tiles = p.tail[0], S = p.tail[1];
-  const int t = blockIdx.x;
-  if (t >= tiles) return;
   const int first_wg = (t & 7) + 8 * ((t >> 3) * S);   // workgroup id of part 0; part s is 8 s further
   const int4v ent = reinterpret_cast<const int4v *>(p.tail + 64)[first_wg];
   const int e = ent[0], row0 = ent[1], rows = ent[2], n0 = (ent[3] & 0xffff) * Cfg::BN;
@@ -1065,10 +1064,22 @@ splitk_reduce_kernel(GroupedArgs p) {
   for (int i = 0; i < 4; ++i) acc[i] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
   const int r_first = blockIdx.y * 16 + (threadIdx.x >> 6);
   const float *src = p.partial + static_cast<size_t>(first_wg) * (Cfg::BM * Cfg::BN) + r_first * Cfg::BN + 4 * c4;
-  for (int s = 0; s < S; ++s) {
+  // four parts at a time: their loads leave together, the sums stay in part order
+  for (int s0 = 0; s0 < S; s0 += 4) {
+    float4v v[4][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      acc[i] += *reinterpret_cast<const float4v *>(src + static_cast<size_t>(8 * s) * (Cfg::BM * Cfg::BN) + 4 * i * Cfg::BN);
+    for (int u = 0; u < 4; ++u) {
+      const int sp = s0 + u < S ? s0 + u : S - 1;                // past the end: a copy that is not added
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        v[u][i] = *reinterpret_cast<const float4v *>(src + static_cast<size_t>(8 * sp) * (Cfg::BM * Cfg::BN) + 4 * i * Cfg::BN);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (s0 + u < S) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += v[u][i];
+      }
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -1092,6 +1103,18 @@ splitk_reduce_kernel(GroupedArgs p) {
     *reinterpret_cast<half4 *>(p.C + crow * p.N + col) = o;
     if (kEpi == kEpiGeluKeep) *reinterpret_cast<half4 *>(p.C2 + static_cast<size_t>(j) * p.N + col) = pre;
   }
+}
+
+template <class Cfg, int kEpi>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(GroupedArgs p) {
+  const int tiles = p.tail[0], S = p.tail[1];
+  for (int t = blockIdx.x; t < tiles; t += gridDim.x) reduce_split_tile<Cfg, kEpi>(p, t, S);
+  if (!p.skinny || p.skinny[3] <= 0) return;
+  const int pairs = p.skinny[0] * SkinnyCfg::TM;
+  const int nblk = gridDim.x * gridDim.y;
+  for (int i = blockIdx.x * gridDim.y + blockIdx.y; i < pairs; i += nblk)
+    skinny_reduce_block<kEpi>(p, i / SkinnyCfg::TM, i % SkinnyCfg::TM);
 }
 
 // ---- kernel table -----------------------------------------------------------------
@@ -1140,7 +1163,7 @@ struct Launch {
   void (*persistent_gelu)(GroupedArgs, int);
 };
 constexpr int kPersistentMinKT = 4;
-constexpr int kSkReduceX = 32;       // x 16 blocks of the reduction launch for the skinny tiles
+constexpr int kReduceX = 32;         // x 16 blocks of the reduction launch
 
 const Launch kVariants[] = {// forward: "plain" = bias and row scale, "gelu" = bias and GELU
                             {Cfg5::BM, Cfg5::BN, Cfg5::THREADS, grouped_gemm_kernel<Cfg5, kEpiPlain>,
@@ -1331,10 +1354,8 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
                        dim3(v.threads), 0, stream, p, static_cast<int>(wgs / 8));
     if (split) {
       if (int rc = check_launch(what)) return rc;
-      // the skinny list may run as a launch of its own: `grid` more workgroups for it; whenever it may be cut
-      // along K (there or inside the persistent launch), more blocks in the reduction
+      // the skinny list may run as a launch of its own: `grid` more workgroups for it
       const bool sk = gs.req.sk_tail_ok;
-      const bool sk_cut = gs.skinny;
       if (!parts_inside || sk) {
         const int split_wgs = parts_inside ? 0 : grid;            // workgroups in front of the skinny list's
         const int tail_grid = split_wgs + (sk ? grid : 0);
@@ -1344,7 +1365,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
                                 stream, p, split_wgs);
         if (int rc = check_launch("grouped_gemm_tail_kernel")) return rc;
       }
-      const dim3 rgrid(kTailMaxTiles + (sk_cut ? kSkReduceX : 0), Cfg5::BM / 16);
+      const dim3 rgrid(kReduceX, Cfg5::BM / 16);
       if (epi == kEpiPlain) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiPlain>), rgrid, dim3(256), 0, stream, p);
       else if (epi == kEpiGelu) hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGelu>), rgrid, dim3(256), 0, stream, p);
       else hipLaunchKernelGGL((splitk_reduce_kernel<Cfg5, kEpiGeluKeep>), rgrid, dim3(256), 0, stream, p);
