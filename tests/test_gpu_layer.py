@@ -541,3 +541,52 @@ def test_fused_layer_random_shapes(T, d, f, E, k, cap, seed):
     if float(ref["out"].abs().mean()) > 1e-6:
         assert O.mean_rel_err(fused.cpu(), ref["out"]) <= MEAN_REL
     assert torch.equal(fused, _staged_forward(ops, args, E, k, cap))
+
+
+def _forced_plan_cases(count, seed):
+    g = torch.Generator().manual_seed(seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    modes = [(-6, 0), (-5, 1), (-1, 0), (-3, 0), (-6, 0), (1, 0), (-4, 0), (-6, 0)]
+    cases = []
+    for i in range(count):
+        E = ri(4, 24)
+        k = ri(1, 2)
+        T = ri(9000, 20000) // k
+        d, f = 256 * ri(2, 4), 256 * ri(2, 5)
+        skinny, sk_tail = modes[i % len(modes)]
+        cases.append((T, d, f, E, k, skinny, sk_tail, 9500 + i))
+    return cases
+
+
+@pytest.mark.parametrize("T,d,f,E,k,skinny,sk_tail,seed", _forced_plan_cases(8, 4321))
+def test_fused_layer_random_shapes_with_forced_plans(T, d, f, E, k, skinny, sk_tail, seed):
+    """Shapes large enough for the persistent launch (more worst-case tiles than CUs), drawn at
+    random, with the tile plan's choices forced in turn: skinny tiles beside the 256-row tiles,
+    cut along K inside the persistent launch or as a launch of their own, and the last round of
+    tiles cut along K (its parts inside the persistent launch) at every K.  Routing bit-exact,
+    whole output within the tolerance, a second call the same bits."""
+    from ccfuser_amd import ops
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).half()
+    x, wg, bg = r(T, d), r(E, d, sc=0.1), r(E, sc=0.1)
+    w1, b1, w2, b2 = r(E, f, d, sc=0.05), r(E, f, sc=0.1), r(E, d, f, sc=0.05), r(E, d, sc=0.1)
+    _say(f"forced plans T={T} d={d} f={f} E={E} k={k} skinny={skinny} skinny_tail={sk_tail}")
+    args = [a.cuda() for a in (x, wg, bg, w1, b1, w2, b2)]
+    ops.set_option("skinny", skinny)
+    ops.set_option("skinny_tail", sk_tail)
+    ops.set_option("split_tail", 2)
+    try:
+        fused, rt = ops.moe_forward(*args, k, -1, return_routing=True)
+        again = ops.moe_forward(*args, k, -1)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_option("skinny", 1)
+        ops.set_option("skinny_tail", 0)
+        ops.set_option("split_tail", 1)
+    ref = O.moe_layer_forward(x, wg, bg, w1, b1, w2, b2, k)
+    assert torch.equal(rt["idx"].cpu().view(-1), ref["idx_kept"].view(-1))
+    assert torch.equal(rt["offsets"].cpu().long(), ref["offsets"].long())
+    ma, mr = O.max_abs_err(fused.cpu(), ref["out"]), O.mean_rel_err(fused.cpu(), ref["out"])
+    _say(f"  counts={ref['counts'].tolist()} max_abs={ma:.3e} mean_rel={mr:.3e}")
+    assert ma <= MAX_ABS and mr <= MEAN_REL
+    assert torch.equal(fused, again)
