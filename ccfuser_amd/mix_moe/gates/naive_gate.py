@@ -8,6 +8,16 @@ from ... import ops
 from .base_gate import BaseGate
 
 
+_ZEROS = {}
+
+
+def _zero_on(device):
+    z = _ZEROS.get(device)
+    if z is None:
+        z = _ZEROS[device] = torch.zeros(1, device=device)
+    return z
+
+
 class _GateFunction(torch.autograd.Function):
     """The fused gate kernel with the backward autograd derives for the reference's
     linear -> topk -> softmax (naive_gate.py:31-38): softmax over the k selected
@@ -72,8 +82,9 @@ class NaiveGate(BaseGate):
         res = _GateFunction.apply(x, self.gate.weight, self.gate.bias, self.top_k, bool(return_all_scores))
         idx = res[0].view(*lead, self.top_k)
         score = res[1]                                   # [(B*L), top_k], as the reference returns it
-        # dummy loss, on the input's device (naive_gate.py:41)
-        self.set_loss(torch.zeros(1, requires_grad=True, device=inp.device))
+        # dummy loss, on the input's device (naive_gate.py:41): a fresh leaf over a zero made once per
+        # device, so that the forward pays no fill kernel for it
+        self.set_loss(_zero_on(inp.device).detach().requires_grad_(True))
         if return_all_scores:
             return idx, score, res[2].view(*lead, self.tot_expert)
         return idx, score

@@ -104,6 +104,10 @@ def test_mirrored_module_staged_equals_fused(workloads):
     assert O.mean_rel_err(fused.view(-1, d).cpu(), ref["out"]) <= MEAN_REL
     # the reference's block arrays, produced on demand, tile every segment
     pos, score, infos = mlp.async_expert_assign.process_data(mlp.gate, x.view(-1, d), E, 1)
+    # the gate leaves the reference's dummy loss (naive_gate.py:41): a zero on the input's device that takes a gradient
+    assert mlp.gate.has_loss
+    loss = mlp.gate.get_loss()
+    assert loss.is_cuda and loss.requires_grad and loss.is_leaf and float(loss) == 0.0 and not mlp.gate.has_loss
     lens, starts, ids = (infos[n].cpu().tolist() for n in ("lens", "start_addrs", "expert_ids"))
     off = infos["offsets"].cpu().tolist()
     covered = sorted((s, s + l) for s, l in zip(starts, lens))
