@@ -107,7 +107,7 @@ def test_mirrored_module_staged_equals_fused(workloads):
     # the gate leaves the reference's dummy loss (naive_gate.py:41): a zero on the input's device that takes a gradient
     assert mlp.gate.has_loss
     loss = mlp.gate.get_loss()
-    assert loss.is_cuda and loss.requires_grad and loss.is_leaf and float(loss) == 0.0 and not mlp.gate.has_loss
+    assert loss.is_cuda and loss.requires_grad and loss.is_leaf and float(loss.detach()) == 0.0 and not mlp.gate.has_loss
     lens, starts, ids = (infos[n].cpu().tolist() for n in ("lens", "start_addrs", "expert_ids"))
     off = infos["offsets"].cpu().tolist()
     covered = sorted((s, s + l) for s, l in zip(starts, lens))
