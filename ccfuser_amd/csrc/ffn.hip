@@ -1232,7 +1232,7 @@ constexpr int kEpiCostGelu = 9, kEpiCostPlain = 5;
 
 struct GemmSetup {
   const Launch *v;
-  bool second, split, skinny;
+  bool second, split, skinny, cut;
   int32_t *skinny_list;
   int grid;
   long long wgs;
@@ -1276,10 +1276,13 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
   // remainder rows as skinny tiles: forward epilogues of the persistent 256 x 256 kernel (either weight layout)
   g.skinny = opt.skinny_pct != 0 && (b_kn ? epi == kEpiPlain && N % 256 == 0 : epi <= kEpiGeluKeep) && g.grid >= 64 && g.grid <= g.wgs &&
              v.bm == Cfg5::BM && v.bn == Cfg5::BN && v.persistent_plain && (!wide || g.split);
+  // skinny tiles may be cut along K (partial tiles in the split scratch, summed by the reduction launch) at any K,
+  // also where the last round of 256-row tiles is not split
+  g.cut = g.skinny && !wide && g.grid <= kTailMaxParts;
   g.skinny_list = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.plan) + plan_core_bytes(max_rows, E, N > K ? N : K));
   g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, opt.split_max_parts, g.plan,
-                  g.split ? g.tail : nullptr, g.skinny ? g.skinny_list : nullptr, g.grid,
-                  gelu ? kEpiCostGelu : kEpiCostPlain, opt.skinny_pct, g.split && g.skinny && opt.skinny_tail, !wide};
+                  (g.split || g.cut) ? g.tail : nullptr, g.skinny ? g.skinny_list : nullptr, g.grid,
+                  gelu ? kEpiCostGelu : kEpiCostPlain, opt.skinny_pct, g.cut && opt.skinny_tail, !wide};
   return g;
 }
 
@@ -1352,12 +1355,12 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
     p.tail_inside = parts_inside ? 1 : 0;
     hipLaunchKernelGGL(second ? v.persistent_gelu : v.persistent_plain, dim3(static_cast<unsigned>(g)),
                        dim3(v.threads), 0, stream, p, static_cast<int>(wgs / 8));
-    if (split) {
+    if (split || gs.cut) {
       if (int rc = check_launch(what)) return rc;
       // the skinny list may run as a launch of its own: `grid` more workgroups for it
       const bool sk = gs.req.sk_tail_ok;
-      if (!parts_inside || sk) {
-        const int split_wgs = parts_inside ? 0 : grid;            // workgroups in front of the skinny list's
+      if ((split && !parts_inside) || sk) {
+        const int split_wgs = (split && !parts_inside) ? grid : 0;  // workgroups in front of the skinny list's
         const int tail_grid = split_wgs + (sk ? grid : 0);
         if (b_kn) hipLaunchKernelGGL((grouped_gemm_tail_kernel<Cfg5, true>), dim3(tail_grid), dim3(Cfg5::THREADS), 0,
                                      stream, p, split_wgs);
@@ -1792,7 +1795,7 @@ extern "C" int ccf_ffn_plan_info(const void *workspace, int max_rows, int num_ex
   for (int i = 0; i < 8; ++i) info[i] = 0;
   hipStream_t st = as_stream(stream);
   hipError_t e = hipSuccess;
-  if (gs.split) e = hipMemcpyAsync(info, gs.tail, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, st);
+  if (gs.split || gs.cut) e = hipMemcpyAsync(info, gs.tail, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, st);
   int32_t where = 0;
   if (gs.skinny && e == hipSuccess) e = hipMemcpyAsync(info + 2, gs.skinny_list, 4 * sizeof(int32_t), hipMemcpyDeviceToHost, st);
   if (gs.skinny && e == hipSuccess) e = hipMemcpyAsync(&where, gs.skinny_list + 4, sizeof(int32_t), hipMemcpyDeviceToHost, st);

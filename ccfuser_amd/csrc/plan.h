@@ -45,7 +45,8 @@ constexpr size_t kTailBytes = kTailHead + kSplitPartialBytes + kSkTailBytes;
 // costs a CU as much as a full one: its K steps are paced by the tile loads, not by the MFMAs
 // it skips.  With a skinny list in the plan request, a remainder of at most kSkinnyRows rows
 // (rows % BM, or all rows of an expert smaller than that) may leave the plan of 256-row tiles
-// and become one entry per N tile of a second list.  A few workgroups per XCD of the persistent
+// and become one entry per N tile of a second list; a remainder of up to twice that may become
+// two (the plan prices both limits and takes the cheaper).  A few workgroups per XCD of the persistent
 // kernel (ffn.hip) then do nothing but those entries, as 64 x 256 tiles that stream their
 // weight panel through a deep LDS pipeline: little arithmetic, mostly memory latency, so they
 // run beside the compute-bound 256-row tiles on bandwidth those leave idle.  Whether that pays
@@ -70,10 +71,16 @@ constexpr size_t kTailBytes = kTailHead + kSplitPartialBytes + kSkTailBytes;
 //   [5] most 256-row tiles a workgroup of the persistent launch runs     [6..7] unused
 //   [kSkinnyHead + 4 i ...] entry i < T: {expert, first sorted row, rows (1..kSkinnyRows), N tile}
 constexpr int kSkinnyRows = 64;
+// Skinny M tiles of a remainder of r rows when remainders up to `limit` rows (kSkinnyRows or twice that) leave the
+// 256-row tiles.
+__host__ __device__ inline int skinny_m_tiles(int r, int limit) {
+  return (r > 0 && r <= limit) ? (r + kSkinnyRows - 1) / kSkinnyRows : 0;
+}
 constexpr int kSkinnyMaxWgs = 4;                     // per XCD
 constexpr int kSkinnyHead = 8;                       // header integers in front of the entries
 __host__ __device__ inline size_t skinny_ints(int max_rows, int E, int n_tiles_n) {
-  const int most = E < max_rows ? E : max_rows;      // at most one skinny M tile per expert
+  const int by_rows = (max_rows + kSkinnyRows - 1) / kSkinnyRows;
+  const int most = 2 * E < by_rows ? 2 * E : by_rows;  // at most two skinny M tiles per expert
   return kSkinnyHead + 4 * static_cast<size_t>(most > 0 ? most : 0) * n_tiles_n;
 }
 
@@ -180,27 +187,41 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   __shared__ int s_ns;             // workgroups per XCD given to skinny tiles (0: none)
   __shared__ int s_tail_q;         // > 0: skinny tiles cut along K, K steps per workgroup
   __shared__ int s_tail_inside;    // 1: inside the persistent launch, 0: as a launch of their own
+  __shared__ int s_sk_limit;       // remainders of at most this many rows are skinny
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
     // Skinny tiles or not: tile counts both ways, then the cheaper plan by the model above.
-    int ns_wgs = 0, tail_q = 0, tail_inside = 0;
+    int ns_wgs = 0, tail_q = 0, tail_inside = 0, sk_limit = kSkinnyRows;
     if (skinny && rq.skinny_pct != 0 && rq.cus >= 64) {
-      int nl0 = 0, nl1 = 0, nk1 = 0;                // 256-row tiles without / with skinny tiles, skinny M tiles
+      // 256-row tiles without skinny tiles; with them, and the skinny M tiles, for both limits on a remainder
+      int nl0 = 0, nl1 = 0, nk1 = 0, nl2 = 0, nk2 = 0;
       for (int e = lane; e < E; e += 64) {
         int cnt = s_off[e + 1] - s_off[e];
         cnt = cnt > 0 ? cnt : 0;
         const int nt = (cnt + BM - 1) / BM, r = cnt % BM;
-        const int sk = (r > 0 && r <= kSkinnyRows) ? 1 : 0;
+        const int sk1 = skinny_m_tiles(r, kSkinnyRows), sk2 = skinny_m_tiles(r, 2 * kSkinnyRows);
         nl0 += nt;
-        nl1 += nt - sk;
-        nk1 += sk;
+        nl1 += nt - (sk1 ? 1 : 0);
+        nk1 += sk1;
+        nl2 += nt - (sk2 ? 1 : 0);
+        nk2 += sk2;
       }
 #pragma unroll
       for (int off = 32; off >= 1; off >>= 1) {
         nl0 += __shfl_xor(nl0, off, 64);
         nl1 += __shfl_xor(nl1, off, 64);
         nk1 += __shfl_xor(nk1, off, 64);
+        nl2 += __shfl_xor(nl2, off, 64);
+        nk2 += __shfl_xor(nk2, off, 64);
       }
+      // candidates 8 .. 15 (below) are candidates 0 .. 7 with the larger limit; forced modes take the larger
+      // limit when it gives more skinny tiles (the same answer in every lane)
+      const bool wide = rq.skinny_pct < 0 ? nk2 > nk1 : ((lane >> 3) & 1) != 0;
+      if (wide) {
+        nl1 = nl2;
+        nk1 = nk2;
+      }
+      const int my_limit = wide ? 2 * kSkinnyRows : kSkinnyRows;
       // the launch of their own: possible when the caller launches the split kernels and a
       // workgroup's range stays within kSkTailSegs tiles
       const int tail_wgs = rq.cus < kSkTailMaxWgs ? rq.cus : kSkTailMaxWgs;
@@ -211,52 +232,56 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
         const int q = steps < (1ll << 30) ? (static_cast<int>(steps) + tail_wgs - 1) / tail_wgs : (1 << 20);
         if (q < (1 << 20) && sk_tail_segments(q, k_tiles) <= kSkTailSegs) q_c = q;
       }
+      if (rq.skinny_pct < 0) sk_limit = my_limit;     // uniform: every lane took the same limit
       if (nk1 > 0 && rq.skinny_pct < -kSkinnyMaxWgs) {
         // forced (tests, measurements); 0 = not possible: no skinny tiles
         tail_inside = rq.skinny_pct == -kSkinnyMaxWgs - 2;
         tail_q = (tail_inside ? rq.sk_beside_ok : rq.sk_tail_ok) ? q_c : 0;
       } else if (nk1 > 0 && rq.skinny_pct < 0) {
         ns_wgs = rq.sk_beside_ok ? -rq.skinny_pct : 0; // forced
-      } else if (nk1 > 0) {
+      } else if (rq.skinny_pct > 0) {
         const int cus_x = rq.cus / 8;
         const bool may_split = spx > 0;
         const int F0 = (nl0 * n_tiles_n + 7) / 8, F1 = (nl1 * n_tiles_n + 7) / 8, T_x = (nk1 * n_tiles_n + 7) / 8;
         // The candidates are priced together, one per lane (the prices are chains of integer divisions, and
         // this wavefront is on the critical path of the launch): 0 = every row in 256-row tiles, 1 ..
         // kSkinnyMaxWgs = that many workgroups per XCD beside them, then the launch of their own and the
-        // ranges inside the persistent launch.  The cheapest wins; of equals, the first in that order.
+        // ranges inside the persistent launch; 8 .. 15 the same with remainders of up to twice kSkinnyRows
+        // rows as skinny tiles.  The cheapest wins; of equals, the first in that order.
         const int cand = lane & 7;
         const int n = (cand >= 1 && cand <= kSkinnyMaxWgs) ? cand : 0;
         int cost = rounds_cost(cand == 0 ? F0 : F1, cus_x - n, k_tiles, rq.epi_cost, may_split, rq.max_parts);
-        bool ok = cand <= kSkinnyMaxWgs + 2;
+        bool ok = cand <= kSkinnyMaxWgs + 2 && (cand == 0 || nk1 > 0);
         if (n > 0) {
           const int sk_tile = (k_tiles * rq.skinny_pct + 99) / 100 + 3;       // one skinny tile, in K steps
           const int sk_c = (T_x + n - 1) / n * sk_tile;
           cost = cost > sk_c ? cost : sk_c;
-          ok = n * 4 <= cus_x && rq.sk_beside_ok;
+          ok = ok && n * 4 <= cus_x && rq.sk_beside_ok;
         } else if (cand == kSkinnyMaxWgs + 1) {
           cost += (q_c * kSkTailStepPct + 99) / 100 + kSkTailFixed;
-          ok = q_c > 0 && rq.sk_tail_ok;
+          ok = ok && q_c > 0 && rq.sk_tail_ok;
         } else if (cand == kSkinnyMaxWgs + 2) {
           cost += (q_c * kSkInsideStepPct + 99) / 100 + kSkInsideFixed;
-          ok = q_c > 0 && rq.sk_beside_ok;
+          ok = ok && q_c > 0 && rq.sk_beside_ok;
         }
         cost = cost < (1 << 26) ? cost : (1 << 26);
-        int key = ok ? (cost << 3) | cand : INT_MAX;
+        int key = ok ? (cost << 4) | (lane & 15) : INT_MAX;
 #pragma unroll
-        for (int off = 4; off >= 1; off >>= 1) {
+        for (int off = 8; off >= 1; off >>= 1) {
           const int other = __shfl_xor(key, off, 64);
           key = other < key ? other : key;
         }
-        const int win = key & 7;                                   // candidate 0 is always there
+        const int win16 = key & 15, win = win16 & 7;               // candidate 0 is always there
+        const int q_win = __shfl(q_c, win16, 64);
+        sk_limit = (win16 >> 3) ? 2 * kSkinnyRows : kSkinnyRows;
         ns_wgs = (win >= 1 && win <= kSkinnyMaxWgs) ? win : 0;
         if (win > kSkinnyMaxWgs) {
-          tail_q = q_c;
+          tail_q = q_win;
           tail_inside = win == kSkinnyMaxWgs + 2 ? 1 : 0;
         }
       }
     }
-    if (lane == 0) { s_ns = ns_wgs; s_tail_q = tail_q; s_tail_inside = tail_inside; }
+    if (lane == 0) { s_ns = ns_wgs; s_tail_q = tail_q; s_tail_inside = tail_inside; s_sk_limit = sk_limit; }
     int carry_l = 0, carry_s = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
@@ -266,8 +291,8 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       int ns, nl;
       if (ns_wgs || tail_q) {
         const int r = cnt % BM;                                   // ns counts skinny M tiles here
-        ns = (r > 0 && r <= kSkinnyRows) ? 1 : 0;
-        nl = nt - ns;
+        ns = skinny_m_tiles(r, sk_limit);
+        nl = nt - (ns ? 1 : 0);
       } else {
         ns = (nt == 1 && cnt <= BM / 2) ? 1 : 0;                  // a short tile only when it is the expert's only one
         nl = nt - ns;
@@ -403,7 +428,11 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     if (ns && use_skinny) {
       int4v *sk = reinterpret_cast<int4v *>(skinny + kSkinnyHead);
       const int first_s = s_short[e] * n_tiles_n;
-      for (int tn = lane; tn < n_tiles_n; tn += 64) sk[first_s + tn] = int4v{e, lo + cnt_long, cnt - cnt_long, tn};
+      for (int m = 0; m < ns; ++m) {                             // one or two skinny M tiles
+        const int r0 = cnt_long + m * kSkinnyRows;
+        const int rows = (cnt - r0) < kSkinnyRows ? (cnt - r0) : kSkinnyRows;
+        for (int tn = lane; tn < n_tiles_n; tn += 64) sk[first_s + m * n_tiles_n + tn] = int4v{e, lo + r0, rows, tn};
+      }
     } else if (ns) {
       const int i = nl;                                          // the expert's last M tile
       const int first_s = s_short[e] * n_tiles_n;

@@ -62,9 +62,10 @@ const char *ccf_last_error(void);
  *   "split_tail"      0 = off, 1 = default, n > 1 = for K of n*64 and more: the tiles of a launch's
  *                     last, partly filled round are cut along K and reduced by a second kernel
  *   "split_parts"     2..8 (default 8): most parts such a tile is cut into
- *   "skinny"          0 = off, 1 = default: rows an expert has beyond its full 256-row tiles (at most 64)
- *                     may run as 64-row tiles in a few workgroups set aside for them, when the tile plan's
- *                     cost model says that beats a padded 256-row tile; n > 1 sets the model's cost of
+ *   "skinny"          0 = off, 1 = default: rows an expert has beyond its full 256-row tiles (at most 128:
+ *                     one or two tiles of 64 rows) may run as 64-row tiles in a few workgroups set aside
+ *                     for them or cut along K over all workgroups, when the tile plan's cost model says
+ *                     that beats a padded 256-row tile; n > 1 sets the model's cost of
  *                     such a tile's K step in percent of a 256-row tile's (default 70); -n (1..4) forces
  *                     them with n workgroups per XCD; -5 forces them as a launch of their own behind the
  *                     persistent kernel, cut along K over all workgroups (the model's third choice); -6 forces

@@ -565,7 +565,7 @@ def test_split_k_tail_all_epilogues():
 # CUs ((ceil(R / 256) + E) * ceil(N / 256) >= 256): only then does the persistent launch set
 # workgroups aside for skinny tiles.  `expect`: which GEMMs must report skinny tiles actually run.
 @pytest.mark.parametrize("R,d,f,E,skew,seed,mode,expect", [
-    (8192, 4096, 4096, 6, False, 31, 1, ""),          # remainders of ~80 rows: above 64, stay in 256-row tiles
+    (8192, 4096, 4096, 6, False, 31, 1, ""),          # remainders of 56..122 rows: one or two skinny tiles each, if the plan wants them
     (8192 + 6 * 200, 4096, 4096, 6, False, 35, 1, ""),   # remainders of ~25 rows, long K: the plan's own choice
     (0, 256, 1024, 60, False, 32, -2, "1"),           # first GEMM with K = 256: four K tiles, the shortest the loop takes
     (2100, 1024, 2048, 70, True, 33, -1, "12"),       # most experts are nothing but a skinny tile, some are empty
@@ -653,7 +653,8 @@ def test_skinny_tiles(R, d, f, E, skew, seed, mode, expect):
         assert O.max_abs_err(y, y_ref) <= MAX_ABS and O.mean_rel_err(y, y_ref) <= MEAN_REL, m
     same = [torch.equal(a, b) for a, b in zip(res[mode], res[0])]
     _say(f"  skinny on/off bitwise equal (h, act, pre, y): {same}")
-    if mode <= -5:
+    cut = any(info[mode, which]["skinny_tail_steps"] != 0 for which in (1, 2))   # the plan's own choice may be a K cut too
+    if mode <= -5 or cut:
         # another summation order: close, and not identical where skinny tiles ran
         for a, b in zip(res[mode], res[0]):
             assert O.max_abs_err(a, b.float()) <= MAX_ABS
