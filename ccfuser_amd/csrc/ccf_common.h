@@ -55,7 +55,7 @@ int gate_forward(const void *x, const void *wg, const void *bg, int tokens, int 
                  int32_t *wg_cnt, long long max_cnt, int *tokens_per_wg);
 
 // tuning knobs set through ccf_set_option()
-extern int g_gate_waves, g_gate_slots;   // gate.hip
+extern int g_gate_waves, g_gate_slots, g_gate_stream;   // gate.hip
 extern int g_route_rows_max;             // route.hip
 
 }  // namespace ccf

@@ -1678,6 +1678,11 @@ extern "C" int ccf_set_option(const char *name, int value) {
     g_gate_waves = value;
     return CCF_OK;
   }
+  if (!strcmp(name, "gate_stream")) {
+    CCF_REQUIRE(value >= -1 && value <= 1, CCF_ERR_ARG, "set_option: gate_stream %d outside -1..1", value);
+    g_gate_stream = value;
+    return CCF_OK;
+  }
   if (!strcmp(name, "fused_combine")) {
     g_fused_combine = value != 0;
     return CCF_OK;

@@ -25,10 +25,12 @@
 #include "mfma_f32.h"
 
 #include <limits.h>
+#include <type_traits>
 
 namespace ccf {
 int g_gate_waves = 8;    // most wavefronts of a gate workgroup (each takes other parts of K), 1..8
 int g_gate_slots = 0;    // parts of K a wavefront works on at a time (1, 2, 4); 0 = by the token count
+int g_gate_stream = -1;  // 1: every wavefront takes its tokens through all of K alone; 0: never; -1: with many tokens
 namespace {
 
 constexpr int kMaxTopK = 8;
@@ -57,28 +59,27 @@ struct Best {
     }
   }
   __device__ inline void offer(float nv, int nid, int k) {
-    float lv = v[0];
-    int li = id[0];
+    if constexpr (KS > 2) {                        // long lists: most offers end at the last kept entry
+      float lv = v[0];
+      int li = id[0];
 #pragma unroll
-    for (int s = 1; s < KS; ++s)
-      if (s == k - 1) {
-        lv = v[s];
-        li = id[s];
-      }
-    if (!better(nv, nid, lv, li)) return;          // not among the k best
+      for (int s = 1; s < KS; ++s)
+        if (s == k - 1) {
+          lv = v[s];
+          li = id[s];
+        }
+      if (!better(nv, nid, lv, li)) return;        // not among the k best
+    }
+    bool beats[KS];                                // short lists: no branch
+#pragma unroll
+    for (int s = 0; s < KS; ++s) beats[s] = better(nv, nid, v[s], id[s]);
 #pragma unroll
     for (int s = KS - 1; s >= 0; --s) {
       if (s < k) {
         const int up = s > 0 ? s - 1 : 0;
-        const bool ahead = s > 0 && better(nv, nid, v[up], id[up]);
-        const bool here = better(nv, nid, v[s], id[s]);
-        if (ahead) {                               // belongs further up: slot s takes its upper neighbour
-          v[s] = v[up];
-          id[s] = id[up];
-        } else if (here) {
-          v[s] = nv;
-          id[s] = nid;
-        }
+        const bool ahead = s > 0 && beats[up];     // belongs further up: slot s takes its upper neighbour
+        v[s] = ahead ? v[up] : (beats[s] ? nv : v[s]);
+        id[s] = ahead ? id[up] : (beats[s] ? nid : id[s]);
       }
     }
   }
@@ -282,15 +283,26 @@ gate_mfma_kernel(const half_t *__restrict__ x, const half_t *__restrict__ wg, co
         }
       }
       __syncthreads();
-      // running sums: the parts of this round in ascending order
+      // running sums: the parts of this round in ascending order.  The part sums are read
+      // eight at a time ahead of the additions, which stay one chain in part order.
+      int np_round = nparts - rd * per_round;
+      np_round = np_round < per_round ? np_round : per_round;
       for (int i = threadIdx.x; i < TW * N; i += blockDim.x) {
         const int tok = i / N, col = i % N;
         float t = rd == 0 ? 0.0f : s_total[tok * kLd + col];
-        for (int q = 0; q < per_round; ++q) {
-          const int p = rd * per_round + q;
-          if (p >= nparts) break;
-          const float ps = s_mem[static_cast<size_t>(q >> LS) * kRegionFloats + (q & (S - 1)) * TW * N + i];
-          t = p == 0 ? ps : t + ps;
+        for (int q0 = 0; q0 < np_round; q0 += 8) {
+          float ps[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            int q = q0 + u;
+            q = q < np_round ? q : np_round - 1;
+            ps[u] = s_mem[static_cast<size_t>(q >> LS) * kRegionFloats + (q & (S - 1)) * TW * N + i];
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const float sum = (rd == 0 && q0 + u == 0) ? ps[u] : t + ps[u];   // the first part starts the chain
+            t = q0 + u < np_round ? sum : t;
+          }
         }
         if (rd == rounds - 1) {
           const int e = e0 + col;
@@ -309,7 +321,15 @@ gate_mfma_kernel(const half_t *__restrict__ x, const half_t *__restrict__ wg, co
     if (threadIdx.x < TW && t0 + threadIdx.x < tokens) {
       const float *lg = s_total + threadIdx.x * kLd;
       const int ne = (E - e0) < N ? (E - e0) : N;
-      for (int c = 0; c < ne; ++c) best.offer(lg[c], e0 + c, k);
+#pragma unroll
+      for (int c0 = 0; c0 < N; c0 += 8) {          // eight logits read ahead of their offers
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = lg[c0 + u];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (c0 + u < ne) best.offer(v[u], e0 + c0 + u, k);
+      }
     }
     // s_total is next written after the next tile's first barrier, which these threads reach later
   }
@@ -323,6 +343,252 @@ gate_mfma_kernel(const half_t *__restrict__ x, const half_t *__restrict__ wg, co
     for (int e = threadIdx.x; e < E; e += blockDim.x) row[e] = 0;
     __syncthreads();
     if (threadIdx.x < TW && t0 + threadIdx.x < tokens) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        if (s < k) atomicAdd(&row[best.id[s]], 1);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) wg_cnt[static_cast<size_t>(blockIdx.x) * E + e] = row[e];
+  }
+}
+
+// fp16 gate for many tokens: every wavefront works alone.  It takes TW tokens through all of
+// K, S parts at a time ("round": 4 stages), in one unbroken stream of stages: the loads run
+// five stages ahead of the MFMAs in four sets of registers, each set parked in the
+// wavefront's LDS one stage ahead of its use, so after the first arrival the matrix pipe
+// does not wait for memory again.  At the end of a round the part sums, which are registers
+// of this lane, go onto the running sums in ascending part order; the logits of a tile of N
+// experts pass through the wavefront's LDS once, for the selection (one lane per token) and
+// the coalesced write.  No barrier before the expert counts of the workgroup.
+constexpr int kStreamWaves = 4;
+
+template <int N, int LS, int KS>
+__global__ void __launch_bounds__(kStreamWaves * 64)
+gate_stream_kernel(const half_t *__restrict__ x, const half_t *__restrict__ wg, const half_t *__restrict__ bg,
+                   int tokens, int d, int E, int k, int64_t *__restrict__ idx_out,
+                   half_t *__restrict__ score_out, half_t *__restrict__ logits_out, int32_t *__restrict__ wg_cnt) {
+  using M = Mfma<N>;
+  constexpr int kBlocks = 64 / N;
+  constexpr int S = 1 << LS;
+  static_assert(S <= kBlocks, "a slot is a block");
+  constexpr int TB = kBlocks / S;                  // token blocks of a wavefront
+  constexpr int TW = TB * N;                       // its tokens
+  constexpr int RB = M::kRegs / kBlocks;           // accumulator registers of a block
+  constexpr int kWLoads = N * S / 16;
+  constexpr int kLd = N + 1;
+  static_assert(TW * kLd <= kRegionFloats, "the logits of a tile fit the wavefront's region");
+  extern __shared__ float s_mem[];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  float *region = s_mem + static_cast<size_t>(wave) * kRegionFloats;
+  const int t0 = (blockIdx.x * kStreamWaves + wave) * TW;
+  const int nparts = (d + kPart - 1) / kPart;
+  const int rounds = (nparts + S - 1) / S;
+  const bool ragged = d % (S * kPart) != 0;        // the last round has K elements to leave out
+
+  const int blk = lane / N, r = lane % N;
+  const int slot = blk & (S - 1);
+  char *tile = reinterpret_cast<char *>(region);
+  const char *my_x = tile + lane * kRowBytes;
+  const char *my_w = tile + kTileBytes + (slot * N + r) * kRowBytes;
+  const int l_row = lane >> 2, l_piece = lane & 3;
+  char *park_at = tile + l_row * kRowBytes + l_piece * 16;
+
+  Best<KS> best;
+  best.clear();
+  if (t0 < tokens) {                               // uniform per wavefront
+    const half_t *x_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int lr = 16 * i + l_row;
+      int t = t0 + ((lr / N) >> LS) * N + lr % N;
+      t = t < tokens ? t : tokens - 1;
+      x_src[i] = x + static_cast<size_t>(t) * d + (((lr / N) & (S - 1)) * kPart + l_piece * 8);
+    }
+    for (int e0 = 0; e0 < E; e0 += N) {
+      // columns past the last expert repeat its weights; nothing reads their logits
+      const bool has_w = e0 + r < E;
+      float my_bias = 0.0f;
+      if (bg && has_w) my_bias = static_cast<float>(bg[e0 + r]);
+      const half_t *w_src[kWLoads];
+#pragma unroll
+      for (int i = 0; i < kWLoads; ++i) {
+        const int wr = 16 * i + l_row;
+        int e = e0 + wr % N;
+        e = e < E ? e : E - 1;
+        w_src[i] = wg + static_cast<size_t>(e) * d + ((wr / N) * kPart + l_piece * 8);
+      }
+      // stage g of the stream: round g / 4, K offset of the round's first part + (g % 4) * kStageK
+      auto stage_k = [&](int g) { return (g >> 2) * (S * kPart) + (g & 3) * kStageK; };
+      typedef int4v XSet[4];
+      typedef int4v WSet[kWLoads];
+      XSet xa, xb, xc, xd;
+      WSet wa, wb, wc, wd;
+      auto fetch = [&](int g, XSet &xv, WSet &wv) {   // past the end of K the loads read the start of x and wg
+        const int ks = stage_k(g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kx = ks + (((16 * i + l_row) / N) & (S - 1)) * kPart + l_piece * 8;
+          xv[i] = *reinterpret_cast<const int4v *>(kx < d ? x_src[i] + ks : x);
+        }
+#pragma unroll
+        for (int i = 0; i < kWLoads; ++i) {
+          const int kw = ks + ((16 * i + l_row) / N) * kPart + l_piece * 8;
+          wv[i] = *reinterpret_cast<const int4v *>(kw < d ? w_src[i] + ks : wg);
+        }
+      };
+      auto park = [&](const XSet &xv, const WSet &wv) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<int4v *>(park_at + 16 * i * kRowBytes) = xv[i];
+#pragma unroll
+        for (int i = 0; i < kWLoads; ++i)
+          *reinterpret_cast<int4v *>(park_at + kTileBytes + 16 * i * kRowBytes) = wv[i];
+      };
+      auto take = [&](int c, half8 &vx, half8 &vw) {
+        vx = *reinterpret_cast<const half8 *>(my_x + c * 16);
+        vw = *reinterpret_cast<const half8 *>(my_w + c * 16);
+      };
+      typename M::Acc acc;
+      // A piece is 8 K elements of a stage.  Its MFMAs run on fp32 copies made during the piece
+      // before, in registers that no MFMA in flight reads: a conversion into a register that the
+      // running MFMA still reads waits for that MFMA, and one wavefront per SIMD has nothing to
+      // cover the wait with.
+      auto convert = [&](auto rag, int g, int c, const half8 &vx, const half8 &vw, float (&fx)[8], float (&fw)[8]) {
+        half8 xs = vx, ws = vw;
+        if constexpr (decltype(rag)::value) {      // K ends inside a round: what lies past it counts as zero
+          const bool in = stage_k(g) + slot * kPart + c * 8 < d;
+          const half8 zero = {};
+          xs = in ? vx : zero;
+          ws = in ? vw : zero;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          fx[j] = static_cast<float>(xs[j]);
+          fw[j] = static_cast<float>(ws[j]);
+        }
+      };
+      auto mma = [&](const float (&fx)[8], const float (&fw)[8]) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc = M::run(fx[j], fw[j], acc);
+      };
+      float total[TB * RB];
+      half8 ax, aw, bx, bw;                        // pieces as read from LDS: even ones in a, odd ones in b
+      float fax[8], faw[8], fbx[8], fbw[8];        // their fp32 copies
+      // eight MFMAs with the next piece's conversions between them
+#define CCF_GATE_PIECE(MMA_F, G, C, RAW, CONV_F)                       \
+  do {                                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+    mma(MMA_F##x, MMA_F##w);                                           \
+    convert(rag, G, C, RAW##x, RAW##w, CONV_F##x, CONV_F##w);          \
+    _Pragma("unroll") for (int q_ = 0; q_ < 8; ++q_) {                 \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               \
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);               \
+    }                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+  } while (0)
+      // One stage, entered with piece 0 converted (fa) and piece 1 read (b).  Reads from LDS
+      // run two pieces ahead, conversions one; the next stage is parked once this stage's last
+      // read is on its way (the LDS works in order), and its first pieces are read behind that.
+#define CCF_GATE_STAGE(g, PARK_NEXT)                                   \
+  do {                                                                 \
+    take(2, ax, aw);                                                   \
+    CCF_GATE_PIECE(fa, g, 1, b, fb);                                   \
+    take(3, bx, bw);                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                 \
+    PARK_NEXT;                                                         \
+    CCF_GATE_PIECE(fb, g, 2, a, fa);                                   \
+    take(0, ax, aw);                                                   \
+    CCF_GATE_PIECE(fa, g, 3, b, fb);                                   \
+    take(1, bx, bw);                                                   \
+    CCF_GATE_PIECE(fb, (g) + 1, 0, a, fa);                             \
+  } while (0)
+      auto all_rounds = [&](auto rag) {
+      asm volatile("" ::: "memory");               // the tile is free: the previous expert tile's logits have been read
+      fetch(0, xa, wa);
+      fetch(1, xb, wb);
+      fetch(2, xc, wc);
+      fetch(3, xd, wd);
+      __builtin_amdgcn_sched_barrier(0);
+      park(xa, wa);                                // stage 0
+      fetch(4, xa, wa);
+      __builtin_amdgcn_sched_barrier(0);
+      take(0, ax, aw);
+      take(1, bx, bw);
+      convert(rag, 0, 0, ax, aw, fax, faw);
+      __builtin_amdgcn_sched_barrier(0);
+      for (int rd = 0; rd < rounds; ++rd) {
+        const int g = 4 * rd;
+#pragma unroll
+        for (int v = 0; v < M::kRegs; ++v) acc[v] = 0.0f;
+        CCF_GATE_STAGE(g, park(xb, wb); fetch(g + 5, xb, wb));
+        CCF_GATE_STAGE(g + 1, park(xc, wc); fetch(g + 6, xc, wc));
+        CCF_GATE_STAGE(g + 2, park(xd, wd); fetch(g + 7, xd, wd));
+        if (rd + 1 < rounds)
+          CCF_GATE_STAGE(g + 3, park(xa, wa); fetch(g + 8, xa, wa));
+        else
+          CCF_GATE_STAGE(g + 3, (void)0);            // its reads ahead find the last stage again; nothing uses them
+        // the round's part sums onto the running sums, ascending part order
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+          for (int sl = 0; sl < S; ++sl) {
+            const int p = rd * S + sl;
+            if (p < nparts) {
+#pragma unroll
+              for (int j = 0; j < RB; ++j) {
+                const float ps = acc[(tb * S + sl) * RB + j];
+                total[tb * RB + j] = p == 0 ? ps : total[tb * RB + j] + ps;
+              }
+            }
+          }
+      }
+      };
+      if (ragged) all_rounds(std::true_type{}); else all_rounds(std::false_type{});
+#undef CCF_GATE_PIECE
+#undef CCF_GATE_STAGE
+      // logits of the tile: bias, one rounding, into the wavefront's LDS as [token][expert]
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < TB * RB; ++j) {
+        float t = total[j];
+        if (has_w) {
+          if (bg) t = t + my_bias;
+          t = round_to<half_t>(t);
+        }
+        region[((j / RB) * N + M::row(j % RB, lane)) * kLd + r] = t;
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+      if (logits_out) {
+        for (int i = lane; i < TW * N; i += 64) {
+          const int tok = i / N, col = i % N;
+          if (e0 + col < E && t0 + tok < tokens)
+            logits_out[static_cast<size_t>(t0 + tok) * E + e0 + col] = static_cast<half_t>(region[tok * kLd + col]);
+        }
+      }
+      if (lane < TW && t0 + lane < tokens) {
+        const float *lg = region + lane * kLd;
+        const int ne = (E - e0) < N ? (E - e0) : N;
+#pragma unroll
+        for (int c0 = 0; c0 < N; c0 += 8) {
+          float v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[u] = lg[c0 + u];
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (c0 + u < ne) best.offer(v[u], e0 + c0 + u, k);
+        }
+      }
+    }
+    if (lane < TW && t0 + lane < tokens) best.template write<half_t>(t0 + lane, k, idx_out, score_out);
+  }
+  if (wg_cnt) {
+    // expert counts of the workgroup's kStreamWaves * TW tokens, as in gate_mfma_kernel
+    __syncthreads();
+    int *row = reinterpret_cast<int *>(s_mem);
+    for (int e = threadIdx.x; e < E; e += blockDim.x) row[e] = 0;
+    __syncthreads();
+    if (lane < TW && t0 + lane < tokens) {
 #pragma unroll
       for (int s = 0; s < KS; ++s)
         if (s < k) atomicAdd(&row[best.id[s]], 1);
@@ -431,21 +697,29 @@ int gate_forward(const void *x, const void *wg, const void *bg, int tokens, int 
   }
   const int slots = 1 << ls;
   const int tw = 64 >> ls;
+  // With a wavefront or more per SIMD even when each works alone (two with the 16-wide tile, whose
+  // MFMAs are shorter), the wavefronts stream through K on their own; with fewer, the wavefronts
+  // of a workgroup share the parts of K.
+  const int tiles = (tokens + tw - 1) / tw;
+  const bool stream_form = g_gate_stream > 0 || (g_gate_stream < 0 && (tiles >= 2048 || (tiles >= 1024 && n == 32)));
   int waves = (nparts + slots - 1) / slots;
   int cap = g_gate_waves < kMaxWaves ? g_gate_waves : kMaxWaves;
   cap = cap < 1 ? 1 : cap;
   waves = waves < cap ? waves : cap;
-  const size_t lds = sizeof(float) * (static_cast<size_t>(waves) * kRegionFloats + static_cast<size_t>(tw) * (n + 1));
+  if (stream_form) waves = kStreamWaves;
+  const int wg_tokens = stream_form ? kStreamWaves * tw : tw;
+  const size_t lds = sizeof(float) * (static_cast<size_t>(waves) * kRegionFloats +
+                                      (stream_form ? 0 : static_cast<size_t>(tw) * (n + 1)));
   CCF_REQUIRE(lds <= 160 * 1024, CCF_ERR_SHAPE, "gate: %zu bytes of LDS needed", lds);
-  dim3 grid((tokens + tw - 1) / tw), block(waves * 64);
+  dim3 grid((tokens + wg_tokens - 1) / wg_tokens), block(waves * 64);
   if (wg_cnt && static_cast<long long>(grid.x) * tot_expert <= max_cnt) {
-    if (tokens_per_wg) *tokens_per_wg = tw;
+    if (tokens_per_wg) *tokens_per_wg = wg_tokens;
   } else {
     wg_cnt = nullptr;
   }
 #define CCF_GATE_LAUNCH(NN, LSV, KSV)                                                              \
   do {                                                                                             \
-    auto kern = gate_mfma_kernel<NN, LSV, KSV>;                                                    \
+    auto kern = stream_form ? gate_stream_kernel<NN, LSV, KSV> : gate_mfma_kernel<NN, LSV, KSV>;   \
     if (lds > 65536) {                                                                             \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                     \
                                          hipFuncAttributeMaxDynamicSharedMemorySize,               \
@@ -459,7 +733,9 @@ int gate_forward(const void *x, const void *wg, const void *bg, int tokens, int 
   } while (0)
 #define CCF_GATE_K(NN, LSV)                                                  \
   do {                                                                       \
-    if (top_k <= 2) CCF_GATE_LAUNCH(NN, LSV, 2); else CCF_GATE_LAUNCH(NN, LSV, kMaxTopK); \
+    if (top_k == 1) CCF_GATE_LAUNCH(NN, LSV, 1);                             \
+    else if (top_k == 2) CCF_GATE_LAUNCH(NN, LSV, 2);                        \
+    else CCF_GATE_LAUNCH(NN, LSV, kMaxTopK);                                 \
   } while (0)
   if (n == 32) {
     if (ls == 0) CCF_GATE_K(32, 0); else CCF_GATE_K(32, 1);

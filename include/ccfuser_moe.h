@@ -92,6 +92,9 @@ const char *ccf_last_error(void);
  *   "wgrad_transpose" 0/1: the backward's weight-gradient GEMM runs on transposed copies of the two
  *                     activation matrices instead of reading them row-major
  *   "gate_waves"      1..8 (default 8): most wavefronts of a gate workgroup; each takes other parts of K
+ *   "gate_stream"     -1 (default), 0 or 1: form of the fp16 gate kernel.  1: every wavefront takes its tokens
+ *                     through all of K alone, in one stream of loads and MFMAs; 0: the wavefronts of a
+ *                     workgroup share the parts of K; -1: the first with 1024 wavefronts of tokens or more
  */
 int ccf_set_option(const char *name, int value);
 

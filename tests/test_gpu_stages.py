@@ -67,40 +67,45 @@ def _gate_case(T, d, E, k):
     return _GATE_CASES[key]
 
 
-@pytest.mark.parametrize("slots,waves", [(0, 8), (1, 2), (2, 1), (4, 8), (1, 8)])
+@pytest.mark.parametrize("slots,waves,stream", [(0, 8, -1), (0, 8, 0), (1, 2, 0), (2, 1, 0), (4, 8, 0), (1, 8, 0),
+                                                (0, 8, 1), (1, 8, 1), (2, 8, 1), (4, 8, 1)])
 @pytest.mark.parametrize("T,d,E,k", [(5000, 512, 8, 2), (9000, 256, 32, 1), (40001, 128, 16, 2),
                                      (33000, 768, 32, 1), (300, 4096, 12, 2), (2100, 2048, 70, 4),
                                      (77, 8192, 8, 2), (130, 520, 40, 3)])
-def test_gate_launch_shapes(slots, waves, T, d, E, k):
+def test_gate_launch_shapes(slots, waves, stream, T, d, E, k):
     """Every way the gate spreads a problem over the machine gives the oracle's bits: 1, 2
     or 4 parts of K per wavefront (fewer tokens per workgroup), 1 to 8 wavefronts per
-    workgroup (several rounds of parts when K is long), both tile widths (16 and 32
-    experts, 1 to 3 tiles), a ragged last token group, a short last part."""
+    workgroup (several rounds of parts when K is long) or every wavefront alone through all
+    of K, both tile widths (16 and 32 experts, 1 to 3 tiles), a ragged last token group, a
+    short last part."""
     from ccfuser_amd import ops
-    _say(f"gate slots={slots} waves={waves} T={T} d={d} E={E} k={k}")
+    _say(f"gate slots={slots} waves={waves} stream={stream} T={T} d={d} E={E} k={k}")
     x, wg, bg, idx_ref, score_ref, logits_ref = _gate_case(T, d, E, k)
     ops.set_option("gate_slots", slots)
     ops.set_option("gate_waves", waves)
+    ops.set_option("gate_stream", stream)
     try:
         idx, score, logits = ops.gate_topk_softmax(dev(x), dev(wg), dev(bg), k, return_logits=True)
         torch.cuda.synchronize()
     finally:
         ops.set_option("gate_slots", 0)
         ops.set_option("gate_waves", 8)
+        ops.set_option("gate_stream", -1)
     assert torch.equal(logits.cpu(), logits_ref), "logits differ bitwise"
     assert torch.equal(idx.cpu(), idx_ref), "expert choice differs"
     assert (score.cpu().float() - score_ref.float()).abs().max() <= 1e-3
 
 
+@pytest.mark.parametrize("stream", [0, 1])
 @pytest.mark.parametrize("E,k", [(32, 2), (8, 1), (70, 3)])
-def test_gate_logits_that_are_nothing_but_rounding_error(E, k):
+def test_gate_logits_that_are_nothing_but_rounding_error(E, k, stream):
     """Inputs whose exact logits are zero: inside every part of 128 the second half of the
     products repeats the first half, permuted and negated (weights are powers of two, so
     every product is exact).  What is left is the rounding error of the fp32 chain, which
     depends on the order of the additions and on every rounding being to nearest even;
     scaled into fp16's range it must equal the oracle's bit for bit."""
     from ccfuser_amd import ops
-    _say(f"gate rounding residue E={E} k={k}")
+    _say(f"gate rounding residue E={E} k={k} stream={stream}")
     g = torch.Generator().manual_seed(E)
     T, d = 300, 512
     x = torch.empty(T, d)
@@ -117,8 +122,12 @@ def test_gate_logits_that_are_nothing_but_rounding_error(E, k):
     assert torch.equal((x.double() @ w.double().t()), torch.zeros(T, E, dtype=torch.float64))
     idx_ref, score_ref, logits_ref = O.naive_gate(x, w, None, k)
     assert (logits_ref != 0).float().mean() > 0.5          # the residue is there
-    idx, score, logits = ops.gate_topk_softmax(dev(x), dev(w), None, k, return_logits=True)
-    torch.cuda.synchronize()
+    ops.set_option("gate_stream", stream)
+    try:
+        idx, score, logits = ops.gate_topk_softmax(dev(x), dev(w), None, k, return_logits=True)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_option("gate_stream", -1)
     assert torch.equal(logits.cpu(), logits_ref), "rounding residue differs"
     assert torch.equal(idx.cpu(), idx_ref)
 
@@ -136,7 +145,8 @@ def test_gate_random_shapes():
             E = rng.choice([1, 2, 3, 8, 15, 16, 17, 31, 32, 33, 64, rng.randint(65, 140)])
             k = rng.randint(1, min(E, 8))
             slots, waves = rng.choice([0, 1, 2, 4]), rng.randint(1, 8)
-            _say(f"gate random case {case}: T={T} d={d} E={E} k={k} slots={slots} waves={waves}")
+            stream = (case * 7 + 1) % 3 - 1
+            _say(f"gate random case {case}: T={T} d={d} E={E} k={k} slots={slots} waves={waves} stream={stream}")
             g = torch.Generator().manual_seed(case)
             x = (torch.randn(T, d, generator=g) * 2.0 ** rng.randint(-3, 3)).half()
             wg = (torch.randn(E, d, generator=g) * 0.05).half()
@@ -144,6 +154,7 @@ def test_gate_random_shapes():
             idx_ref, score_ref, logits_ref = O.naive_gate(x, wg, bg, k)
             ops.set_option("gate_slots", slots)
             ops.set_option("gate_waves", waves)
+            ops.set_option("gate_stream", stream)
             idx, score, logits = ops.gate_topk_softmax(dev(x), dev(wg), None if bg is None else dev(bg), k,
                                                        return_logits=True)
             torch.cuda.synchronize()
@@ -153,6 +164,7 @@ def test_gate_random_shapes():
     finally:
         ops.set_option("gate_slots", 0)
         ops.set_option("gate_waves", 8)
+        ops.set_option("gate_stream", -1)
 
 
 @pytest.mark.parametrize("tile", [32, 16])
