@@ -252,7 +252,8 @@ int padded_rows(int max_rows, int E) {
 int launch_kseg(const int32_t *offsets, int E, int max_rows, int seg_rows, int n_blk, int32_t *k_seg,
                 int32_t *row_off, int32_t *blk_row0, int32_t *blk_cnt, int32_t *row_lo, half_t *zero_row,
                 const PlanReq *rows_plan, const PlanReq *w_plan, hipStream_t stream) {
-  const int per_plan = (E + 15) / 16 > 8 ? 8 : (E + 15) / 16;     // a wavefront per expert, at most 8 workgroups
+  // a wavefront per expert at least, 4 to 8 workgroups: wavefronts beyond the experts share their entries
+  const int per_plan = (E + 15) / 16 > 8 ? 8 : ((E + 15) / 16 < 4 ? 4 : (E + 15) / 16);
   const int na = rows_plan ? per_plan : 0, nb = w_plan ? per_plan : 0;
   const PlanReq none{};
   hipLaunchKernelGGL(kseg_kernel, dim3(1 + na + nb), dim3(1024), 0, stream, offsets, E, max_rows, seg_rows,

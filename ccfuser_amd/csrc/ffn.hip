@@ -37,10 +37,9 @@ __global__ void __launch_bounds__(kPlanThreads)
 plan_kernel(PlanReq rq, const int32_t *__restrict__ offsets, int E) {
   build_plan(rq, offsets, E, blockIdx.x, gridDim.x);
 }
-inline int plan_workgroups(int E) {
-  const int w = (E + kPlanThreads / 64 - 1) / (kPlanThreads / 64);
-  return w > 8 ? 8 : (w < 1 ? 1 : w);
-}
+// Workgroups that build a plan: a wavefront per expert at least; wavefronts beyond that share the experts'
+// entries (the builder is on the critical path of its launch, and the chip is idle beside it).
+inline int plan_workgroups(int) { return 8; }
 
 // ---- grouped GEMM kernel -------------------------------------------------------
 struct GroupedArgs {
@@ -1280,6 +1279,7 @@ GemmSetup setup_gemm(int max_rows, int E, int N, int K, int epi, bool b_kn, void
   // also where the last round of 256-row tiles is not split
   g.cut = g.skinny && !wide && g.grid <= kTailMaxParts;
   g.skinny_list = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(g.plan) + plan_core_bytes(max_rows, E, N > K ? N : K));
+  static_assert(plan_bm_ok(Cfg5::BM) && plan_bm_ok(Cfg8::BM), "build_plan shifts by the tile height");
   g.req = PlanReq{v.bm, max_tiles, max_rows, n_tiles_n, g.split ? g.grid / 8 : 0, K / 64, opt.split_max_parts, g.plan,
                   (g.split || g.cut) ? g.tail : nullptr, g.skinny ? g.skinny_list : nullptr, g.grid,
                   gelu ? kEpiCostGelu : kEpiCostPlain, opt.skinny_pct, g.cut && opt.skinny_tail, !wide};
@@ -1317,7 +1317,7 @@ int grouped_gemm(const half_t *A, const int32_t *a_rows, const int32_t *offsets,
   const bool second = gs.second, split = gs.split;
   const int grid = gs.grid;
   const long long wgs = gs.wgs;
-  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
+  CCF_REQUIRE(wgs < (1ll << 24), CCF_ERR_SHAPE, "%s: grid too large", what);
   if (!plan_ready) {
     hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream, gs.req, offsets, E);
     if (int rc = check_launch("plan_kernel")) return rc;
@@ -1404,7 +1404,7 @@ int grouped_gemm_kseg(const half_t *A, int lda, const half_t *B, int ldb, const 
   const int max_tiles = max_tiles_for(max_rows, E, Cfg5::BM);
   const int n_tiles_n = (N + Cfg5::BN - 1) / Cfg5::BN;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
-  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
+  CCF_REQUIRE(wgs < (1ll << 24), CCF_ERR_SHAPE, "%s: grid too large", what);
   if (!plan_ready) {
     hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream,
                        wgrad_plan_request(E, M, N, workspace), row_off, E);
@@ -1462,7 +1462,7 @@ int grouped_gemm_krows(const half_t *A, int lda, const half_t *B, int ldb, const
   const int max_tiles = max_tiles_for(max_rows, E, Cfg5::BM);
   const int n_tiles_n = N / Cfg5::BN;
   const long long wgs = launched_wgs(max_tiles, n_tiles_n);
-  CCF_REQUIRE(wgs < (1ll << 31), CCF_ERR_SHAPE, "%s: grid too large", what);
+  CCF_REQUIRE(wgs < (1ll << 24), CCF_ERR_SHAPE, "%s: grid too large", what);
   if (!plan_ready) {
     hipLaunchKernelGGL(plan_kernel, dim3(plan_workgroups(E)), dim3(kPlanThreads), 0, stream,
                        wgrad_plan_request(E, M, N, workspace), row_off, E);
@@ -1720,7 +1720,7 @@ bool forward_plan_request(int which, int max_rows, int E, int d, int f, void *wo
   const int N = which == 1 ? f : d, K = which == 1 ? d : f;
   const GemmSetup gs = setup_gemm(max_rows, E, N, K, which == 1 ? kEpiGelu : (which == 3 ? kEpiCombine : kEpiPlain),
                                   false, workspace, which == 1 ? 0 : 1, opt);
-  if (gs.wgs >= (1ll << 31)) return false;
+  if (gs.wgs >= (1ll << 24)) return false;
   *out = gs.req;
   return true;
 }
@@ -1807,7 +1807,7 @@ extern "C" int ccf_ffn_plan_info(const void *workspace, int max_rows, int num_ex
   if (e == hipSuccess) e = hipStreamSynchronize(st);
   if (e != hipSuccess) return fail(CCF_ERR_HIP, "ffn_plan_info: %s", hipGetErrorString(e));
   info[6] = gs.grid;
-  info[7] = static_cast<int32_t>(gs.wgs < (1ll << 31) ? gs.wgs : -1);
+  info[7] = static_cast<int32_t>(gs.wgs < (1ll << 24) ? gs.wgs : -1);
   if (where == 1) info[5] = -info[5];                 // cut along K inside the persistent launch
   return CCF_OK;
 }

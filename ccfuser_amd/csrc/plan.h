@@ -22,6 +22,8 @@ __host__ __device__ inline long long launched_wgs(int max_tiles, int n_tiles_n) 
 }
 
 constexpr int kOrderGroupM = 8;
+// build_plan divides by the tile height with shifts
+__host__ __device__ constexpr bool plan_bm_ok(int bm) { return bm > 0 && (bm & (bm - 1)) == 0; }
 
 // Scratch of the split last round, in front of the plan in the caller's workspace:
 //   [0, 16)              header: tile slots T (a multiple of 8; slot t belongs to XCD t % 8), parts S
@@ -84,22 +86,39 @@ __host__ __device__ inline size_t skinny_ints(int max_rows, int E, int n_tiles_n
   return kSkinnyHead + 4 * static_cast<size_t>(most > 0 ? most : 0) * n_tiles_n;
 }
 
+// n / d for 0 <= n < 2^24 and d > 0 through the reciprocal of d as a float (made once per divisor): the
+// product is off by at most one either way, which the remainder shows.  An integer division proper is ~30
+// dependent instructions, and the plan is built on the critical path of its launch.
+struct FastDiv {
+  int d;
+  float r;
+  __device__ inline explicit FastDiv(int dd) : d(dd), r(1.0f / static_cast<float>(dd)) {}
+  __device__ inline int div(int n) const {
+    int q = static_cast<int>(static_cast<float>(n) * r);
+    int rem = n - q * d;
+    q += rem >= d ? 1 : 0;
+    q -= rem < 0 ? 1 : 0;
+    return q;
+  }
+};
+
 // Time, in K steps of a 256-row tile, that F tiles of k_tiles K steps and an epilogue worth
 // `epi` K steps take on spx workgroups: whole rounds, then the last, partly filled round, which
 // is cut along K when the request allows it (same rule as the split below).
 __device__ inline int rounds_cost(int F, int spx, int k_tiles, int epi, bool may_split, int max_parts) {
   if (spx <= 0) return INT_MAX / 2;
-  const int r = F % spx;
-  int cost = F / spx * (k_tiles + epi);
+  const int full = FastDiv(spx).div(F);            // every count here is far below 2^24
+  const int r = F - full * spx;
+  int cost = full * (k_tiles + epi);
   if (r > 0) {
     int S = 0;
     if (may_split && 2 * r <= spx) {
-      S = spx / r;
+      S = FastDiv(r).div(spx);
       S = S > max_parts ? max_parts : S;
       S = S > k_tiles / 4 ? k_tiles / 4 : S;
       S = (S >= 2 && 8 * r * S <= 256) ? S : 0;
     }
-    cost += S ? k_tiles / S + 28 : k_tiles + epi;    // 28: two more launches, pipeline fill, the reduction (measured)
+    cost += S ? FastDiv(S).div(k_tiles) + 28 : k_tiles + epi;    // 28: two more launches, pipeline fill, the reduction (measured)
   }
   return cost;
 }
@@ -173,6 +192,10 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   int32_t *__restrict__ plan = rq.plan;
   int32_t *__restrict__ tail = rq.tail;
   int32_t *__restrict__ skinny = rq.skinny;
+  // tile counts and remainders by BM as shifts: BM is a power of two (plan_bm_ok, checked where requests are made)
+  const int bm_shift = 31 - __clz(BM);
+  auto tiles_of = [&](int cnt) { return (cnt + BM - 1) >> bm_shift; };
+  auto rem_of = [&](int cnt) { return cnt & (BM - 1); };
   __shared__ int s_full[8];        // split last round: slots of XCD x from s_full[x] on go to the tail list
   __shared__ int s_used[8];        // tiles of XCD x
   __shared__ int s_parts;          // parts per tail tile, 0 = no split
@@ -198,7 +221,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       for (int e = lane; e < E; e += 64) {
         int cnt = s_off[e + 1] - s_off[e];
         cnt = cnt > 0 ? cnt : 0;
-        const int nt = (cnt + BM - 1) / BM, r = cnt % BM;
+        const int nt = tiles_of(cnt), r = rem_of(cnt);
         const int sk1 = skinny_m_tiles(r, kSkinnyRows), sk2 = skinny_m_tiles(r, 2 * kSkinnyRows);
         nl0 += nt;
         nl1 += nt - (sk1 ? 1 : 0);
@@ -228,9 +251,9 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       int q_c = 0;
       if (tail && (rq.sk_tail_ok || rq.sk_beside_ok) && nk1 > 0 && k_tiles > 0) {
         const long long steps = static_cast<long long>(nk1) * n_tiles_n * k_tiles;
-        // (a 32-bit division: more steps than fit one are more than a workgroup's range may hold anyway)
-        const int q = steps < (1ll << 30) ? (static_cast<int>(steps) + tail_wgs - 1) / tail_wgs : (1 << 20);
-        if (q < (1 << 20) && sk_tail_segments(q, k_tiles) <= kSkTailSegs) q_c = q;
+        // (more than 2^23 steps are more than the workgroups' ranges may hold anyway)
+        const int q = steps < (1ll << 23) ? FastDiv(tail_wgs).div(static_cast<int>(steps) + tail_wgs - 1) : (1 << 20);
+        if (q < (1 << 20) && FastDiv(k_tiles).div(q - 1 + k_tiles - 1) + 1 <= kSkTailSegs) q_c = q;   // sk_tail_segments(q, k_tiles)
       }
       if (rq.skinny_pct < 0) sk_limit = my_limit;     // uniform: every lane took the same limit
       if (nk1 > 0 && rq.skinny_pct < -kSkinnyMaxWgs) {
@@ -254,7 +277,7 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
         bool ok = cand <= kSkinnyMaxWgs + 2 && (cand == 0 || nk1 > 0);
         if (n > 0) {
           const int sk_tile = (k_tiles * rq.skinny_pct + 99) / 100 + 3;       // one skinny tile, in K steps
-          const int sk_c = (T_x + n - 1) / n * sk_tile;
+          const int sk_c = FastDiv(n).div(T_x + n - 1) * sk_tile;
           cost = cost > sk_c ? cost : sk_c;
           ok = ok && n * 4 <= cus_x && rq.sk_beside_ok;
         } else if (cand == kSkinnyMaxWgs + 1) {
@@ -287,10 +310,10 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       const int e = e0 + lane;
       int cnt = e < E ? s_off[e + 1] - s_off[e] : 0;
       cnt = cnt > 0 ? cnt : 0;
-      const int nt = (cnt + BM - 1) / BM;
+      const int nt = tiles_of(cnt);
       int ns, nl;
       if (ns_wgs || tail_q) {
-        const int r = cnt % BM;                                   // ns counts skinny M tiles here
+        const int r = rem_of(cnt);                                // ns counts skinny M tiles here
         ns = skinny_m_tiles(r, sk_limit);
         nl = nt - (ns ? 1 : 0);
       } else {
@@ -309,8 +332,49 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       carry_s += __shfl(inc_s, 63, 64);
     }
     if (lane == 0) { s_long[E] = carry_l; s_short[E] = carry_s; }
+    // The split last round (run by grouped_gemm_tail_kernel and splitk_reduce_kernel in ffn.hip).
+    // XCD x holds used_x tiles; with spx persistent workgroups per XCD the last used_x % spx of
+    // them form a partly filled round.
+    // When that round is at most half full on every XCD, its tiles leave the plan: tile i of
+    // XCD x's last round, part s of S, becomes tail entry x + 8 * (i * S + s), the workgroup id
+    // that the hardware places on the same XCD, so the patch of neighbouring tiles keeps sharing
+    // its operands through that XCD's L2 (parts of the same K range walk K in step).
+    // Lane x < 8 takes XCD x.
+    {
+      const bool use_sk = ns_wgs > 0 || tail_q > 0;
+      const int spx_w = spx > 0 ? spx - ns_wgs : spx;
+      const int total_l = carry_l * n_tiles_n, total_s = use_sk ? 0 : carry_s * n_tiles_n;
+      const int per_l = (total_l + 7) / 8, per_s = (total_s + 7) / 8;
+      const int x = lane & 7;
+      int nl_x = total_l - x * per_l, ns_x = total_s - x * per_s;
+      nl_x = nl_x < 0 ? 0 : (nl_x > per_l ? per_l : nl_x);
+      ns_x = ns_x < 0 ? 0 : (ns_x > per_s ? per_s : ns_x);
+      const int used = nl_x + ns_x;
+      const int full = spx_w > 0 ? used / spx_w * spx_w : used;
+      int max_r = used - full;
+#pragma unroll
+      for (int off = 4; off >= 1; off >>= 1) {
+        const int other = __shfl_xor(max_r, off, 64);
+        max_r = other > max_r ? other : max_r;
+      }
+      int S = 0;
+      if (tail && spx_w > 0 && max_r > 0 && max_r * 2 <= spx_w) {
+        S = spx_w / max_r;
+        S = S > rq.max_parts ? rq.max_parts : S;
+        S = S > k_tiles / 4 ? k_tiles / 4 : S;           // at least four K tiles per part
+        S = (S >= 2 && 8 * max_r * S <= kTailMaxParts) ? S : 0;
+      }
+      if (lane < 8) {
+        s_used[lane] = used;
+        s_full[lane] = S ? full : INT_MAX;
+      }
+      if (lane == 0) {
+        s_parts = S;
+        if (tail && part == 0) { tail[0] = S ? 8 * max_r : 0; tail[1] = S; }
+      }
+    }
   }
-  // the launcher checks that the worst-case tile count, and with it every count below, fits an int
+  // the launcher checks that the worst-case tile count, and with it every count below, is below 2^24
   const int wgs = static_cast<int>(launched_wgs(max_tiles, n_tiles_n));
   int4v *entry = reinterpret_cast<int4v *>(plan);
   int4v *tent = tail ? reinterpret_cast<int4v *>(tail + 64) : nullptr;
@@ -341,38 +405,6 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
   }
   const int per_long = (total_long + 7) / 8;
   const int per_short = (total_short + 7) / 8;
-  // The split last round (run by grouped_gemm_tail_kernel and splitk_reduce_kernel in ffn.hip).
-  // XCD x holds used_x tiles; with spx persistent workgroups per XCD the last used_x % spx of
-  // them form a partly filled round.
-  // When that round is at most half full on every XCD, its tiles leave the plan: tile i of
-  // XCD x's last round, part s of S, becomes tail entry x + 8 * (i * S + s), the workgroup id
-  // that the hardware places on the same XCD, so the patch of neighbouring tiles keeps sharing
-  // its operands through that XCD's L2 (parts of the same K range walk K in step).
-  if (threadIdx.x == 0) {
-    int max_r = 0;
-    for (int x = 0; x < 8; ++x) {
-      int nl_x = total_long - x * per_long, ns_x = total_short - x * per_short;
-      nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
-      ns_x = ns_x < 0 ? 0 : (ns_x > per_short ? per_short : ns_x);
-      const int used = nl_x + ns_x;
-      const int full = spx > 0 ? used / spx * spx : used;
-      s_used[x] = used;
-      s_full[x] = full;
-      max_r = (used - full) > max_r ? (used - full) : max_r;
-    }
-    int S = 0;
-    if (tail && spx > 0 && max_r > 0 && max_r * 2 <= spx) {
-      S = spx / max_r;
-      S = S > rq.max_parts ? rq.max_parts : S;
-      S = S > k_tiles / 4 ? k_tiles / 4 : S;           // at least four K tiles per part
-      S = (S >= 2 && 8 * max_r * S <= kTailMaxParts) ? S : 0;
-    }
-    s_parts = S;
-    if (!S)
-      for (int x = 0; x < 8; ++x) s_full[x] = INT_MAX;
-    if (tail && part == 0) { tail[0] = S ? 8 * max_r : 0; tail[1] = S; }
-  }
-  __syncthreads();
   const int S = s_parts;
   // idle entries: slot j of XCD x holds a tile while j < used_x (and j < full_x when the last
   // round is split off); tail entry x + 8 * (i * S + s) while i < used_x - full_x
@@ -396,10 +428,17 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       entry[b] = v;
     }
   };
-  // one wavefront per expert
+  // A wavefront per expert; with more wavefronts than experts (few experts), `sub_n` wavefronts share an
+  // expert's entries.
   const int lane = threadIdx.x & 63, nwave = (blockDim.x >> 6) * nparts;
   const int wave = (threadIdx.x >> 6) * nparts + part;          // interleaved over the workgroups
-  for (int e = wave; e < E; e += nwave) {
+  const int sub_n = nwave >= 2 * E ? nwave / E : 1;
+  const int takers = sub_n > 1 ? sub_n * E : nwave;             // wavefronts that take entries
+  const int sub = sub_n > 1 ? wave / E : 0;
+  const int l0 = lane + 64 * sub, l_step = 64 * sub_n;
+  // per-entry divisions by divisors that are the same for the whole workgroup
+  const FastDiv by_run(kOrderGroupM * n_tiles_n), by_long(per_long > 0 ? per_long : 1), by_short(per_short > 0 ? per_short : 1);
+  for (int e = sub_n > 1 ? wave % E : wave; wave < takers && e < E; e += nwave) {
     const int lo = s_off[e];
     int cnt = s_off[e + 1] - lo;
     cnt = cnt > 0 ? cnt : 0;
@@ -412,18 +451,19 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
     // for a M tiles, a token tile once for 32/a N tiles, and HBM traffic per
     // patch, which goes as 1/a + a/32, is near its minimum for a = 4..8.
     const int first = s_long[e] * n_tiles_n;
-    const int cnt_long = (use_skinny && ns) ? cnt - cnt % BM : cnt;   // rows the 256-row tiles hold
-    for (int l = lane; l < nl * n_tiles_n; l += 64) {
-      const int run = l / (kOrderGroupM * n_tiles_n);            // which run of M tiles
+    const int cnt_long = (use_skinny && ns) ? cnt - rem_of(cnt) : cnt;   // rows the 256-row tiles hold
+    for (int l = l0; l < nl * n_tiles_n; l += l_step) {
+      const int run = by_run.div(l);                             // which run of M tiles
       const int run_first = run * kOrderGroupM;
       const int run_size = (nl - run_first) < kOrderGroupM ? (nl - run_first) : kOrderGroupM;
       const int in_run = l - run * kOrderGroupM * n_tiles_n;
-      const int i = run_first + in_run % run_size;               // M tile within the expert
-      const int tn = in_run / run_size;
+      const int tn = FastDiv(run_size).div(in_run);
+      const int i = run_first + (in_run - tn * run_size);        // M tile within the expert
       const int logical = first + l;
       int first_row, rows;
       tile_rows(cnt_long, nl, i, BM, first_row, rows);
-      place(logical % per_long, logical / per_long, int4v{e, lo + first_row, rows, tn});   // hardware id = slot * 8 + XCD
+      const int x = by_long.div(logical);
+      place(logical - x * per_long, x, int4v{e, lo + first_row, rows, tn});   // hardware id = slot * 8 + XCD
     }
     if (ns && use_skinny) {
       int4v *sk = reinterpret_cast<int4v *>(skinny + kSkinnyHead);
@@ -431,17 +471,17 @@ __device__ inline void build_plan(const PlanReq &rq, const int32_t *__restrict__
       for (int m = 0; m < ns; ++m) {                             // one or two skinny M tiles
         const int r0 = cnt_long + m * kSkinnyRows;
         const int rows = (cnt - r0) < kSkinnyRows ? (cnt - r0) : kSkinnyRows;
-        for (int tn = lane; tn < n_tiles_n; tn += 64) sk[first_s + m * n_tiles_n + tn] = int4v{e, lo + r0, rows, tn};
+        for (int tn = l0; tn < n_tiles_n; tn += l_step) sk[first_s + m * n_tiles_n + tn] = int4v{e, lo + r0, rows, tn};
       }
     } else if (ns) {
       const int i = nl;                                          // the expert's last M tile
       const int first_s = s_short[e] * n_tiles_n;
-      for (int tn = lane; tn < n_tiles_n; tn += 64) {
+      for (int tn = l0; tn < n_tiles_n; tn += l_step) {
         const int logical = first_s + tn;
-        const int x = logical / per_short;
+        const int x = by_short.div(logical);
         int nl_x = total_long - x * per_long;              // long tiles on this XCD
         nl_x = nl_x < 0 ? 0 : (nl_x > per_long ? per_long : nl_x);
-        place(nl_x + logical % per_short, x, int4v{e, lo + i * BM, cnt - i * BM, tn});
+        place(nl_x + (logical - x * per_short), x, int4v{e, lo + i * BM, cnt - i * BM, tn});
       }
     }
   }

@@ -389,9 +389,9 @@ int route_impl(const int64_t *gate_idx, int n_flat, int E, int top_k, int capaci
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(pos_lds));
     if (e != hipSuccess) return fail(CCF_ERR_HIP, "route: LDS attribute: %s", hipGetErrorString(e));
   }
-  // a plan is built by enough workgroups of kThreads that every expert has a wavefront (at most 8)
-  int plan_wgs = (E + kThreads / 64 - 1) / (kThreads / 64);
-  plan_wgs = plan_wgs > 8 ? 8 : plan_wgs;
+  // a plan is built by 8 workgroups of kThreads: a wavefront per expert at least, and the wavefronts beyond
+  // that share the experts' entries
+  const int plan_wgs = 8;
   hipLaunchKernelGGL(pos_kernel, dim3(nchunk + n_plans * plan_wgs), dim3(kThreads), pos_lds, stream,
                      gate_idx, n_flat, E, nbits, top_k, capacity, chunk_cnt, offsets, pos, src_row,
                      dst_row, inv_pos, idx_kept, nchunk, plan_wgs, n_plans > 0 ? plans[0] : none,
