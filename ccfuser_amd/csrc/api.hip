@@ -245,16 +245,21 @@ extern "C" int ccf_moe_ffn_segments(const void *x, const int32_t *seg_start, con
   int rc;
   mark_stage(0, st);
   mark_stage(1, st);                                  // no gate in this call
-  if ((rc = ccf_segments_to_rows(seg_start, seg_len, seg_expert, n_seg, num_expert, total_rows,
-                                 w.counts, w.offsets, w.rows, stream)))
+  // the tile plans of both GEMMs are built by more workgroups of the regrouping launch, as in ccf_moe_forward
+  PlanReq plans[2];
+  const GemmOptions opt = forward_options();
+  const bool planned = forward_plan_request(1, total_rows, num_expert, d_model, d_ffn, w.ffn_ws, opt, &plans[0]) &&
+                       forward_plan_request(2, total_rows, num_expert, d_model, d_ffn, w.ffn_ws, opt, &plans[1]);
+  if ((rc = segments_with_plans(seg_start, seg_len, seg_expert, n_seg, num_expert, total_rows, w.counts, w.offsets,
+                                w.rows, st, plans, planned ? 2 : 0)))
     return rc;
   mark_stage(2, st);
-  if ((rc = ccf_ffn1_forward(x, w.rows, nullptr, w.offsets, total_rows, num_expert, d_model, d_ffn, w1, b1, 1,
-                             w.h, w.ffn_ws, w.ffn_bytes, stream)))
+  if ((rc = ffn1_forward(x, w.rows, nullptr, w.offsets, total_rows, num_expert, d_model, d_ffn, w1, b1, 1,
+                         w.h, w.ffn_ws, w.ffn_bytes, st, planned ? &opt : nullptr)))
     return rc;
   mark_stage(3, st);
-  rc = ccf_ffn2_forward(w.h, nullptr, w.rows, w.offsets, total_rows, num_expert, d_model, d_ffn, w2, b2,
-                        nullptr, y, w.ffn_ws, w.ffn_bytes, stream);
+  rc = ffn2_forward(w.h, nullptr, w.rows, w.offsets, total_rows, num_expert, d_model, d_ffn, w2, b2,
+                    nullptr, y, w.ffn_ws, w.ffn_bytes, st, planned ? &opt : nullptr);
   mark_stage(4, st);
   mark_stage(5, st);                                  // no combine either
   return rc;

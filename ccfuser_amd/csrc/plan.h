@@ -521,6 +521,10 @@ int route_with_plans(const int64_t *gate_idx, int n_flat, int num_expert, int to
                      int32_t *counts, int32_t *offsets, int64_t *pos, int32_t *src_row, int32_t *dst_row,
                      int32_t *inv_pos, int64_t *idx_kept, void *workspace, size_t workspace_bytes,
                      hipStream_t stream, const PlanReq *plans, int n_plans, int gate_row_len);
+// route.hip: ccf_segments_to_rows(), whose launch also builds n_plans (0..2) tile plans
+int segments_with_plans(const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_expert, int n_seg,
+                        int num_expert, int total_rows, int32_t *counts, int32_t *offsets, int32_t *rows,
+                        hipStream_t stream, const PlanReq *plans, int n_plans);
 // most entries of a table of per-run expert counts that the routing stage takes from the gate kernel
 long long route_rows_max_ints();
 

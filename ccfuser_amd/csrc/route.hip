@@ -291,28 +291,44 @@ __global__ void __launch_bounds__(1024)
 segments_kernel(const int32_t *__restrict__ seg_start, const int32_t *__restrict__ seg_len,
                 const int32_t *__restrict__ seg_expert, int n_seg, int E, int total_rows,
                 int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
-                int32_t *__restrict__ rows) {
+                int32_t *__restrict__ rows, int plan_wgs, PlanReq plan0, PlanReq plan1) {
   __shared__ int s_cnt[kMaxExpert];
   __shared__ int s_off[kMaxExpert + 1];
-  for (int e = threadIdx.x; e < E; e += blockDim.x) {
-    int run = 0;
-    for (int s = 0; s < n_seg; ++s)
-      if (seg_expert[s] == e && seg_len[s] > 0) run += seg_len[s];
-    s_cnt[e] = run;
-    counts[e] = run;
+  // every workgroup: rows per expert (a thread per triple, integer adds in LDS), then the experts' starts
+  for (int e = threadIdx.x; e < E; e += blockDim.x) s_cnt[e] = 0;
+  __syncthreads();
+  for (int s = threadIdx.x; s < n_seg; s += blockDim.x) {
+    const int e = seg_expert[s], len = seg_len[s];
+    if (e >= 0 && e < E && len > 0) atomicAdd(&s_cnt[e], len);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int e = 0; e < E; ++e) {
-      s_off[e] = run;
-      offsets[e] = run;
-      run += s_cnt[e];
+  if (threadIdx.x < 64) {
+    int carry = 0;
+    const int lane = threadIdx.x;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      const int v = (e0 + lane < E) ? s_cnt[e0 + lane] : 0;
+      int inc = v;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        int o = __shfl_up(inc, off, 64);
+        if (lane >= off) inc += o;
+      }
+      if (e0 + lane < E) s_off[e0 + lane] = carry + inc - v;
+      carry += __shfl(inc, 63, 64);
     }
-    s_off[E] = run;
-    offsets[E] = run;
+    if (lane == 0) s_off[E] = carry;
   }
   __syncthreads();
+  // workgroups past the first build the tile plans of the GEMMs that follow (the offsets are final)
+  if (blockIdx.x > 0) {
+    const int r = static_cast<int>(blockIdx.x) - 1;
+    build_plan(r < plan_wgs ? plan0 : plan1, s_off, E, r % plan_wgs, plan_wgs);
+    return;
+  }
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) {
+    offsets[e] = s_off[e];
+    if (e < E) counts[e] = s_cnt[e];
+  }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = blockDim.x >> 6;
   for (int s = wave; s < n_seg; s += nwave) {
     const int e = seg_expert[s];
@@ -593,20 +609,33 @@ extern "C" int ccf_route_static(const int64_t *gate_idx, int n_flat, int num_exp
                     dst_row, inv_pos, idx_kept, ws, sizeof(int32_t) * kStaticScratchInts, as_stream(stream));
 }
 
-extern "C" int ccf_segments_to_rows(const int32_t *seg_start, const int32_t *seg_len,
-                                    const int32_t *seg_expert, int n_seg, int num_expert,
-                                    int total_rows, int32_t *counts, int32_t *offsets,
-                                    int32_t *rows, ccf_stream_t stream) {
-  using namespace ccf;
+namespace ccf {
+// ccf_segments_to_rows(), whose launch also builds n_plans (0..2) tile plans from the offsets.
+int segments_with_plans(const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_expert, int n_seg,
+                        int num_expert, int total_rows, int32_t *counts, int32_t *offsets, int32_t *rows,
+                        hipStream_t stream, const PlanReq *plans, int n_plans) {
   CCF_REQUIRE(seg_start && seg_len && seg_expert && counts && offsets && rows, CCF_ERR_ARG,
               "segments_to_rows: null pointer");
   CCF_REQUIRE(n_seg >= 0 && num_expert > 0 && total_rows >= 0, CCF_ERR_ARG,
               "segments_to_rows: bad size");
   CCF_REQUIRE(num_expert <= kMaxExpert, CCF_ERR_SHAPE, "segments_to_rows: num_expert=%d exceeds %d",
               num_expert, kMaxExpert);
-  hipLaunchKernelGGL(segments_kernel, dim3(1), dim3(1024), 0, as_stream(stream), seg_start, seg_len,
-                     seg_expert, n_seg, num_expert, total_rows, counts, offsets, rows);
+  CCF_REQUIRE(n_plans >= 0 && n_plans <= 2 && (n_plans == 0 || plans), CCF_ERR_ARG, "segments_to_rows: bad plan requests");
+  const PlanReq none{0, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
+  const int plan_wgs = 4;                            // of 1024 threads: 64 wavefronts per plan
+  hipLaunchKernelGGL(segments_kernel, dim3(1 + n_plans * plan_wgs), dim3(1024), 0, stream, seg_start, seg_len,
+                     seg_expert, n_seg, num_expert, total_rows, counts, offsets, rows, plan_wgs,
+                     n_plans > 0 ? plans[0] : none, n_plans > 1 ? plans[1] : none);
   return check_launch("segments_kernel");
+}
+}  // namespace ccf
+
+extern "C" int ccf_segments_to_rows(const int32_t *seg_start, const int32_t *seg_len,
+                                    const int32_t *seg_expert, int n_seg, int num_expert,
+                                    int total_rows, int32_t *counts, int32_t *offsets,
+                                    int32_t *rows, ccf_stream_t stream) {
+  return ccf::segments_with_plans(seg_start, seg_len, seg_expert, n_seg, num_expert, total_rows, counts, offsets,
+                                  rows, ccf::as_stream(stream), nullptr, 0);
 }
 
 extern "C" int ccf_plan_blocks(const int32_t *counts, int num_expert, int block_size, int rank,

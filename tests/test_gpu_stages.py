@@ -310,6 +310,41 @@ def test_plan_blocks_matches_divide_into_block(case):
     assert got32["ranks"][:t32].tolist() == [3] * t32
 
 
+@pytest.mark.parametrize("n_seg,E,seed", [(64, 8, 0), (1, 1, 1), (700, 37, 2), (3000, 200, 3), (5, 1024, 4)])
+def test_segments_to_rows(n_seg, E, seed):
+    """(start, len, expert) triples -> counts, offsets and the row list grouped by expert, rows of
+    an expert in the order of the triple list and then row order (what the reference's kernels do
+    per block through start_addrs / lens / expert_ids, mix_gemm.cu:296-301).  Triples with no
+    rows or with an expert outside 0..E-1 are skipped.  Many triples, empty experts, bit for bit."""
+    from ccfuser_amd import ops
+    import numpy as np
+    _say(f"segments_to_rows n_seg={n_seg} E={E} seed={seed}")
+    rng = np.random.default_rng(seed)
+    seg_len = rng.integers(0, 40, n_seg).astype(np.int32)
+    seg_len[rng.random(n_seg) < 0.1] = 0
+    seg_expert = rng.integers(0, E, n_seg).astype(np.int32)
+    bad = rng.random(n_seg) < 0.05
+    seg_expert[bad] = rng.choice([-1, E, E + 5], bad.sum())
+    total = int(seg_len.sum())
+    seg_start = (np.cumsum(seg_len) - seg_len).astype(np.int32)
+    order = rng.permutation(n_seg)                       # the list is in no particular order
+    seg_start, seg_len, seg_expert = seg_start[order], seg_len[order], seg_expert[order]
+    counts_ref = np.zeros(E, dtype=np.int32)
+    per = [[] for _ in range(E)]
+    for st, ln, e in zip(seg_start, seg_len, seg_expert):
+        if 0 <= e < E and ln > 0:
+            counts_ref[e] += ln
+            per[e].extend(range(st, st + ln))
+    offsets_ref = np.concatenate([[0], np.cumsum(counts_ref)]).astype(np.int32)
+    rows_ref = np.array([r for e in range(E) for r in per[e]], dtype=np.int32)
+    counts, offsets, rows = ops.segments_to_rows(dev(torch.from_numpy(seg_start)), dev(torch.from_numpy(seg_len)),
+                                                 dev(torch.from_numpy(seg_expert)), E, max(total, 1))
+    torch.cuda.synchronize()
+    assert np.array_equal(counts.cpu().numpy(), counts_ref)
+    assert np.array_equal(offsets.cpu().numpy(), offsets_ref)
+    assert np.array_equal(rows.cpu().numpy()[:len(rows_ref)], rows_ref)
+
+
 # ------------------------------------------------- row moves and combine
 def test_local_scatter_gather_with_reference_pos_vector():
     """The reference's own scatter check: index_select(input, 0, pos) with its
