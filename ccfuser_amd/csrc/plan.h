@@ -86,9 +86,11 @@ __host__ __device__ inline size_t skinny_ints(int max_rows, int E, int n_tiles_n
   return kSkinnyHead + 4 * static_cast<size_t>(most > 0 ? most : 0) * n_tiles_n;
 }
 
-// n / d for 0 <= n < 2^24 and d > 0 through the reciprocal of d as a float (made once per divisor): the
-// product is off by at most one either way, which the remainder shows.  An integer division proper is ~30
-// dependent instructions, and the plan is built on the critical path of its launch.
+// n / d for 0 <= n < 2^24, d > 0 and a quotient below 2^22 (every count a plan divides is far below: at
+// most the tiles of an XCD) through the reciprocal of d as a float, made once per divisor: n and d are exact
+// as floats, the reciprocal and the product are each within an ulp, so the truncated product is off by at
+// most one either way, which the remainder shows.  An integer division proper is ~30 dependent
+// instructions, and the plan is built on the critical path of its launch.
 struct FastDiv {
   int d;
   float r;
