@@ -338,6 +338,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c3_mixtral")
+    ap.add_argument("--no-steady-state", action="store_true",
+                    help="with fewer than 45 steps in all: do not run on to time the step after the clock ramp")
     ap.add_argument("--stage-events", choices=("timed", "after"), default="timed",
                     help="record the per-stage HIP events inside the timed steps, or in a second pass of the same steps")
     ap.add_argument("--gemm-variant", type=int, default=None)
@@ -440,16 +442,19 @@ def main():
         wall_events = wall
     _lib.call("ccf_moe_forward_set_events", None, 0)
     # Beside the contract's figure: the same step once the clocks have settled.  The chip ramps its clocks over
-    # the first ~25 steps of a load, so a run with few warm-up steps times the ramp; this runs on until 45
-    # steps have passed since the start and then times 30 more.  Reported as "steady_state", never as "value".
-    for _ in range(max(0, 45 - W - K)):
-        run()
-    torch.cuda.synchronize()
-    t2 = time.perf_counter()
-    for _ in range(30):
-        run()
-    torch.cuda.synchronize()
-    steady_ms = (time.perf_counter() - t2) / 30 * 1e3
+    # the first ~25 steps of a load, so a run with few warm-up steps times the ramp; such a run (fewer than 45
+    # steps in all) goes on until 45 steps have passed since the start and then times 30 more.  Reported as
+    # "steady_state", never as "value".
+    steady_ms = None
+    if W + K < 45 and not a.no_steady_state:
+        for _ in range(45 - W - K):
+            run()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for _ in range(30):
+            run()
+        torch.cuda.synchronize()
+        steady_ms = (time.perf_counter() - t2) / 30 * 1e3
     routed = T if segments else int(offsets[-1].item())
     stage_names = ("gate", "route", "ffn1", "ffn2", "combine")
     stage_ms = {n: sum(ev.elapsed_ms(events[i][s], events[i][s + 1]) for i in range(K)) / K
@@ -479,11 +484,12 @@ def main():
     }
     line["stages_ms"] = stage_ms
     line["ms_per_step_with_stage_events"] = wall_events / K * 1e3
-    line["steady_state"] = {"ms_per_step": steady_ms, "tokens_per_s": T / (steady_ms * 1e-3),
-                            "frac_fp16_mfma_peak": flops / (steady_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
-                            "steps": 30, "after_steps": max(45, W + K),
-                            "what": "the same call, timed after the clock ramp of the first ~25 steps; "
-                                    "no stage events; not the contract's figure"}
+    if steady_ms is not None:
+        line["steady_state"] = {"ms_per_step": steady_ms, "tokens_per_s": T / (steady_ms * 1e-3),
+                                "frac_fp16_mfma_peak": flops / (steady_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
+                                "steps": 30, "after_steps": 45,
+                                "what": "the same call, timed after the clock ramp of the first ~25 steps; "
+                                        "no stage events; not the contract's figure"}
     dom = "ffn1" if stage_ms["ffn1"] >= stage_ms["ffn2"] else "ffn2"
     ach = (flops / 2) / (stage_ms[dom] * 1e-3) / 1e12
     traffic, stale, traffic_file = measured_traffic(wl.name, dom)
