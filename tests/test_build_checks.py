@@ -64,3 +64,24 @@ _ZN3ccf5otherE:
     assert len(bad) == 1 and "a17" in bad[0][1][0]
     clean = asm.replace("\tv_accvgpr_write_b32 a17, v3\n", "\tv_accvgpr_write_b32 a[17], 0\n")
     assert B.acc_register_violations(clean, B.ACC_CHECKED["ffn.hip"]) == []
+
+
+@needs_hipcc
+def test_gate_kernels_keep_their_values_in_registers(tmp_path):
+    """Both forms of the fp16 gate (wavefronts sharing K, and every wavefront alone through all of K
+    with four sets of loads in flight) are built for a register budget: none of their instantiations
+    may spill (the kernel metadata's private segment size is what a spill would need)."""
+    import re
+    from ccfuser_amd import build as B
+    text = B.device_assembly("gate.hip", tmp_path / "gate.s")
+    sizes = {}
+    for m in re.finditer(r"\.name:\s+(\S*gate_(?:mfma|stream)_kernel\S*)(.*?)\.private_segment_fixed_size:\s+(\d+)", text, flags=re.S):
+        if ".name:" in m.group(2):                      # ran into the next kernel's record
+            continue
+        sizes[m.group(1)] = int(m.group(3))
+    forms = {"mfma": 0, "stream": 0}
+    for name, size in sizes.items():
+        assert size == 0, f"{name} spills {size} bytes"
+        forms["stream" if "stream" in name else "mfma"] += 1
+    # tile widths 16 and 32, 1/2/4 slots, three list lengths of the selection
+    assert forms["mfma"] >= 15 and forms["stream"] >= 15, forms
